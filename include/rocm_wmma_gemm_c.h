@@ -1,0 +1,94 @@
+/*
+ * C ABI of librocm_wmma_gemm_gfx950.so -- the drop-in boundary of the GEMM path.
+ *
+ * The first four functions are exactly the symbols the reference's runtime
+ * loader resolves with dlsym (reference rocm_wmma_gemm/include/rocm_wmma_gemm/
+ * kernel_loader.hpp:53-54,110-113) and that its arch library defines
+ * (reference rocm_wmma_gemm/src/gemm.cpp:219-250).  The rest are additions with
+ * no counterpart in the reference: introspection and tuning hooks.
+ *
+ * Conventions for every gemm entry point:
+ *   C (M x N) = A (M x K) * B (K x N); C is overwritten; operands are dense and
+ *   packed in the stated layout; layout_* is 0 for row-major, 1 for column-major;
+ *   batch b uses A + b*M*K, B + b*K*N, C + b*M*N (elements);
+ *   `stream` is the ADDRESS of the caller's hipStream_t (a hipStream_t*), not the
+ *   handle itself; the work is enqueued there and the call returns at once;
+ *   all pointers are device pointers owned by the caller;
+ *   a layout value outside {0,1} makes the call a no-op (reference behaviour,
+ *   src/gemm.cpp:243); M, N or batch_count of 0 is a no-op; K of 0 zero-fills C.
+ */
+#ifndef ROCM_WMMA_GEMM_C_H
+#define ROCM_WMMA_GEMM_C_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* fp16 A,B -> fp16 C.  Replaces reference src/gemm.cpp:247 (DEFINE_C_DISPATCH(f16_f16, half, half)). */
+void rocm_wmma_gemm_f16_f16(void* C, void* A, void* B, size_t M, size_t N, size_t K,
+                            size_t batch_count, int layout_c, int layout_a, int layout_b,
+                            void* stream);
+
+/* fp16 A,B -> fp32 C.  Replaces reference src/gemm.cpp:248. */
+void rocm_wmma_gemm_f32_f16(void* C, void* A, void* B, size_t M, size_t N, size_t K,
+                            size_t batch_count, int layout_c, int layout_a, int layout_b,
+                            void* stream);
+
+/* bf16 A,B -> bf16 C.  Replaces reference src/gemm.cpp:249. */
+void rocm_wmma_gemm_bf16_bf16(void* C, void* A, void* B, size_t M, size_t N, size_t K,
+                              size_t batch_count, int layout_c, int layout_a, int layout_b,
+                              void* stream);
+
+/* bf16 A,B -> fp32 C.  Replaces reference src/gemm.cpp:250. */
+void rocm_wmma_gemm_f32_bf16(void* C, void* A, void* B, size_t M, size_t N, size_t K,
+                             size_t batch_count, int layout_c, int layout_a, int layout_b,
+                             void* stream);
+
+/* ---- additions (no counterpart in the reference) ------------------------ */
+
+/* type_idx values, in the reference launcher's order (kernel_launcher.hpp:78-83). */
+#define ROCM_WMMA_GEMM_TYPE_F16_F16 0
+#define ROCM_WMMA_GEMM_TYPE_F32_F16 1
+#define ROCM_WMMA_GEMM_TYPE_BF16_BF16 2
+#define ROCM_WMMA_GEMM_TYPE_F32_BF16 3
+
+/* Description of one compiled kernel variant. */
+typedef struct rocm_wmma_gemm_variant_info
+{
+    int block_m, block_n, block_k; /* workgroup tile */
+    int warps_m, warps_n;          /* wave grid inside the workgroup */
+    int warp_tile_m, warp_tile_n;  /* 32x32 MFMA tiles per wave */
+    int pipeline;                  /* 0 = register-staged general path, 1 = direct-to-LDS */
+    int lds_bytes;                 /* static LDS per workgroup */
+    int threads;                   /* workgroup size */
+} rocm_wmma_gemm_variant_info;
+
+/* "gfx950": the architecture this library was compiled for. */
+const char* rocm_wmma_gemm_arch(void);
+
+/* Number of compiled tile variants; fills *info for variant in [0, count). Returns 0 on success. */
+int rocm_wmma_gemm_variant_count(void);
+int rocm_wmma_gemm_variant_info_get(int variant, rocm_wmma_gemm_variant_info* info);
+
+/* Which variant the dispatcher would pick for this problem (the table built from
+ * gemm_config_gfx950_*.json, then shape heuristics).  type_idx as above.
+ * Also reports the swizzle (tile-row group height) and split-K factor. Returns the
+ * variant index, or -1 for invalid arguments. */
+int rocm_wmma_gemm_select(size_t M, size_t N, size_t K, int type_idx, int layout_c, int layout_a,
+                          int layout_b, int* swizzle, int* split_k);
+
+/* Same computation as the four entry points above, but with the tile variant,
+ * swizzle and split-K factor forced (tuner hook).  Returns 0 on success, -1 if the
+ * variant cannot run this problem, -2 for invalid arguments. */
+int rocm_wmma_gemm_run_variant(int type_idx, int variant, int swizzle, int split_k, void* C,
+                               void* A, void* B, size_t M, size_t N, size_t K,
+                               size_t batch_count, int layout_c, int layout_a, int layout_b,
+                               void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* ROCM_WMMA_GEMM_C_H */

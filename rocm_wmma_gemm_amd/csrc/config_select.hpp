@@ -1,0 +1,61 @@
+// Shape -> launch plan.  The tuned table comes from gemm_config_gfx950_*.json via
+// config/generate_config.py; shapes the table does not name are served by its
+// nearest entry, and layouts it does not cover at all by a shape heuristic.
+//
+// Selection order follows the reference's generated find_best_config /
+// find_closest_config (reference rocm_wmma_gemm/config/generate_config.py:174-271):
+//   1. exact (M, N, K, type group, layouts) hit;
+//   2. for the fp32-output group, an exact hit in the 16-bit-output group;
+//   3. nearest entry with the same type group and layouts: nearest K first, then
+//      smallest squared (M, N) distance; an empty group falls back to group 0.
+// Unlike the reference there is no sentinel index doubling as "not found", so a
+// genuine hit on any entry is honoured.
+#ifndef ROCM_WMMA_GEMM_CONFIG_SELECT_HPP
+#define ROCM_WMMA_GEMM_CONFIG_SELECT_HPP
+
+#include <cstddef>
+
+namespace rocm_wmma_gemm
+{
+namespace host
+{
+
+struct launch_plan
+{
+    int variant; // index into the compiled variant table
+    int swizzle; // tile-row band height of the tile map
+    int split_k; // K slices (1 = off)
+};
+
+struct tuned_entry
+{
+    size_t m, n, k;
+    int    type_group; // 0: C is 16-bit (f16_f16, bf16_bf16); 1: C is fp32
+    int    layout_a, layout_b, layout_c; // 0 row-major, 1 column-major
+    launch_plan plan;
+};
+
+// Defined in config_select.cpp
+extern const tuned_entry* const tuned_table;
+extern const size_t             tuned_count;
+
+// Pure functions over a table (unit-testable with any table).
+bool find_exact(const tuned_entry* table, size_t count, size_t m, size_t n, size_t k,
+                int type_group, int la, int lb, int lc, launch_plan* out);
+bool find_closest(const tuned_entry* table, size_t count, size_t m, size_t n, size_t k,
+                  int type_group, int la, int lb, int lc, launch_plan* out);
+launch_plan heuristic_plan(size_t m, size_t n, size_t k, int lc);
+launch_plan select_plan_from(const tuned_entry* table, size_t count, size_t m, size_t n, size_t k,
+                             int type_idx, int lc, int la, int lb);
+
+inline int type_group_of(int type_idx)
+{
+    return (type_idx == 1 || type_idx == 3) ? 1 : 0;
+}
+
+launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int la, int lb);
+
+} // namespace host
+} // namespace rocm_wmma_gemm
+
+#endif

@@ -1,0 +1,486 @@
+// Host side of librocm_wmma_gemm_gfx950.so: the templated gemm<> entry points, the
+// config lookup, the launch, and the C ABI that the runtime loader binds.
+//
+// Interface parity: reference rocm_wmma_gemm/src/gemm.cpp:8-53 (dispatch),
+// :56-198 (explicit instantiations), :207-250 (C ABI).
+#include <rocm_wmma_gemm/gemm.hpp>
+#include <rocm_wmma_gemm_c.h>
+
+#include <mutex>
+#include <stdexcept>
+#include <string>
+#include <type_traits>
+
+#include "config_select.hpp"
+#include "kernel_table.hpp"
+
+namespace rocm_wmma_gemm
+{
+namespace host
+{
+
+#define RWG_VARIANT(IDX, BM, BN, BK, WM, WN, PIPE)                                         \
+    {BM, BN, BK, WM, WN, PIPE, 2 * (BM + BN) * (BK / 8) * 16, 64 * WM * WN},
+const variant_desc variant_table[num_variants] = {
+#include "variants.def"
+};
+#undef RWG_VARIANT
+
+kernel_fn lookup_kernel(int type_idx, bool a_kmajor, bool b_kmajor, int variant, int mode)
+{
+    if(type_idx < 0 || type_idx >= num_types || variant < 0 || variant >= num_variants || mode < 0
+       || mode >= num_modes)
+    {
+        return nullptr;
+    }
+    const int key = type_idx * 4 + (a_kmajor ? 2 : 0) + (b_kmajor ? 1 : 0);
+    switch(key)
+    {
+#define RWG_CASE(T, AK, BK_) \
+    case T * 4 + AK * 2 + BK_: return kernel_slice_##T##_##AK##_##BK_[variant][mode];
+        RWG_CASE(0, 0, 0)
+        RWG_CASE(0, 0, 1)
+        RWG_CASE(0, 1, 0)
+        RWG_CASE(0, 1, 1)
+        RWG_CASE(1, 0, 0)
+        RWG_CASE(1, 0, 1)
+        RWG_CASE(1, 1, 0)
+        RWG_CASE(1, 1, 1)
+        RWG_CASE(2, 0, 0)
+        RWG_CASE(2, 0, 1)
+        RWG_CASE(2, 1, 0)
+        RWG_CASE(2, 1, 1)
+        RWG_CASE(3, 0, 0)
+        RWG_CASE(3, 0, 1)
+        RWG_CASE(3, 1, 0)
+        RWG_CASE(3, 1, 1)
+#undef RWG_CASE
+        default: return nullptr;
+    }
+}
+
+namespace
+{
+
+constexpr size_t in_bytes = 2;
+
+size_t out_bytes(int type_idx)
+{
+    return (type_idx == 1 || type_idx == 3) ? 4 : 2;
+}
+
+// Split-K workspace: one fp32 buffer per device, allocated on first use and kept
+// for the life of the process.  Calls that need more than the cap run with fewer
+// slices instead.
+constexpr size_t workspace_cap_bytes = size_t{256} << 20;
+constexpr int    max_devices         = 64;
+std::mutex       workspace_mutex;
+float*           workspace_ptr[max_devices] = {};
+
+float* workspace_for_current_device()
+{
+    int dev = 0;
+    if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= max_devices)
+    {
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(workspace_mutex);
+    if(workspace_ptr[dev] == nullptr)
+    {
+        void* p = nullptr;
+        if(hipMalloc(&p, workspace_cap_bytes) != hipSuccess)
+        {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        workspace_ptr[dev] = static_cast<float*>(p);
+    }
+    return workspace_ptr[dev];
+}
+
+bool aligned16(const void* p)
+{
+    return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+// The problem as the kernels see it: C row-major, operands tagged by whether K is
+// their contiguous dimension.
+struct kernel_problem
+{
+    void*       C;
+    const void* A;
+    const void* B;
+    size_t      M, N, K, batch;
+    bool        a_kmajor, b_kmajor;
+    size_t      stride_a, stride_b, stride_c;
+};
+
+kernel_problem to_kernel_space(void* C, void* A, void* B, size_t M, size_t N, size_t K,
+                               size_t batch, int layout_c, int layout_a, int layout_b)
+{
+    kernel_problem p;
+    p.K     = K;
+    p.batch = batch;
+    p.C     = C;
+    if(layout_c == 0)
+    {
+        p.A        = A;
+        p.B        = B;
+        p.M        = M;
+        p.N        = N;
+        p.a_kmajor = layout_a == 0; // row-major M x K: K contiguous
+        p.b_kmajor = layout_b == 1; // column-major K x N: K contiguous
+        p.stride_a = M * K;
+        p.stride_b = K * N;
+    }
+    else
+    {
+        // Column-major C (M x N) is the row-major N x M matrix C^T = B^T * A^T.  B^T
+        // (N x K) is the same buffer as B with the opposite layout tag, likewise A^T.
+        p.A        = B;
+        p.B        = A;
+        p.M        = N;
+        p.N        = M;
+        p.a_kmajor = layout_b == 1; // B^T is K-contiguous iff B is column-major
+        p.b_kmajor = layout_a == 0; // A^T (K x M) is K-contiguous iff A is row-major
+        p.stride_a = K * N;
+        p.stride_b = M * K;
+    }
+    p.stride_c = M * N;
+    return p;
+}
+
+int pick_mode(const kernel_problem& p, const variant_desc& v, int split_k)
+{
+    const bool batch_ok = p.batch == 1 || ((p.stride_a % 8 == 0) && (p.stride_b % 8 == 0));
+    const bool a_vec    = (p.a_kmajor ? p.K % 8 == 0 : p.M % 8 == 0) && aligned16(p.A);
+    const bool b_vec    = (p.b_kmajor ? p.K % 8 == 0 : p.N % 8 == 0) && aligned16(p.B);
+    if(!(a_vec && b_vec && batch_ok))
+    {
+        return static_cast<int>(device::load_mode::scalar);
+    }
+    (void)split_k;
+    const bool full = p.M % v.block_m == 0 && p.N % v.block_n == 0 && p.K % v.block_k == 0;
+    return static_cast<int>(full ? device::load_mode::vec_unguarded
+                                 : device::load_mode::vec_guarded);
+}
+
+template<class OutT>
+void zero_fill(void* C, size_t count, hipStream_t stream)
+{
+    const int blocks = static_cast<int>(std::min<size_t>((count + 255) / 256, 65535));
+    device::fill_zero<OutT><<<dim3(blocks), dim3(256), 0, stream>>>(static_cast<OutT*>(C),
+                                                                     static_cast<long long>(count));
+}
+
+template<class OutT>
+int launch(int type_idx, const launch_plan& plan, const kernel_problem& p, hipStream_t stream)
+{
+    if(plan.variant < 0 || plan.variant >= num_variants)
+    {
+        return -1;
+    }
+    const variant_desc& v = variant_table[plan.variant];
+    if(p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull)
+    {
+        throw std::runtime_error("rocm_wmma_gemm: M, N and K must each fit in 31 bits");
+    }
+    const size_t grid_m = (p.M + v.block_m - 1) / v.block_m;
+    const size_t grid_n = (p.N + v.block_n - 1) / v.block_n;
+    if(grid_m * grid_n > 0x7fffffffull)
+    {
+        throw std::runtime_error("rocm_wmma_gemm: tile grid too large");
+    }
+
+    int       split_k = plan.split_k < 1 ? 1 : plan.split_k;
+    const int k_steps = static_cast<int>((p.K + v.block_k - 1) / v.block_k);
+    if(split_k > k_steps)
+    {
+        split_k = k_steps;
+    }
+    float* partials = nullptr;
+    if(split_k > 1)
+    {
+        // shrink the split until one chunk of batches fits the workspace
+        const size_t plane = p.M * p.N * sizeof(float);
+        while(split_k > 1 && plane * split_k > workspace_cap_bytes)
+        {
+            --split_k;
+        }
+        partials = split_k > 1 ? workspace_for_current_device() : nullptr;
+        if(partials == nullptr)
+        {
+            split_k = 1;
+        }
+    }
+    if(grid_m * grid_n * split_k > 0x7fffffffull)
+    {
+        split_k = 1;
+    }
+
+    const int mode = pick_mode(p, v, split_k);
+    kernel_fn fn   = lookup_kernel(type_idx, p.a_kmajor, p.b_kmajor, plan.variant, mode);
+    if(fn == nullptr)
+    {
+        // reference kernel_launcher.hpp:119-125 throws the same way
+        throw std::runtime_error("No kernel available for the requested configuration and layout");
+    }
+
+    // Batches per launch: bounded by grid.y and, under split-K, by the workspace.
+    size_t batches_per_launch = 65535;
+    if(split_k > 1)
+    {
+        const size_t fit = workspace_cap_bytes / (p.M * p.N * sizeof(float) * split_k);
+        batches_per_launch = std::min(batches_per_launch, std::max<size_t>(fit, 1));
+    }
+
+    for(size_t b0 = 0; b0 < p.batch; b0 += batches_per_launch)
+    {
+        const size_t nb = std::min(batches_per_launch, p.batch - b0);
+        device::gemm_args args;
+        args.C = static_cast<char*>(p.C) + b0 * p.stride_c * sizeof(OutT);
+        args.A = static_cast<const char*>(p.A) + b0 * p.stride_a * in_bytes;
+        args.B = static_cast<const char*>(p.B) + b0 * p.stride_b * in_bytes;
+        args.M = static_cast<int>(p.M);
+        args.N = static_cast<int>(p.N);
+        args.K = static_cast<int>(p.K);
+        args.batch_stride_a = static_cast<long long>(p.stride_a);
+        args.batch_stride_b = static_cast<long long>(p.stride_b);
+        args.batch_stride_c = static_cast<long long>(p.stride_c);
+        args.grid_m         = static_cast<int>(grid_m);
+        args.grid_n         = static_cast<int>(grid_n);
+        args.group          = plan.swizzle < 1 ? 1 : plan.swizzle;
+        args.k_slices       = split_k;
+        args.partials       = partials;
+
+        const dim3 grid(static_cast<unsigned>(grid_m * grid_n * split_k), static_cast<unsigned>(nb));
+        fn<<<grid, dim3(v.threads), 0, stream>>>(args);
+        if(split_k > 1)
+        {
+            const long long plane  = static_cast<long long>(p.M) * static_cast<long long>(p.N);
+            const int       blocks = static_cast<int>(std::min<long long>((plane + 255) / 256, 4096));
+            device::reduce_partials<OutT>
+                <<<dim3(blocks, static_cast<unsigned>(nb)), dim3(256), 0, stream>>>(
+                    static_cast<OutT*>(args.C), partials, plane, split_k, args.batch_stride_c);
+        }
+    }
+    return 0;
+}
+
+template<class OutT>
+int run(int type_idx, const launch_plan* forced, void* C, void* A, void* B, size_t M, size_t N,
+        size_t K, size_t batch, int layout_c, int layout_a, int layout_b, hipStream_t stream)
+{
+    if((layout_c | layout_a | layout_b) & ~1)
+    {
+        return -2; // reference src/gemm.cpp:243: unknown layout key -> nothing happens
+    }
+    if(M == 0 || N == 0 || batch == 0)
+    {
+        return 0;
+    }
+    if(K == 0)
+    {
+        zero_fill<OutT>(C, M * N * batch, stream);
+        return 0;
+    }
+    const kernel_problem p = to_kernel_space(C, A, B, M, N, K, batch, layout_c, layout_a, layout_b);
+    launch_plan          plan
+        = forced ? *forced : select_plan(M, N, K, type_idx, layout_c, layout_a, layout_b);
+    if(!forced)
+    {
+        // The 2-byte-load fallback keeps far more values in flight per thread; the
+        // small tile is the variant built to hold them without spilling.
+        const int mode = pick_mode(p, variant_table[plan.variant], plan.split_k);
+        if(mode == static_cast<int>(device::load_mode::scalar))
+        {
+            plan.variant = 0;
+        }
+    }
+    return launch<OutT>(type_idx, plan, p, stream);
+}
+
+template<class T, class U>
+constexpr int type_index()
+{
+    if(std::is_same<T, half>::value && std::is_same<U, half>::value)
+        return 0;
+    if(std::is_same<T, float>::value && std::is_same<U, half>::value)
+        return 1;
+    if(std::is_same<T, __hip_bfloat16>::value && std::is_same<U, __hip_bfloat16>::value)
+        return 2;
+    if(std::is_same<T, float>::value && std::is_same<U, __hip_bfloat16>::value)
+        return 3;
+    return -1;
+}
+
+int run_by_type(int type_idx, const launch_plan* forced, void* C, void* A, void* B, size_t M,
+                size_t N, size_t K, size_t batch, int lc, int la, int lb, hipStream_t stream)
+{
+    switch(type_idx)
+    {
+        case 0: return run<_Float16>(0, forced, C, A, B, M, N, K, batch, lc, la, lb, stream);
+        case 1: return run<float>(1, forced, C, A, B, M, N, K, batch, lc, la, lb, stream);
+        case 2: return run<__bf16>(2, forced, C, A, B, M, N, K, batch, lc, la, lb, stream);
+        case 3: return run<float>(3, forced, C, A, B, M, N, K, batch, lc, la, lb, stream);
+        default: return -2;
+    }
+}
+
+} // namespace
+} // namespace host
+
+// ---------------------------------------------------------------------------
+// C++ API (reference gemm.hpp:50-73, src/gemm.cpp:8-53)
+// ---------------------------------------------------------------------------
+template<m_layout layout_C, m_layout layout_A, m_layout layout_B, class T, class U>
+__host__ void
+    gemm(T* C, U* A, U* B, size_t M, size_t N, size_t K, size_t batch_count, hipStream_t& stream)
+{
+    constexpr int type_idx = host::type_index<T, U>();
+    static_assert(type_idx >= 0, "unsupported type pair");
+    host::run_by_type(type_idx,
+                      nullptr,
+                      C,
+                      A,
+                      B,
+                      M,
+                      N,
+                      K,
+                      batch_count,
+                      static_cast<int>(layout_C),
+                      static_cast<int>(layout_A),
+                      static_cast<int>(layout_B),
+                      stream);
+}
+
+template<m_layout layout_C, m_layout layout_A, m_layout layout_B, class T, class U>
+__host__ void gemm(T* C, U* A, U* B, size_t M, size_t N, size_t K, hipStream_t& stream)
+{
+    gemm<layout_C, layout_A, layout_B, T, U>(C, A, B, M, N, K, size_t{1}, stream);
+}
+
+#define ROCM_WMMA_GEMM_INSTANTIATE(LC, LA, LB, T, U)                                          \
+    template void gemm<LC, LA, LB, T, U>(T*, U*, U*, size_t, size_t, size_t, hipStream_t&);   \
+    template void gemm<LC, LA, LB, T, U>(T*, U*, U*, size_t, size_t, size_t, size_t,          \
+                                         hipStream_t&);
+ROCM_WMMA_GEMM_FOR_EACH_TYPE_PAIR(ROCM_WMMA_GEMM_INSTANTIATE)
+#undef ROCM_WMMA_GEMM_INSTANTIATE
+
+} // namespace rocm_wmma_gemm
+
+// ---------------------------------------------------------------------------
+// C ABI (reference src/gemm.cpp:207-250)
+// ---------------------------------------------------------------------------
+namespace
+{
+inline hipStream_t stream_of(void* stream)
+{
+    return stream ? *static_cast<hipStream_t*>(stream) : nullptr;
+}
+} // namespace
+
+extern "C" {
+
+void rocm_wmma_gemm_f16_f16(void* C, void* A, void* B, size_t M, size_t N, size_t K,
+                            size_t batch_count, int layout_c, int layout_a, int layout_b,
+                            void* stream)
+{
+    rocm_wmma_gemm::host::run_by_type(
+        0, nullptr, C, A, B, M, N, K, batch_count, layout_c, layout_a, layout_b, stream_of(stream));
+}
+
+void rocm_wmma_gemm_f32_f16(void* C, void* A, void* B, size_t M, size_t N, size_t K,
+                            size_t batch_count, int layout_c, int layout_a, int layout_b,
+                            void* stream)
+{
+    rocm_wmma_gemm::host::run_by_type(
+        1, nullptr, C, A, B, M, N, K, batch_count, layout_c, layout_a, layout_b, stream_of(stream));
+}
+
+void rocm_wmma_gemm_bf16_bf16(void* C, void* A, void* B, size_t M, size_t N, size_t K,
+                              size_t batch_count, int layout_c, int layout_a, int layout_b,
+                              void* stream)
+{
+    rocm_wmma_gemm::host::run_by_type(
+        2, nullptr, C, A, B, M, N, K, batch_count, layout_c, layout_a, layout_b, stream_of(stream));
+}
+
+void rocm_wmma_gemm_f32_bf16(void* C, void* A, void* B, size_t M, size_t N, size_t K,
+                             size_t batch_count, int layout_c, int layout_a, int layout_b,
+                             void* stream)
+{
+    rocm_wmma_gemm::host::run_by_type(
+        3, nullptr, C, A, B, M, N, K, batch_count, layout_c, layout_a, layout_b, stream_of(stream));
+}
+
+const char* rocm_wmma_gemm_arch(void)
+{
+    return "gfx950";
+}
+
+int rocm_wmma_gemm_variant_count(void)
+{
+    return rocm_wmma_gemm::host::num_variants;
+}
+
+int rocm_wmma_gemm_variant_info_get(int variant, rocm_wmma_gemm_variant_info* info)
+{
+    using namespace rocm_wmma_gemm::host;
+    if(variant < 0 || variant >= num_variants || info == nullptr)
+    {
+        return -1;
+    }
+    const variant_desc& v = variant_table[variant];
+    info->block_m         = v.block_m;
+    info->block_n         = v.block_n;
+    info->block_k         = v.block_k;
+    info->warps_m         = v.waves_m;
+    info->warps_n         = v.waves_n;
+    info->warp_tile_m     = v.block_m / v.waves_m / 32;
+    info->warp_tile_n     = v.block_n / v.waves_n / 32;
+    info->pipeline        = v.pipeline;
+    info->lds_bytes       = v.lds_bytes;
+    info->threads         = v.threads;
+    return 0;
+}
+
+int rocm_wmma_gemm_select(size_t M, size_t N, size_t K, int type_idx, int layout_c, int layout_a,
+                          int layout_b, int* swizzle, int* split_k)
+{
+    using namespace rocm_wmma_gemm::host;
+    if(type_idx < 0 || type_idx >= num_types || ((layout_c | layout_a | layout_b) & ~1))
+    {
+        return -1;
+    }
+    const launch_plan plan = select_plan(M, N, K, type_idx, layout_c, layout_a, layout_b);
+    if(swizzle)
+    {
+        *swizzle = plan.swizzle;
+    }
+    if(split_k)
+    {
+        *split_k = plan.split_k;
+    }
+    return plan.variant;
+}
+
+int rocm_wmma_gemm_run_variant(int type_idx, int variant, int swizzle, int split_k, void* C,
+                               void* A, void* B, size_t M, size_t N, size_t K,
+                               size_t batch_count, int layout_c, int layout_a, int layout_b,
+                               void* stream)
+{
+    using namespace rocm_wmma_gemm::host;
+    if(type_idx < 0 || type_idx >= num_types || variant < 0 || variant >= num_variants)
+    {
+        return -2;
+    }
+    launch_plan plan;
+    plan.variant = variant;
+    plan.swizzle = swizzle;
+    plan.split_k = split_k;
+    return run_by_type(type_idx, &plan, C, A, B, M, N, K, batch_count, layout_c, layout_a,
+                       layout_b, stream_of(stream));
+}
+
+} // extern "C"

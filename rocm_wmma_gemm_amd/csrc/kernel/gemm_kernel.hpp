@@ -1,0 +1,561 @@
+// Register-staged MFMA GEMM kernel for gfx950 (wave64, v_mfma_f32_32x32x16).
+//
+// One workgroup computes a BM x BN tile of a ROW-MAJOR C over the whole K range
+// (or over one K slice when split-K is on).  Column-major C is served by the host
+// as the transposed problem, so no kernel here ever writes a column-major C.
+//
+// Data path per K step of BK:
+//   global --(16-byte or 2-byte guarded loads)--> VGPRs --> LDS --> MFMA operands
+// Both operand tiles live in LDS in the same K-contiguous form, whatever their
+// layout in memory: row r of the tile is BK elements, stored as BK/8 chunks of
+// 16 bytes, chunk c of row r at slot c ^ swizzle(r).  An operand that is
+// contiguous along M or N in memory is transposed in registers (8x8 blocks of
+// 16-bit elements) on its way to LDS, so its global loads stay 16 bytes wide and
+// coalesced along the contiguous dimension.
+//
+// This kernel replaces the reference's gemm_impl / prefetch_fragment /
+// load_matrix / store_matrix / load_shared_to_global chain (reference
+// rocm_wmma_gemm/include/rocm_wmma_gemm/kernel/kernel.hpp:108-556,
+// kernel/load.hpp:348-966, kernel/fragment.hpp:191-404) and its WMMA wrapper
+// (kernel/wmma.hpp:44-85).  Unlike the reference it accumulates in fp32 for every
+// type pair, guards M, N and K tails, and accepts odd leading dimensions.
+#ifndef ROCM_WMMA_GEMM_GEMM_KERNEL_HPP
+#define ROCM_WMMA_GEMM_GEMM_KERNEL_HPP
+
+#include <hip/hip_runtime.h>
+
+#include "tile_map.hpp"
+
+namespace rocm_wmma_gemm
+{
+namespace device
+{
+
+using u32x4  = unsigned int __attribute__((ext_vector_type(4)));
+using f16x8  = _Float16 __attribute__((ext_vector_type(8)));
+using bf16x8 = __bf16 __attribute__((ext_vector_type(8)));
+using f32x16 = float __attribute__((ext_vector_type(16)));
+
+enum class in_kind
+{
+    f16  = 0,
+    bf16 = 1
+};
+
+// How operand tiles are fetched from global memory.
+enum class load_mode
+{
+    vec_unguarded = 0, // 16-byte loads, tile fully inside the matrix, K % BK == 0
+    vec_guarded   = 1, // 16-byte loads, whole chunks zero-filled outside the matrix
+    scalar        = 2 // 2-byte guarded loads: any leading dimension, any alignment
+};
+
+struct gemm_args
+{
+    void*       C;
+    const void* A;
+    const void* B;
+    int         M, N, K; // C is M x N row-major in kernel space
+    long long   batch_stride_a, batch_stride_b, batch_stride_c; // elements
+    int         grid_m, grid_n; // tiles along M and N
+    int         group; // tile-row band height of the tile map
+    int         k_slices; // split-K factor (1 = off)
+    float*      partials; // split-K workspace: [slice][M][N] fp32, or nullptr
+};
+
+template<in_kind IN>
+__device__ __forceinline__ f32x16 mfma_32x32x16(u32x4 a, u32x4 b, f32x16 c)
+{
+    if constexpr(IN == in_kind::f16)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(
+            __builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    else
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+}
+
+// fp32 -> C element, round to nearest even.
+template<class OutT>
+__device__ __forceinline__ OutT to_out(float v)
+{
+    return static_cast<OutT>(v);
+}
+
+// Chunk slot swizzle: rows whose chunks would otherwise land in the same LDS
+// banks get distinct slots.  CH = chunks per row (8 for BK=64, 4 for BK=32).
+template<int CH>
+__device__ __forceinline__ int swizzle_of_row(int row)
+{
+    static_assert(CH == 8 || CH == 4 || CH == 2, "unsupported BK");
+    return (row * CH / 8) % CH;
+}
+
+// 16-byte chunk index (in u32x4 units) of (row, chunk) inside a tile.
+template<int CH>
+__device__ __forceinline__ int lds_chunk_index(int row, int chunk)
+{
+    return row * CH + (chunk ^ swizzle_of_row<CH>(row));
+}
+
+// ---------------------------------------------------------------------------
+// Global -> register staging of one operand tile.
+//
+// The tile is ROWS x BK in (row, k) space; element (row, k) of the operand sits at
+// base[row * stride_row + k * stride_k], with (stride_row, stride_k) = (ld, 1) for a
+// K-contiguous operand (KMAJOR) and (1, ld) otherwise.  Rows >= rows_left and
+// k >= k_left read as zero.
+// ---------------------------------------------------------------------------
+template<bool KMAJOR, int ROWS, int BK, int THREADS, load_mode MODE>
+struct operand_stage
+{
+    static constexpr int CH     = BK / 8; // 16-byte chunks per tile row
+    static constexpr int CHUNKS = ROWS * CH; // chunks per tile
+    static_assert(CHUNKS % THREADS == 0, "tile must divide evenly over the workgroup");
+    static constexpr int PER_THREAD = CHUNKS / THREADS;
+
+    // M/N-contiguous operands in vector mode are moved as 8(k) x VW(row) blocks.
+    static constexpr int VW     = PER_THREAD >= 8 ? 8 : (PER_THREAD >= 4 ? 4 : (PER_THREAD >= 2 ? 2 : 1));
+    static constexpr int BLOCKS = PER_THREAD / VW; // blocks per thread (transposed path)
+    static constexpr bool TRANSPOSED = !KMAJOR && MODE != load_mode::scalar;
+    static_assert(!TRANSPOSED || VW >= 2, "transposed path needs at least 2 chunks per thread");
+    static_assert(!TRANSPOSED || ROWS % VW == 0, "rows must divide into blocks");
+
+    // Data in flight.  KMAJOR/scalar: regs[i] is the finished LDS chunk i.
+    // TRANSPOSED: regs[b*VW .. b*VW+VW) hold block b, already transposed by fetch().
+    u32x4 regs[PER_THREAD];
+
+    // --- chunk ownership -------------------------------------------------
+    // K-contiguous / scalar K-contiguous: consecutive threads take consecutive
+    // chunks of a row (coalesced along k).  Scalar M/N-contiguous: consecutive
+    // threads take consecutive rows of the same chunk column (coalesced along row).
+    __device__ __forceinline__ static void chunk_of(int i, int tid, int& row, int& chunk)
+    {
+        const int c = tid + i * THREADS;
+        if constexpr(KMAJOR)
+        {
+            row   = c / CH;
+            chunk = c % CH;
+        }
+        else
+        {
+            row   = c % ROWS;
+            chunk = c / ROWS;
+        }
+    }
+    // Transposed path: block b covers rows [rb*VW, rb*VW+VW) and chunk column kb.
+    __device__ __forceinline__ static void block_of(int b, int tid, int& row0, int& chunk)
+    {
+        constexpr int ROW_BLOCKS = ROWS / VW;
+        const int     c          = tid + b * THREADS;
+        row0                     = (c % ROW_BLOCKS) * VW;
+        chunk                    = c / ROW_BLOCKS;
+    }
+
+    template<class InT>
+    __device__ __forceinline__ void fetch(const InT* __restrict__ base,
+                                          long long               stride_row,
+                                          long long               stride_k,
+                                          int                     rows_left,
+                                          int                     k_left,
+                                          int                     tid)
+    {
+        if constexpr(MODE == load_mode::scalar)
+        {
+#pragma unroll
+            for(int i = 0; i < PER_THREAD; ++i)
+            {
+                int row, chunk;
+                chunk_of(i, tid, row, chunk);
+                unsigned short e[8];
+#pragma unroll
+                for(int j = 0; j < 8; ++j)
+                {
+                    const int  k  = chunk * 8 + j;
+                    const bool ok = row < rows_left && k < k_left;
+                    const auto* p = reinterpret_cast<const unsigned short*>(base)
+                                    + (ok ? row * stride_row + k * stride_k : 0);
+                    const unsigned short v = *p;
+                    e[j]                   = ok ? v : (unsigned short)0;
+                }
+                u32x4 r;
+                r.x     = (unsigned)e[0] | ((unsigned)e[1] << 16);
+                r.y     = (unsigned)e[2] | ((unsigned)e[3] << 16);
+                r.z     = (unsigned)e[4] | ((unsigned)e[5] << 16);
+                r.w     = (unsigned)e[6] | ((unsigned)e[7] << 16);
+                regs[i] = r;
+            }
+        }
+        else if constexpr(KMAJOR)
+        {
+#pragma unroll
+            for(int i = 0; i < PER_THREAD; ++i)
+            {
+                int row, chunk;
+                chunk_of(i, tid, row, chunk);
+                const int k = chunk * 8;
+                if constexpr(MODE == load_mode::vec_unguarded)
+                {
+                    regs[i] = *reinterpret_cast<const u32x4*>(base + row * stride_row + k);
+                }
+                else
+                {
+                    const bool ok = row < rows_left && k < k_left;
+                    u32x4      v  = {0u, 0u, 0u, 0u};
+                    if(ok)
+                    {
+                        v = *reinterpret_cast<const u32x4*>(base + row * stride_row + k);
+                    }
+                    regs[i] = v;
+                }
+            }
+        }
+        else
+        {
+            // 8 (k) x VW (row) block: VW*2-byte loads down 8 consecutive k, then an
+            // in-register transpose so that each of the VW rows owns 8 consecutive k.
+#pragma unroll
+            for(int b = 0; b < BLOCKS; ++b)
+            {
+                int row0, chunk;
+                block_of(b, tid, row0, chunk);
+                unsigned int src[8][VW / 2]; // src[kk][pair of rows]
+#pragma unroll
+                for(int kk = 0; kk < 8; ++kk)
+                {
+                    const int  k = chunk * 8 + kk;
+                    const bool ok
+                        = MODE == load_mode::vec_unguarded || (row0 < rows_left && k < k_left);
+                    const InT* p = base + (ok ? k * stride_k + row0 : 0);
+                    if constexpr(VW == 8)
+                    {
+                        u32x4 v = *reinterpret_cast<const u32x4*>(p);
+                        src[kk][0] = ok ? v.x : 0u;
+                        src[kk][1] = ok ? v.y : 0u;
+                        src[kk][2] = ok ? v.z : 0u;
+                        src[kk][3] = ok ? v.w : 0u;
+                    }
+                    else if constexpr(VW == 4)
+                    {
+                        uint2 v    = *reinterpret_cast<const uint2*>(p);
+                        src[kk][0] = ok ? v.x : 0u;
+                        src[kk][1] = ok ? v.y : 0u;
+                    }
+                    else
+                    {
+                        unsigned int v = *reinterpret_cast<const unsigned int*>(p);
+                        src[kk][0]     = ok ? v : 0u;
+                    }
+                }
+#pragma unroll
+                for(int r = 0; r < VW; ++r)
+                {
+                    // row r of the block takes half (r & 1) of dword r/2 from each k.
+                    const unsigned sel = (r & 1) ? 0x07060302u : 0x05040100u;
+                    u32x4          out;
+                    out.x = __builtin_amdgcn_perm(src[1][r / 2], src[0][r / 2], sel);
+                    out.y = __builtin_amdgcn_perm(src[3][r / 2], src[2][r / 2], sel);
+                    out.z = __builtin_amdgcn_perm(src[5][r / 2], src[4][r / 2], sel);
+                    out.w = __builtin_amdgcn_perm(src[7][r / 2], src[6][r / 2], sel);
+                    regs[b * VW + r] = out;
+                }
+            }
+        }
+    }
+
+    __device__ __forceinline__ void commit(u32x4* __restrict__ tile, int tid) const
+    {
+        if constexpr(TRANSPOSED)
+        {
+#pragma unroll
+            for(int b = 0; b < BLOCKS; ++b)
+            {
+                int row0, chunk;
+                block_of(b, tid, row0, chunk);
+#pragma unroll
+                for(int r = 0; r < VW; ++r)
+                {
+                    tile[lds_chunk_index<CH>(row0 + r, chunk)] = regs[b * VW + r];
+                }
+            }
+        }
+        else
+        {
+#pragma unroll
+            for(int i = 0; i < PER_THREAD; ++i)
+            {
+                int row, chunk;
+                chunk_of(i, tid, row, chunk);
+                tile[lds_chunk_index<CH>(row, chunk)] = regs[i];
+            }
+        }
+    }
+};
+
+// ---------------------------------------------------------------------------
+// The kernel
+// ---------------------------------------------------------------------------
+template<in_kind IN,
+         class OutT,
+         bool      A_KMAJOR,
+         bool      B_KMAJOR,
+         int       BM,
+         int       BN,
+         int       BK,
+         int       WAVES_M,
+         int       WAVES_N,
+         load_mode MODE>
+struct staged_gemm
+{
+    using InT = typename std::conditional<IN == in_kind::f16, _Float16, __bf16>::type;
+
+    static constexpr int THREADS = 64 * WAVES_M * WAVES_N;
+    static constexpr int WTM     = BM / WAVES_M; // rows per wave
+    static constexpr int WTN     = BN / WAVES_N; // columns per wave
+    static constexpr int TM      = WTM / 32; // MFMA tiles per wave along M
+    static constexpr int TN      = WTN / 32;
+    static constexpr int CH      = BK / 8;
+    static constexpr int A_TILE  = BM * CH; // u32x4 units
+    static constexpr int B_TILE  = BN * CH;
+    static constexpr int STAGE   = A_TILE + B_TILE;
+    static constexpr int LDS_BYTES = 2 * STAGE * 16;
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be built from 32x32 MFMA tiles");
+    static_assert(BK % 16 == 0, "BK must hold whole MFMA K steps");
+    static_assert(LDS_BYTES <= 160 * 1024, "tile does not fit the 160 KB LDS");
+
+    using stage_a = operand_stage<A_KMAJOR, BM, BK, THREADS, MODE>;
+    using stage_b = operand_stage<B_KMAJOR, BN, BK, THREADS, MODE>;
+
+    __device__ __forceinline__ static void compute_stage(const u32x4* __restrict__ lds_a,
+                                                         const u32x4* __restrict__ lds_b,
+                                                         f32x16 (&acc)[TM][TN],
+                                                         int row_in_wave_a,
+                                                         int row_in_wave_b,
+                                                         int lane_hi)
+    {
+#pragma unroll
+        for(int kk = 0; kk < BK / 16; ++kk)
+        {
+            u32x4     a[TM], b[TN];
+            const int chunk = kk * 2 + lane_hi;
+#pragma unroll
+            for(int i = 0; i < TM; ++i)
+            {
+                a[i] = lds_a[lds_chunk_index<CH>(row_in_wave_a + i * 32, chunk)];
+            }
+#pragma unroll
+            for(int j = 0; j < TN; ++j)
+            {
+                b[j] = lds_b[lds_chunk_index<CH>(row_in_wave_b + j * 32, chunk)];
+            }
+#pragma unroll
+            for(int i = 0; i < TM; ++i)
+            {
+#pragma unroll
+                for(int j = 0; j < TN; ++j)
+                {
+                    acc[i][j] = mfma_32x32x16<IN>(a[i], b[j], acc[i][j]);
+                }
+            }
+        }
+    }
+
+    __device__ static void run(const gemm_args& args)
+    {
+        __shared__ u32x4 lds[2 * STAGE];
+
+        const int tid     = threadIdx.x;
+        const int lane    = tid & 63;
+        const int wave    = tid >> 6;
+        const int wave_m  = wave / WAVES_N;
+        const int wave_n  = wave % WAVES_N;
+        const int lane_lo = lane & 31;
+        const int lane_hi = lane >> 5;
+
+        // blockIdx.x enumerates (k slice, tile); blockIdx.y the batch entry.
+        const int tiles   = args.grid_m * args.grid_n;
+        const int slice   = blockIdx.x / tiles;
+        const int tile_id = blockIdx.x - slice * tiles;
+        const tile_coord t = map_tile(tile_id, args.grid_m, args.grid_n, args.group);
+        const int row0 = t.m * BM;
+        const int col0 = t.n * BN;
+
+        // K range of this slice, in whole BK steps.
+        const int k_steps_total = (args.K + BK - 1) / BK;
+        const int steps_per     = (k_steps_total + args.k_slices - 1) / args.k_slices;
+        const int step_begin    = slice * steps_per;
+        int       step_end      = step_begin + steps_per;
+        if(step_end > k_steps_total)
+        {
+            step_end = k_steps_total;
+        }
+
+        const long long batch = blockIdx.y;
+        const InT* A = static_cast<const InT*>(args.A) + batch * args.batch_stride_a;
+        const InT* B = static_cast<const InT*>(args.B) + batch * args.batch_stride_b;
+
+        // Element (row, k) of A at A[row*a_sr + k*a_sk]; element (k, col) of B at B[col*b_sr + k*b_sk].
+        const long long a_sr = A_KMAJOR ? args.K : 1;
+        const long long a_sk = A_KMAJOR ? 1 : args.M;
+        const long long b_sr = B_KMAJOR ? args.K : 1;
+        const long long b_sk = B_KMAJOR ? 1 : args.N;
+
+        const InT* a_tile = A + row0 * a_sr;
+        const InT* b_tile = B + col0 * b_sr;
+        const int  rows_a = args.M - row0;
+        const int  rows_b = args.N - col0;
+
+        f32x16 acc[TM][TN];
+#pragma unroll
+        for(int i = 0; i < TM; ++i)
+        {
+#pragma unroll
+            for(int j = 0; j < TN; ++j)
+            {
+#pragma unroll
+                for(int v = 0; v < 16; ++v)
+                {
+                    acc[i][j][v] = 0.0f;
+                }
+            }
+        }
+
+        stage_a sa;
+        stage_b sb;
+
+        const int row_in_wave_a = wave_m * WTM + lane_lo;
+        const int row_in_wave_b = wave_n * WTN + lane_lo;
+
+        if(step_begin < step_end)
+        {
+            int k0 = step_begin * BK;
+            sa.fetch(a_tile + k0 * a_sk, a_sr, a_sk, rows_a, args.K - k0, tid);
+            sb.fetch(b_tile + k0 * b_sk, b_sr, b_sk, rows_b, args.K - k0, tid);
+            sa.commit(lds, tid);
+            sb.commit(lds + A_TILE, tid);
+            __syncthreads();
+
+            int cur = 0;
+            for(int step = step_begin; step < step_end; ++step)
+            {
+                const bool more = step + 1 < step_end;
+                if(more)
+                {
+                    k0 = (step + 1) * BK;
+                    sa.fetch(a_tile + k0 * a_sk, a_sr, a_sk, rows_a, args.K - k0, tid);
+                    sb.fetch(b_tile + k0 * b_sk, b_sr, b_sk, rows_b, args.K - k0, tid);
+                }
+                const u32x4* lds_a = lds + cur * STAGE;
+                compute_stage(lds_a, lds_a + A_TILE, acc, row_in_wave_a, row_in_wave_b, lane_hi);
+                if(more)
+                {
+                    u32x4* nxt = lds + (cur ^ 1) * STAGE;
+                    sa.commit(nxt, tid);
+                    sb.commit(nxt + A_TILE, tid);
+                }
+                __syncthreads();
+                cur ^= 1;
+            }
+        }
+
+        // Epilogue.  Accumulator register v of a 32x32 tile holds row
+        // 8*(v/4) + 4*(lane/32) + v%4 and column lane%32.
+        const bool guarded = MODE != load_mode::vec_unguarded;
+        if(args.k_slices == 1)
+        {
+            OutT* C = static_cast<OutT*>(args.C) + batch * args.batch_stride_c;
+#pragma unroll
+            for(int i = 0; i < TM; ++i)
+            {
+#pragma unroll
+                for(int j = 0; j < TN; ++j)
+                {
+                    const int col = col0 + wave_n * WTN + j * 32 + lane_lo;
+#pragma unroll
+                    for(int v = 0; v < 16; ++v)
+                    {
+                        const int row
+                            = row0 + wave_m * WTM + i * 32 + 8 * (v / 4) + 4 * lane_hi + (v % 4);
+                        if(!guarded || (row < args.M && col < args.N))
+                        {
+                            C[(long long)row * args.N + col] = to_out<OutT>(acc[i][j][v]);
+                        }
+                    }
+                }
+            }
+        }
+        else
+        {
+            // split-K: fp32 partial sums, reduced by a second kernel.
+            float* P = args.partials
+                       + ((long long)batch * args.k_slices + slice) * (long long)args.M * args.N;
+#pragma unroll
+            for(int i = 0; i < TM; ++i)
+            {
+#pragma unroll
+                for(int j = 0; j < TN; ++j)
+                {
+                    const int col = col0 + wave_n * WTN + j * 32 + lane_lo;
+#pragma unroll
+                    for(int v = 0; v < 16; ++v)
+                    {
+                        const int row
+                            = row0 + wave_m * WTM + i * 32 + 8 * (v / 4) + 4 * lane_hi + (v % 4);
+                        if(!guarded || (row < args.M && col < args.N))
+                        {
+                            P[(long long)row * args.N + col] = acc[i][j][v];
+                        }
+                    }
+                }
+            }
+        }
+    }
+};
+
+template<class Impl>
+__global__ void __launch_bounds__(Impl::THREADS) gemm_entry(const gemm_args args)
+{
+    Impl::run(args);
+}
+
+// Sums the k_slices fp32 partial planes of split-K in ascending slice order and
+// writes C (row-major M x N per batch entry) in its own element type.
+template<class OutT>
+__global__ void __launch_bounds__(256) reduce_partials(OutT* __restrict__ C,
+                                                       const float* __restrict__ partials,
+                                                       long long plane, // M*N
+                                                       int       k_slices,
+                                                       long long batch_stride_c)
+{
+    const long long batch = blockIdx.y;
+    const float*    P     = partials + batch * k_slices * plane;
+    OutT*           out   = C + batch * batch_stride_c;
+    for(long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < plane;
+        i += (long long)gridDim.x * blockDim.x)
+    {
+        float s = 0.0f;
+        for(int k = 0; k < k_slices; ++k)
+        {
+            s += P[k * plane + i];
+        }
+        out[i] = to_out<OutT>(s);
+    }
+}
+
+template<class OutT>
+__global__ void __launch_bounds__(256) fill_zero(OutT* __restrict__ C, long long count)
+{
+    for(long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < count;
+        i += (long long)gridDim.x * blockDim.x)
+    {
+        C[i] = to_out<OutT>(0.0f);
+    }
+}
+
+} // namespace device
+} // namespace rocm_wmma_gemm
+
+#endif // ROCM_WMMA_GEMM_GEMM_KERNEL_HPP

@@ -1,0 +1,373 @@
+// Hardware probe for gfx950: checks, on the GPU in the machine, the register
+// layouts and data-movement semantics the GEMM kernels are written against, and
+// measures two ceilings (MFMA issue rate, HBM copy rate).
+//
+//   mfma_probe            run every check, print PASS/FAIL lines and the ceilings
+//   mfma_probe --dump     additionally print raw lane dumps of the LDS paths
+//   mfma_probe --copy N   run only the copy kernel over N MiB (reference point for
+//                         scaling FETCH_SIZE / WRITE_SIZE counters)
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#define CHECK(x)                                                                          \
+    do                                                                                    \
+    {                                                                                     \
+        hipError_t e_ = (x);                                                              \
+        if(e_ != hipSuccess)                                                              \
+        {                                                                                 \
+            std::fprintf(stderr, "%s:%d %s: %s\n", __FILE__, __LINE__, #x, hipGetErrorString(e_)); \
+            std::exit(2);                                                                 \
+        }                                                                                 \
+    } while(0)
+
+using f16x8  = _Float16 __attribute__((ext_vector_type(8)));
+using bf16x8 = __bf16 __attribute__((ext_vector_type(8)));
+using f32x16 = float __attribute__((ext_vector_type(16)));
+using f32x4  = float __attribute__((ext_vector_type(4)));
+using u32x4  = unsigned __attribute__((ext_vector_type(4)));
+typedef __fp16 fp16x4_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
+
+// ---- 1. MFMA 32x32x16 layout --------------------------------------------------
+// Assumed: A operand lane l holds row l%32, k = 8*(l/32)+0..7; B operand lane l
+// holds column l%32, same k; D register v of lane l is row 8*(v/4)+4*(l/32)+v%4,
+// column l%32.
+template<bool BF16>
+__global__ void mfma32_layout(const float* A, const float* B, float* D)
+{
+    const int l = threadIdx.x;
+    f32x16    c = {0};
+    if constexpr(BF16)
+    {
+        bf16x8 a, b;
+        for(int j = 0; j < 8; ++j)
+        {
+            a[j] = (__bf16)A[(l % 32) * 16 + 8 * (l / 32) + j];
+            b[j] = (__bf16)B[(8 * (l / 32) + j) * 32 + (l % 32)];
+        }
+        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    else
+    {
+        f16x8 a, b;
+        for(int j = 0; j < 8; ++j)
+        {
+            a[j] = (_Float16)A[(l % 32) * 16 + 8 * (l / 32) + j];
+            b[j] = (_Float16)B[(8 * (l / 32) + j) * 32 + (l % 32)];
+        }
+        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    for(int v = 0; v < 16; ++v)
+    {
+        D[(8 * (v / 4) + 4 * (l / 32) + v % 4) * 32 + (l % 32)] = c[v];
+    }
+}
+
+// Assumed for 16x16x32: A lane l row l%16, k = 8*(l/16)+0..7; D register v of lane
+// l is row 4*(l/16)+v, column l%16.
+__global__ void mfma16_layout(const float* A, const float* B, float* D)
+{
+    const int l = threadIdx.x;
+    f16x8     a, b;
+    for(int j = 0; j < 8; ++j)
+    {
+        a[j] = (_Float16)A[(l % 16) * 32 + 8 * (l / 16) + j];
+        b[j] = (_Float16)B[(8 * (l / 16) + j) * 16 + (l % 16)];
+    }
+    f32x4 c = {0};
+    c       = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    for(int v = 0; v < 4; ++v)
+    {
+        D[(4 * (l / 16) + v) * 16 + (l % 16)] = c[v];
+    }
+}
+
+// ---- 2. ds_read_b64_tr_b16 ----------------------------------------------------
+// LDS holds element value == element index; lane l reads from byte address
+// addr[l]; out[l*4+j] = element j of the lane's result.
+__global__ void tr16_dump(const int* addr, float* out)
+{
+    __shared__ _Float16 lds[2048];
+    for(int i = threadIdx.x; i < 2048; i += 64)
+    {
+        lds[i] = (_Float16)(float)i;
+    }
+    __syncthreads();
+    const int l = threadIdx.x;
+    auto* p = (__attribute__((address_space(3))) fp16x4_t*)((__attribute__((address_space(3))) char*)lds + addr[l]);
+    fp16x4_t t = __builtin_amdgcn_ds_read_tr16_b64_v4f16(p);
+    for(int j = 0; j < 4; ++j)
+    {
+        out[l * 4 + j] = (float)t[j];
+    }
+}
+
+// ---- 3. global_load_lds_dwordx4 ------------------------------------------------
+// Each lane fetches 16 bytes from src + goff[l] (elements); the whole LDS array is
+// then dumped so the placement of every lane's data can be read off.
+__global__ void lds_dma_dump(const _Float16* src, const int* goff, float* out, int lds_base_elems)
+{
+    __shared__ _Float16 lds[2048];
+    for(int i = threadIdx.x; i < 2048; i += 64)
+    {
+        lds[i] = (_Float16)-1.0f;
+    }
+    __syncthreads();
+    const int l = threadIdx.x;
+    __builtin_amdgcn_global_load_lds(
+        (const __attribute__((address_space(1))) void*)(src + goff[l]),
+        (__attribute__((address_space(3))) void*)(lds + lds_base_elems), 16, 0, 0);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    for(int i = threadIdx.x; i < 2048; i += 64)
+    {
+        out[i] = (float)lds[i];
+    }
+}
+
+// ---- 4. MFMA issue ceiling ------------------------------------------------------
+template<int CHAINS>
+__global__ void __launch_bounds__(256) mfma_peak(float* out, int iters)
+{
+    f32x16 acc[CHAINS];
+    for(int c = 0; c < CHAINS; ++c)
+    {
+        for(int v = 0; v < 16; ++v)
+        {
+            acc[c][v] = 0.0f;
+        }
+    }
+    f16x8 a, b;
+    for(int j = 0; j < 8; ++j)
+    {
+        a[j] = (_Float16)(float)(threadIdx.x % 3);
+        b[j] = (_Float16)(float)(threadIdx.x % 5);
+    }
+    for(int i = 0; i < iters; ++i)
+    {
+#pragma unroll
+        for(int c = 0; c < CHAINS; ++c)
+        {
+            acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[c], 0, 0, 0);
+        }
+    }
+    float s = 0.0f;
+    for(int c = 0; c < CHAINS; ++c)
+    {
+        for(int v = 0; v < 16; ++v)
+        {
+            s += acc[c][v];
+        }
+    }
+    if(s == 12345.678f)
+    {
+        out[0] = s;
+    }
+}
+
+// ---- 5. copy kernel (HBM reference point) --------------------------------------
+__global__ void __launch_bounds__(256) copy_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src, size_t n)
+{
+    for(size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    {
+        dst[i] = src[i];
+    }
+}
+
+static float time_ms(hipEvent_t a, hipEvent_t b)
+{
+    float ms = 0.0f;
+    CHECK(hipEventElapsedTime(&ms, a, b));
+    return ms;
+}
+
+template<class F>
+static bool check_product(const char* name, int M, int N, int K, F launch)
+{
+    std::vector<float> A(M * K), B(K * N), D(M * N, -1.0f), want(M * N, 0.0f);
+    for(int i = 0; i < M * K; ++i)
+        A[i] = (float)((i * 7 + 3) % 11 - 5);
+    for(int i = 0; i < K * N; ++i)
+        B[i] = (float)((i * 5 + 1) % 13 - 6);
+    for(int i = 0; i < M; ++i)
+        for(int j = 0; j < N; ++j)
+            for(int k = 0; k < K; ++k)
+                want[i * N + j] += A[i * K + k] * B[k * N + j];
+    float *dA, *dB, *dD;
+    CHECK(hipMalloc(&dA, A.size() * 4));
+    CHECK(hipMalloc(&dB, B.size() * 4));
+    CHECK(hipMalloc(&dD, D.size() * 4));
+    CHECK(hipMemcpy(dA, A.data(), A.size() * 4, hipMemcpyHostToDevice));
+    CHECK(hipMemcpy(dB, B.data(), B.size() * 4, hipMemcpyHostToDevice));
+    launch(dA, dB, dD);
+    CHECK(hipDeviceSynchronize());
+    CHECK(hipMemcpy(D.data(), dD, D.size() * 4, hipMemcpyDeviceToHost));
+    int bad = 0;
+    for(int i = 0; i < M * N; ++i)
+        bad += D[i] != want[i];
+    std::printf("%-28s %s (%d mismatches of %d)\n", name, bad ? "FAIL" : "PASS", bad, M * N);
+    CHECK(hipFree(dA));
+    CHECK(hipFree(dB));
+    CHECK(hipFree(dD));
+    return bad == 0;
+}
+
+int main(int argc, char** argv)
+{
+    bool   dump     = false;
+    size_t copy_mib = 0;
+    for(int i = 1; i < argc; ++i)
+    {
+        if(!std::strcmp(argv[i], "--dump"))
+            dump = true;
+        if(!std::strcmp(argv[i], "--copy") && i + 1 < argc)
+            copy_mib = std::strtoull(argv[++i], nullptr, 10);
+    }
+    hipDeviceProp_t prop;
+    CHECK(hipGetDeviceProperties(&prop, 0));
+    hipEvent_t e0, e1;
+    CHECK(hipEventCreate(&e0));
+    CHECK(hipEventCreate(&e1));
+
+    if(copy_mib)
+    {
+        const size_t bytes = copy_mib << 20, n = bytes / 16;
+        u32x4 *      s, *d;
+        CHECK(hipMalloc(&s, bytes));
+        CHECK(hipMalloc(&d, bytes));
+        CHECK(hipMemset(s, 1, bytes));
+        copy_kernel<<<4096, 256>>>(d, s, n);
+        CHECK(hipDeviceSynchronize());
+        std::printf("copy_kernel moved %zu MiB read + %zu MiB written\n", copy_mib, copy_mib);
+        return 0;
+    }
+
+    std::printf("device: %s, %d CUs, clock %d MHz, LDS/block %zu B\n", prop.gcnArchName,
+                prop.multiProcessorCount, prop.clockRate / 1000, prop.sharedMemPerBlock);
+
+    bool ok = true;
+    ok &= check_product("mfma_f32_32x32x16_f16 layout", 32, 32, 16, [](float* a, float* b, float* d) { mfma32_layout<false><<<1, 64>>>(a, b, d); });
+    ok &= check_product("mfma_f32_32x32x16_bf16 layout", 32, 32, 16, [](float* a, float* b, float* d) { mfma32_layout<true><<<1, 64>>>(a, b, d); });
+    ok &= check_product("mfma_f32_16x16x32_f16 layout", 16, 16, 32, [](float* a, float* b, float* d) { mfma16_layout<<<1, 64>>>(a, b, d); });
+
+    // ds_read_b64_tr_b16: lane l reads 8 bytes at l*8 (elements 4l..4l+3)
+    {
+        std::vector<int> addr(64);
+        for(int l = 0; l < 64; ++l)
+            addr[l] = l * 8;
+        int*   dAddr;
+        float* dOut;
+        CHECK(hipMalloc(&dAddr, 64 * 4));
+        CHECK(hipMalloc(&dOut, 256 * 4));
+        CHECK(hipMemcpy(dAddr, addr.data(), 64 * 4, hipMemcpyHostToDevice));
+        tr16_dump<<<1, 64>>>(dAddr, dOut);
+        CHECK(hipDeviceSynchronize());
+        std::vector<float> out(256);
+        CHECK(hipMemcpy(out.data(), dOut, 256 * 4, hipMemcpyDeviceToHost));
+        // Hypothesis: inside each block of 16 lanes the 16x4 elements form a matrix
+        // src[i][j] (i = lane in block, j = element); result lane i, element j is
+        // src[4*(i/4) + j][i%4] ... checked against the dump below.
+        int bad = 0;
+        for(int l = 0; l < 64; ++l)
+            for(int j = 0; j < 4; ++j)
+            {
+                const int blk = l / 16, i = l % 16;
+                const int src_lane = blk * 16 + 4 * j + i / 4; // hypothesis A
+                const int want     = src_lane * 4 + i % 4;
+                bad += (int)out[l * 4 + j] != want;
+            }
+        std::printf("%-28s %s (hypothesis: out[lane i][j] = in[lane 4j + i/4][i%%4])\n",
+                    "ds_read_b64_tr_b16", bad ? "FAIL" : "PASS");
+        if(dump || bad)
+        {
+            for(int l = 0; l < 64; ++l)
+                std::printf("  tr16 lane %2d: %4d %4d %4d %4d\n", l, (int)out[l * 4], (int)out[l * 4 + 1], (int)out[l * 4 + 2], (int)out[l * 4 + 3]);
+        }
+        ok &= bad == 0;
+    }
+
+    // global_load_lds_dwordx4: lane l fetches elements [8*(63-l), +8) (reversed so
+    // that lane order and address order differ); LDS base offset 64 elements.
+    {
+        std::vector<_Float16> src(1024);
+        for(int i = 0; i < 1024; ++i)
+            src[i] = (_Float16)(float)i;
+        std::vector<int> goff(64);
+        for(int l = 0; l < 64; ++l)
+            goff[l] = 8 * (63 - l);
+        _Float16* dSrc;
+        int*      dOff;
+        float*    dOut;
+        CHECK(hipMalloc(&dSrc, 2048));
+        CHECK(hipMalloc(&dOff, 256));
+        CHECK(hipMalloc(&dOut, 2048 * 4));
+        CHECK(hipMemcpy(dSrc, src.data(), 2048, hipMemcpyHostToDevice));
+        CHECK(hipMemcpy(dOff, goff.data(), 256, hipMemcpyHostToDevice));
+        lds_dma_dump<<<1, 64>>>(dSrc, dOff, dOut, 64);
+        CHECK(hipDeviceSynchronize());
+        std::vector<float> out(2048);
+        CHECK(hipMemcpy(out.data(), dOut, 2048 * 4, hipMemcpyDeviceToHost));
+        // Hypothesis: lane l's 16 bytes land at LDS base + l*16 bytes.
+        int bad = 0;
+        for(int l = 0; l < 64; ++l)
+            for(int j = 0; j < 8; ++j)
+                bad += (int)out[64 + l * 8 + j] != goff[l] + j;
+        for(int i = 0; i < 64; ++i)
+            bad += out[i] != -1.0f;
+        for(int i = 64 + 512; i < 2048; ++i)
+            bad += out[i] != -1.0f;
+        std::printf("%-28s %s (hypothesis: lane l -> LDS base + 16*l bytes)\n", "global_load_lds_dwordx4", bad ? "FAIL" : "PASS");
+        if(dump || bad)
+        {
+            for(int i = 0; i < 640; i += 8)
+                std::printf("  lds[%4d..]: %5d %5d %5d %5d %5d %5d %5d %5d\n", i, (int)out[i], (int)out[i + 1], (int)out[i + 2], (int)out[i + 3], (int)out[i + 4], (int)out[i + 5], (int)out[i + 6], (int)out[i + 7]);
+        }
+        ok &= bad == 0;
+    }
+
+    // MFMA ceiling: 4 waves per CU (one per SIMD) and 8 waves per CU
+    {
+        float* dOut;
+        CHECK(hipMalloc(&dOut, 4));
+        const int    iters = 20000;
+        const double flop_per_wave = 2.0 * 32 * 32 * 16 * 8 /*chains*/ * (double)iters;
+        for(int wg_per_cu = 1; wg_per_cu <= 2; ++wg_per_cu)
+        {
+            const int blocks = prop.multiProcessorCount * wg_per_cu;
+            mfma_peak<8><<<blocks, 256>>>(dOut, 100);
+            CHECK(hipDeviceSynchronize());
+            CHECK(hipEventRecord(e0));
+            mfma_peak<8><<<blocks, 256>>>(dOut, iters);
+            CHECK(hipEventRecord(e1));
+            CHECK(hipEventSynchronize(e1));
+            const float  ms = time_ms(e0, e1);
+            const double tf = flop_per_wave * 4 * blocks / (ms * 1e-3) / 1e12;
+            std::printf("mfma ceiling, %d waves/CU: %.1f TFLOP/s  (=> %.0f MHz at 1024 FLOP/clk/SIMD)\n", 4 * wg_per_cu, tf,
+                        tf * 1e12 / (prop.multiProcessorCount * 4.0 * 1024.0) / 1e6);
+        }
+    }
+
+    // HBM copy ceiling
+    {
+        const size_t bytes = size_t{1} << 30, n = bytes / 16;
+        u32x4 *      s, *d;
+        CHECK(hipMalloc(&s, bytes));
+        CHECK(hipMalloc(&d, bytes));
+        CHECK(hipMemset(s, 1, bytes));
+        copy_kernel<<<8192, 256>>>(d, s, n);
+        CHECK(hipDeviceSynchronize());
+        CHECK(hipEventRecord(e0));
+        for(int r = 0; r < 5; ++r)
+            copy_kernel<<<8192, 256>>>(d, s, n);
+        CHECK(hipEventRecord(e1));
+        CHECK(hipEventSynchronize(e1));
+        const float ms = time_ms(e0, e1) / 5;
+        std::printf("copy 1 GiB: %.3f ms -> %.2f TB/s (read+write)\n", ms, 2.0 * bytes / (ms * 1e-3) / 1e12);
+    }
+    std::printf("%s\n", ok ? "ALL LAYOUT CHECKS PASS" : "SOME LAYOUT CHECKS FAILED");
+    return ok ? 0 : 1;
+}

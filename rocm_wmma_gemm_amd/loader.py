@@ -1,0 +1,222 @@
+"""Python mirror of ``rocm_wmma_gemm::loader``.
+
+Reference interface: rocm_wmma_gemm/include/rocm_wmma_gemm/kernel_loader.hpp:51-182
+ - library name ``librocm_wmma_gemm_<arch>.so`` with ``<arch>`` taken from device 0's
+   architecture string cut at the first ':' (:74-91);
+ - search order: the configured library directory first, then the dynamic linker's
+   own path (:93-102);
+ - the four ``rocm_wmma_gemm_<Ctype>_<ABtype>`` symbols are resolved eagerly and a
+   missing library or symbol raises (:104-113) -- here ``GemmLibraryError``;
+ - ``gemm`` takes (C, A, B, M, N, K[, batch_count], stream) with the layouts in
+   C, A, B order and passes the ADDRESS of the stream handle (:138-154).
+
+There is no CPU fallback: if the library cannot be loaded every call fails.
+"""
+from __future__ import annotations
+
+import ctypes
+import enum
+import os
+import subprocess
+from dataclasses import dataclass
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_DEFAULT_LIB_DIR = os.path.join(_HERE, "lib")
+
+ENTRY_SUFFIXES = ("f16_f16", "f32_f16", "bf16_bf16", "f32_bf16")
+
+
+class GemmLibraryError(RuntimeError):
+    """Library or symbol could not be loaded (the C++ loader throws std::runtime_error)."""
+
+
+class m_layout(enum.IntEnum):
+    row_major = 0
+    col_major = 1
+
+
+row_major = m_layout.row_major
+col_major = m_layout.col_major
+
+
+class _VariantInfoC(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int) for n in (
+        "block_m", "block_n", "block_k", "warps_m", "warps_n", "warp_tile_m", "warp_tile_n",
+        "pipeline", "lds_bytes", "threads")]
+
+
+@dataclass(frozen=True)
+class VariantInfo:
+    index: int
+    block_m: int
+    block_n: int
+    block_k: int
+    warps_m: int
+    warps_n: int
+    warp_tile_m: int
+    warp_tile_n: int
+    pipeline: int
+    lds_bytes: int
+    threads: int
+
+
+def library_dir() -> str:
+    """Directory searched first (the C++ loader's ROCM_WMMA_GEMM_LIB_DIR define)."""
+    return os.environ.get("ROCM_WMMA_GEMM_LIB_DIR", _DEFAULT_LIB_DIR)
+
+
+def library_path(arch: str = "gfx950") -> str:
+    return os.path.join(library_dir(), f"librocm_wmma_gemm_{arch}.so")
+
+
+def build_library(jobs: int = 8, force: bool = False) -> str:
+    """Compile the HIP library in-tree (cross-compiles without a GPU)."""
+    cmd = ["make", "-C", os.path.join(_HERE, "csrc"), f"-j{jobs}", "all"]
+    if force:
+        cmd.insert(1, "-B")
+    subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL)
+    return os.path.join(_DEFAULT_LIB_DIR, "librocm_wmma_gemm_gfx950.so")
+
+
+def detect_arch() -> str:
+    import torch
+
+    if not torch.cuda.is_available():
+        raise GemmLibraryError("rocm_wmma_gemm::loader: hipGetDeviceProperties failed (no GPU)")
+    name = torch.cuda.get_device_properties(0).gcnArchName
+    return name.split(":", 1)[0]
+
+
+def _type_slot(c_dtype, ab_dtype) -> int:
+    import torch
+
+    table = {(torch.float16, torch.float16): 0, (torch.float32, torch.float16): 1,
+             (torch.bfloat16, torch.bfloat16): 2, (torch.float32, torch.bfloat16): 3}
+    try:
+        return table[(c_dtype, ab_dtype)]
+    except KeyError:
+        raise TypeError(f"Unsupported type pair for rocm_wmma_gemm loader: C={c_dtype}, A/B={ab_dtype}")
+
+
+class Loader:
+    """Opens the per-architecture library and forwards gemm calls through its C ABI."""
+
+    _ENTRY_ARGS = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+                   ctypes.c_size_t, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_int, ctypes.c_int,
+                   ctypes.c_int, ctypes.c_void_p]
+
+    def __init__(self, arch: str | None = None, lib_dir: str | None = None):
+        self.arch = arch if arch is not None else detect_arch()
+        name = f"librocm_wmma_gemm_{self.arch}.so"
+        first = os.path.join(lib_dir if lib_dir is not None else library_dir(), name)
+        errors = []
+        self._lib = None
+        for candidate in (first, name):
+            try:
+                self._lib = ctypes.CDLL(candidate, mode=os.RTLD_NOW | os.RTLD_LOCAL)
+                self.path = candidate
+                break
+            except OSError as e:
+                errors.append(str(e))
+        if self._lib is None:
+            raise GemmLibraryError(f"rocm_wmma_gemm::loader: could not open {name}: " + "; ".join(errors))
+        self._entries = []
+        for suffix in ENTRY_SUFFIXES:
+            sym = "rocm_wmma_gemm_" + suffix
+            try:
+                fn = getattr(self._lib, sym)
+            except AttributeError as e:
+                raise GemmLibraryError(f"rocm_wmma_gemm::loader: symbol not found: {sym} ({e})")
+            fn.restype = None
+            fn.argtypes = self._ENTRY_ARGS
+            self._entries.append(fn)
+        self._bind_extras()
+
+    # ------------------------------------------------------------------ extras
+    def _bind_extras(self):
+        L = self._lib
+        self._has_extras = hasattr(L, "rocm_wmma_gemm_run_variant")
+        if not self._has_extras:
+            return
+        L.rocm_wmma_gemm_arch.restype = ctypes.c_char_p
+        L.rocm_wmma_gemm_arch.argtypes = []
+        L.rocm_wmma_gemm_variant_count.restype = ctypes.c_int
+        L.rocm_wmma_gemm_variant_count.argtypes = []
+        L.rocm_wmma_gemm_variant_info_get.restype = ctypes.c_int
+        L.rocm_wmma_gemm_variant_info_get.argtypes = [ctypes.c_int, ctypes.POINTER(_VariantInfoC)]
+        L.rocm_wmma_gemm_select.restype = ctypes.c_int
+        L.rocm_wmma_gemm_select.argtypes = [ctypes.c_size_t] * 3 + [ctypes.c_int] * 4 + [
+            ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
+        L.rocm_wmma_gemm_run_variant.restype = ctypes.c_int
+        L.rocm_wmma_gemm_run_variant.argtypes = [ctypes.c_int] * 4 + self._ENTRY_ARGS
+
+    def library_arch(self) -> str:
+        return self._lib.rocm_wmma_gemm_arch().decode()
+
+    def variants(self) -> list[VariantInfo]:
+        out = []
+        for i in range(self._lib.rocm_wmma_gemm_variant_count()):
+            c = _VariantInfoC()
+            if self._lib.rocm_wmma_gemm_variant_info_get(i, ctypes.byref(c)) != 0:
+                raise GemmLibraryError(f"variant {i} not described by the library")
+            out.append(VariantInfo(i, *[getattr(c, n) for n, _ in _VariantInfoC._fields_]))
+        return out
+
+    def select(self, M: int, N: int, K: int, type_idx: int, layout_c: int, layout_a: int,
+               layout_b: int) -> tuple[int, int, int]:
+        """(variant, swizzle, split_k) the dispatcher picks for this problem."""
+        swz, sk = ctypes.c_int(0), ctypes.c_int(0)
+        v = self._lib.rocm_wmma_gemm_select(M, N, K, type_idx, int(layout_c), int(layout_a),
+                                            int(layout_b), ctypes.byref(swz), ctypes.byref(sk))
+        return v, swz.value, sk.value
+
+    # ------------------------------------------------------------------ gemm
+    @staticmethod
+    def _stream_handle(stream) -> int:
+        import torch
+
+        if stream is None:
+            stream = torch.cuda.current_stream()
+        return int(stream.cuda_stream) if hasattr(stream, "cuda_stream") else int(stream)
+
+    @staticmethod
+    def _check(C, A, B, M, N, K, batch):
+        for name, t, need in (("A", A, M * K * batch), ("B", B, K * N * batch), ("C", C, M * N * batch)):
+            if not t.is_cuda:
+                raise ValueError(f"{name} must be a device tensor")
+            if not t.is_contiguous():
+                raise ValueError(f"{name} must be densely packed")
+            if t.numel() < need:
+                raise ValueError(f"{name} holds {t.numel()} elements, the problem needs {need}")
+        if A.dtype != B.dtype:
+            raise TypeError("A and B must share an element type")
+
+    def gemm(self, C, A, B, M: int, N: int, K: int, layout_c=row_major, layout_a=row_major,
+             layout_b=row_major, batch_count: int = 1, stream=None) -> None:
+        """C = A * B, enqueued on ``stream`` (default: torch's current stream).
+
+        C, A, B are device tensors used as flat packed storage in the stated layouts."""
+        self._check(C, A, B, M, N, K, batch_count)
+        slot = _type_slot(C.dtype, A.dtype)
+        handle = ctypes.c_void_p(self._stream_handle(stream))
+        self._entries[slot](C.data_ptr(), A.data_ptr(), B.data_ptr(), M, N, K, batch_count,
+                            int(layout_c), int(layout_a), int(layout_b), ctypes.byref(handle))
+
+    def gemm_raw(self, slot: int, c_ptr: int, a_ptr: int, b_ptr: int, M: int, N: int, K: int,
+                 batch_count: int, layout_c: int, layout_a: int, layout_b: int,
+                 stream_handle: int) -> None:
+        """Direct C-ABI call with raw device addresses (no checks)."""
+        handle = ctypes.c_void_p(stream_handle)
+        self._entries[slot](c_ptr, a_ptr, b_ptr, M, N, K, batch_count, layout_c, layout_a,
+                            layout_b, ctypes.byref(handle))
+
+    def run_variant(self, variant: int, swizzle: int, split_k: int, C, A, B, M: int, N: int,
+                    K: int, layout_c=row_major, layout_a=row_major, layout_b=row_major,
+                    batch_count: int = 1, stream=None) -> int:
+        """Same as gemm() with the tile variant, swizzle and split-K forced (tuner hook)."""
+        self._check(C, A, B, M, N, K, batch_count)
+        slot = _type_slot(C.dtype, A.dtype)
+        handle = ctypes.c_void_p(self._stream_handle(stream))
+        return self._lib.rocm_wmma_gemm_run_variant(
+            slot, variant, swizzle, split_k, C.data_ptr(), A.data_ptr(), B.data_ptr(), M, N, K,
+            batch_count, int(layout_c), int(layout_a), int(layout_b), ctypes.byref(handle))

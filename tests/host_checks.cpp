@@ -1,0 +1,134 @@
+// Host-only checks of the pieces of the library that need no GPU: the tile map
+// (compiled here for the CPU) and the config selection functions.
+#include <cstdio>
+#include <cstring>
+#include <set>
+#include <utility>
+#include <vector>
+
+#include "config_select.hpp"
+#include "kernel/tile_map.hpp"
+
+using namespace rocm_wmma_gemm::device;
+using namespace rocm_wmma_gemm::host;
+
+static int fail(const char* what)
+{
+    std::printf("FAIL: %s\n", what);
+    return 1;
+}
+
+static int check_tilemap()
+{
+    const int groups[] = {1, 2, 4, 8, 16, 100};
+    for(int gm = 1; gm <= 40; ++gm)
+        for(int gn = 1; gn <= 40; ++gn)
+            for(int g : groups)
+            {
+                std::set<std::pair<int, int>> seen;
+                for(int wg = 0; wg < gm * gn; ++wg)
+                {
+                    tile_coord t = map_tile(wg, gm, gn, g);
+                    if(t.m < 0 || t.m >= gm || t.n < 0 || t.n >= gn)
+                        return fail("tile outside grid");
+                    if(!seen.insert({t.m, t.n}).second)
+                        return fail("tile visited twice");
+                }
+            }
+    // xcd_remap alone is a permutation for any total
+    for(int total = 1; total <= 300; ++total)
+    {
+        std::vector<int> hit(total, 0);
+        for(int wg = 0; wg < total; ++wg)
+        {
+            int id = xcd_remap(wg, total);
+            if(id < 0 || id >= total || hit[id]++)
+                return fail("xcd_remap not a permutation");
+        }
+    }
+    std::printf("tilemap ok\n");
+    return 0;
+}
+
+static int check_xcd()
+{
+    // 16 x 16 tiles, band height 4: the 32 workgroups of one XCD (ids = xcd mod 8)
+    // must cover a 4 x 8 rectangle: 4 distinct tile rows, 8 distinct tile columns.
+    for(int xcd = 0; xcd < 8; ++xcd)
+    {
+        std::set<int> rows, cols;
+        for(int wg = xcd; wg < 256; wg += 8)
+        {
+            tile_coord t = map_tile(wg, 16, 16, 4);
+            rows.insert(t.m);
+            cols.insert(t.n);
+        }
+        if(rows.size() != 4 || cols.size() != 8)
+            return fail("XCD footprint is not a 4x8 rectangle");
+    }
+    std::printf("xcd ok\n");
+    return 0;
+}
+
+static int check_select()
+{
+    // layouts: la, lb, lc ; plan {variant, swizzle, split_k}
+    const tuned_entry table[] = {
+        {1024, 1024, 1024, 0, 0, 1, 0, {1, 4, 1}},
+        {2048, 2048, 2048, 0, 0, 1, 0, {2, 8, 1}},
+        {65536, 2048, 2048, 0, 0, 1, 0, {3, 8, 1}},
+        {4096, 4096, 4096, 0, 0, 1, 0, {4, 16, 1}},
+        {4096, 4096, 4096, 1, 0, 1, 0, {5, 16, 1}},
+        {4096, 16384, 4096, 0, 0, 1, 0, {6, 16, 1}},
+        {512, 512, 512, 0, 1, 1, 1, {7, 4, 2}},
+    };
+    const size_t n = sizeof(table) / sizeof(table[0]);
+    auto pick = [&](size_t m, size_t nn, size_t k, int type_idx, int lc, int la, int lb) {
+        return select_plan_from(table, n, m, nn, k, type_idx, lc, la, lb).variant;
+    };
+    // exact hit, 16-bit group
+    if(pick(4096, 4096, 4096, 0, 0, 0, 1) != 4)
+        return fail("exact hit");
+    // exact hit in the fp32 group wins over group 0
+    if(pick(4096, 4096, 4096, 1, 0, 0, 1) != 5)
+        return fail("group-1 exact hit");
+    // fp32 group without its own exact entry falls back to group 0's exact entry
+    if(pick(2048, 2048, 2048, 3, 0, 0, 1) != 2)
+        return fail("group-1 -> group-0 exact fallback");
+    // nearest K first (2048), then nearest (M, N): (2048,2048) beats (65536,2048)
+    if(pick(8192, 4096, 2048, 0, 0, 0, 1) != 2)
+        return fail("closest: K first then MN");
+    // K = 4096 group: (4096,14336) is nearer to (4096,16384) than to (4096,4096)
+    if(pick(4096, 14336, 4096, 0, 0, 0, 1) != 6)
+        return fail("closest: MN distance");
+    // a genuine hit on the LAST entry is honoured (no sentinel collision)
+    if(pick(512, 512, 512, 0, 1, 1, 1) != 7)
+        return fail("hit on last entry");
+    // layout triple with no entries at all -> heuristic (variant 0 or 1)
+    launch_plan h = select_plan_from(table, n, 300, 300, 300, 0, 1, 0, 0);
+    if(h.variant != 0 || h.split_k != 1)
+        return fail("heuristic for uncovered layout");
+    // heuristic: few tiles and long K -> split-K
+    launch_plan lk = heuristic_plan(1024, 1024, 65536, 0);
+    if(lk.split_k < 2)
+        return fail("heuristic split-K on long K");
+    // empty table
+    launch_plan e = select_plan_from(nullptr, 0, 4096, 4096, 4096, 0, 0, 0, 1);
+    if(e.variant != 1)
+        return fail("heuristic on empty table");
+    std::printf("select ok\n");
+    return 0;
+}
+
+int main(int argc, char** argv)
+{
+    if(argc < 2)
+        return 2;
+    if(!std::strcmp(argv[1], "tilemap"))
+        return check_tilemap();
+    if(!std::strcmp(argv[1], "xcd"))
+        return check_xcd();
+    if(!std::strcmp(argv[1], "select"))
+        return check_select();
+    return 2;
+}

@@ -1,0 +1,234 @@
+"""GPU parity: the HIP library, called through its C ABI, against the CPU oracle.
+
+Tolerance (stated once, used everywhere): |gpu - cpu| <= 2*K*2^-24 * sum_k|a_ik*b_kj|
++ 1 ulp of the C element type -- the bound on the difference between two fp32
+summation orders of K products, plus output rounding.  Where the reference states
+its own criterion it is asserted as well: absolute 1e-4 for fp32 C on its 13 test
+shapes (test/gemm/test_float_accum.cpp:128-136), cosine similarity > 0.995 / 0.97
+for same-precision C (test/test.hpp:199-215).
+"""
+import numpy as np
+import pytest
+
+import oracle as O
+from gemm_harness import (LAYOUTS8, TYPE_PAIRS, check_against_oracle, checksum_check, layout_id,
+                          make_inputs, run_gpu, to_device, to_host, torch_dtype)
+
+pytestmark = pytest.mark.gpu
+
+# reference test/gemm/test_float_accum.cpp:161-224 and test_same_prec.cpp:145-213
+REFERENCE_SIZES = [(128, 128, 128), (128, 256, 128), (128, 128, 256), (256, 128, 128),
+                   (256, 256, 256), (320, 320, 320), (320, 512, 512), (512, 320, 320),
+                   (512, 512, 320), (512, 320, 512), (512, 512, 512), (1024, 256, 256),
+                   (256, 1024, 256)]
+
+
+@pytest.fixture(scope="module")
+def loader():
+    import torch
+
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    import rocm_wmma_gemm_amd as R
+
+    L = R.Loader()  # probes device 0, opens librocm_wmma_gemm_gfx950.so; raises if missing
+    assert L.arch == "gfx950" and L.library_arch() == "gfx950"
+    return L
+
+
+@pytest.mark.parametrize("type_name", list(TYPE_PAIRS))
+@pytest.mark.parametrize("lc,la,lb", LAYOUTS8, ids=[layout_id(*l) for l in LAYOUTS8])
+def test_reference_test_matrix(loader, type_name, lc, la, lb):
+    """The reference's own 13 shapes x 8 layouts x 4 type pairs, seeded as it seeds them."""
+    din, dout = TYPE_PAIRS[type_name]
+    for (M, N, K) in REFERENCE_SIZES:
+        A, B = make_inputs(M, N, K, la, lb, din)
+        gpu = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout)
+        _, g, c = check_against_oracle(gpu, A, B, M, N, K, lc, la, lb, din, dout)
+        if dout == O.F32:
+            assert np.abs(g - c).max() <= 1e-4, (M, N, K)
+        else:
+            cpu = O.gemm(A, B, M, N, K, lc, la, lb, din, dout)
+            cos = O.cosine_similarity(gpu, cpu, M, N, lc, dout)
+            assert cos > O.cosine_threshold(dout), (M, N, K, cos)
+
+
+@pytest.mark.parametrize("lc,la,lb", LAYOUTS8, ids=[layout_id(*l) for l in LAYOUTS8])
+def test_bit_exact_on_integer_inputs(loader, lc, la, lb):
+    """Small-integer operands make every partial sum exact, so any summation order
+    must give the oracle's bits exactly -- pins index maps and transpositions."""
+    rng = np.random.default_rng(42)
+    for din, dout in ((O.F16, O.F32), (O.BF16, O.BF16), (O.F16, O.F16)):
+        for (M, N, K) in ((96, 160, 64), (200, 72, 136), (257, 129, 65)):
+            Al = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+            Bl = rng.integers(-3, 4, size=(K, N)).astype(np.float32)
+            conv = O.f32_to_f16_bits if din == O.F16 else O.f32_to_bf16_bits
+            A = np.ascontiguousarray(conv(Al) if la == 0 else conv(Al).T).ravel()
+            B = np.ascontiguousarray(conv(Bl) if lb == 0 else conv(Bl).T).ravel()
+            gpu = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout)
+            cpu = O.gemm(A, B, M, N, K, lc, la, lb, din, dout)
+            assert np.array_equal(gpu, cpu), (din, dout, M, N, K)
+            if dout == O.F32:
+                assert np.array_equal(O.logical(gpu, M, N, lc), Al @ Bl)
+
+
+@pytest.mark.parametrize("type_name", list(TYPE_PAIRS))
+def test_identity_and_ones_closed_forms(loader, type_name):
+    din, dout = TYPE_PAIRS[type_name]
+    one = 0x3C00 if din == O.F16 else 0x3F80
+    # A = I  =>  C = B (exactly, after rounding B's values to the C type: they are already there)
+    M = N = K = 192
+    for (lc, la, lb) in LAYOUTS8:
+        A = np.zeros(M * K, dtype=np.uint16)
+        A[np.arange(M) * K + np.arange(M)] = one  # identity is symmetric: same in both layouts
+        B = O.init_matrix(K, N, lb, din, seed=5)
+        gpu = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout)
+        want = O.bits_to_f32(O.logical(B, K, N, lb), din)
+        assert np.array_equal(O.bits_to_f32(O.logical(gpu, M, N, lc), dout), want), (lc, la, lb)
+    # all ones => C = K (exactly representable: K <= 2048 in f16, <= 256 in bf16)
+    Kones = 2048 if dout != O.BF16 else 256
+    M, N = 64, 96
+    A = np.full(M * Kones, one, dtype=np.uint16)
+    B = np.full(Kones * N, one, dtype=np.uint16)
+    gpu = run_gpu(loader, A, B, M, N, Kones, 0, 0, 1, din, dout)
+    assert np.array_equal(O.bits_to_f32(gpu, dout), np.full(M * N, float(Kones), dtype=np.float32))
+
+
+EDGE_SHAPES = [(1, 1, 1), (1, 7, 3), (5, 1, 9), (17, 33, 5), (31, 63, 127), (129, 65, 31),
+               (64, 64, 8), (100, 36, 1), (255, 257, 259), (1000, 1000, 1000), (33, 4096, 40),
+               (3000, 17, 520)]
+
+
+@pytest.mark.parametrize("type_name", list(TYPE_PAIRS))
+@pytest.mark.parametrize("lc,la,lb", LAYOUTS8, ids=[layout_id(*l) for l in LAYOUTS8])
+def test_ragged_and_tiny_shapes(loader, type_name, lc, la, lb):
+    """Shapes the reference cannot run: M, N not tile multiples, K not a multiple of
+    16, odd leading dimensions (2-byte load path), single elements."""
+    din, dout = TYPE_PAIRS[type_name]
+    for (M, N, K) in EDGE_SHAPES:
+        A, B = make_inputs(M, N, K, la, lb, din, seed_a=3, seed_b=4, lo=-0.5, hi=0.5)
+        gpu = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout)
+        check_against_oracle(gpu, A, B, M, N, K, lc, la, lb, din, dout)
+
+
+def test_does_not_write_outside_c(loader):
+    """Guard rows/columns around C stay untouched for ragged shapes."""
+    import torch
+
+    M, N, K = 130, 70, 50
+    for (lc, la, lb) in LAYOUTS8:
+        A, B = make_inputs(M, N, K, la, lb, O.F16)
+        dA, dB = to_device(A, O.F16), to_device(B, O.F16)
+        pad = 4096
+        buf = torch.full((M * N + 2 * pad,), 7.0, dtype=torch.float32, device="cuda")
+        loader.gemm(buf[pad:pad + M * N], dA, dB, M, N, K, lc, la, lb)
+        torch.cuda.synchronize()
+        assert torch.all(buf[:pad] == 7.0) and torch.all(buf[pad + M * N:] == 7.0), (lc, la, lb)
+
+
+@pytest.mark.parametrize("type_name", ["f16_f16", "f32_bf16"])
+def test_batched_equals_per_slice_calls(loader, type_name):
+    """Batch b equals the unbatched call on slices at b*M*K, b*K*N, b*M*N
+    (reference kernel.hpp:165-167); bit-identical because the same kernel runs."""
+    import torch
+
+    din, dout = TYPE_PAIRS[type_name]
+    M, N, K, batch = 200, 136, 96, 5
+    for (lc, la, lb) in [(0, 0, 1), (1, 1, 0), (0, 1, 1), (1, 0, 0)]:
+        A = np.concatenate([O.init_matrix(M, K, la, din, seed=10 + b) for b in range(batch)])
+        B = np.concatenate([O.init_matrix(K, N, lb, din, seed=20 + b) for b in range(batch)])
+        got = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout, batch=batch)
+        for b in range(batch):
+            Ab, Bb = A[b * M * K:(b + 1) * M * K], B[b * K * N:(b + 1) * K * N]
+            one = run_gpu(loader, Ab, Bb, M, N, K, lc, la, lb, din, dout)
+            assert np.array_equal(got[b * M * N:(b + 1) * M * N], one), (lc, la, lb, b)
+            check_against_oracle(one, Ab, Bb, M, N, K, lc, la, lb, din, dout)
+
+
+def test_every_variant_and_split_k_agree_with_oracle(loader):
+    """Each compiled tile variant, forced through the tuner hook, with and without
+    split-K, on aligned and ragged shapes."""
+    for v in loader.variants():
+        for split_k in (1, 3):
+            for (M, N, K) in ((512, 512, 512), (300, 520, 264), (77, 91, 1003)):
+                for (lc, la, lb) in [(0, 0, 1), (0, 1, 0), (1, 0, 0), (1, 1, 1)]:
+                    for tname in ("f16_f16", "f32_bf16"):
+                        din, dout = TYPE_PAIRS[tname]
+                        A, B = make_inputs(M, N, K, la, lb, din, seed_a=7, seed_b=8)
+                        gpu = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout,
+                                      variant=(v.index, 4, split_k))
+                        check_against_oracle(gpu, A, B, M, N, K, lc, la, lb, din, dout)
+
+
+def test_degenerate_arguments(loader):
+    import torch
+
+    a = torch.ones(64, dtype=torch.float16, device="cuda")
+    c = torch.full((64,), 3.0, dtype=torch.float16, device="cuda")
+    loader.gemm(c, a, a, 0, 8, 8)          # M == 0: nothing happens
+    loader.gemm(c, a, a, 8, 8, 8, batch_count=0)
+    torch.cuda.synchronize()
+    assert torch.all(c == 3.0)
+    loader.gemm(c, a, a, 8, 8, 0)          # K == 0: empty sum, C = 0
+    torch.cuda.synchronize()
+    assert torch.all(c == 0.0)
+    c.fill_(3.0)
+    # layout codes outside {0,1}: silent no-op (reference src/gemm.cpp:243)
+    loader.gemm_raw(0, c.data_ptr(), a.data_ptr(), a.data_ptr(), 8, 8, 8, 1, 2, 0, 0,
+                    torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.all(c == 3.0)
+    with pytest.raises(TypeError):
+        loader.gemm(c, a.float(), a.float(), 8, 8, 8)
+
+
+def test_runs_on_the_callers_stream(loader):
+    import torch
+
+    M = N = K = 256
+    A, B = make_inputs(M, N, K, 0, 1, O.F16)
+    dA, dB = to_device(A, O.F16), to_device(B, O.F16)
+    dC = torch.zeros(M * N, dtype=torch.float16, device="cuda")
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        loader.gemm(dC, dA, dB, M, N, K, 0, 0, 1)  # picks up torch's current stream
+        ev = torch.cuda.Event()
+        ev.record(s)
+    ev.synchronize()
+    check_against_oracle(to_host(dC, O.F16), A, B, M, N, K, 0, 0, 1, O.F16, O.F16)
+
+
+# ---------------------------------------------------------------- full-size configurations
+def _full_size_case(loader, M, N, K, lc, la, lb, tname, row_bands, **gen):
+    din, dout = TYPE_PAIRS[tname]
+    A, B = make_inputs(M, N, K, la, lb, din, **gen)
+    gpu = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout)
+    checksum_check(gpu, A, B, M, N, K, lc, la, lb, din, dout)
+    for r0 in row_bands:
+        check_against_oracle(gpu, A, B, M, N, K, lc, la, lb, din, dout, rows=(r0, min(M, r0 + 32)))
+
+
+@pytest.mark.parametrize("lc,la,lb", LAYOUTS8, ids=[layout_id(*l) for l in LAYOUTS8])
+def test_half_half_4096_cubed_all_layouts(loader, lc, la, lb):
+    """fp16 -> fp16, M=N=K=4096, uniform[-1,1] seeded: every element through the
+    row/column checksums, three 32-row bands element by element."""
+    _full_size_case(loader, 4096, 4096, 4096, lc, la, lb, "f16_f16", (0, 2048 + 96, 4096 - 32))
+
+
+def test_float_bf16_8192_cubed(loader):
+    """bf16 -> fp32, M=N=K=8192, A row / B col / C row, normal(0,1) seeded."""
+    _full_size_case(loader, 8192, 8192, 8192, 0, 0, 1, "f32_bf16", (0, 4096 + 160, 8192 - 32),
+                    dist="normal", lo=0.0, hi=1.0)
+
+
+@pytest.mark.parametrize("M,N,K", [(4096, 5120, 5120), (8192, 4096, 2048), (4096, 14336, 4096),
+                                   (16, 8192, 8192), (64, 8192, 8192), (128, 8192, 8192)])
+def test_llm_projection_shapes(loader, M, N, K):
+    for (lc, la, lb) in [(0, 0, 1), (1, 0, 0)]:
+        _full_size_case(loader, M, N, K, lc, la, lb, "f32_f16", (0, max(0, M - 32)))
+
+
+@pytest.mark.parametrize("M,N,K", [(4095, 5121, 3001), (1000, 1000, 1000), (1024, 1024, 65536)])
+def test_edge_tile_and_long_k(loader, M, N, K):
+    for (lc, la, lb) in [(0, 0, 1), (1, 0, 0), (0, 1, 0), (1, 1, 1)]:
+        _full_size_case(loader, M, N, K, lc, la, lb, "bf16_bf16", (0, max(0, M - 32)),
+                        lo=-0.5, hi=0.5)

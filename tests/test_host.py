@@ -1,0 +1,150 @@
+"""CPU-only checks: the library loads, exports what include/rocm_wmma_gemm_c.h
+declares, the loader mirror fails the way the reference's loader does, the tile
+map is a bijection, and config selection follows the documented order."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def built_library():
+    import rocm_wmma_gemm_amd as R
+
+    path = R.library_path("gfx950")
+    if not os.path.exists(path):
+        R.build_library()
+    assert os.path.exists(path), "librocm_wmma_gemm_gfx950.so is not built"
+    return path
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "rocm_wmma_gemm_c.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rocm_wmma_gemm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_four_reference_entry_points():
+    names = declared_symbols()
+    for suffix in ("f16_f16", "f32_f16", "bf16_bf16", "f32_bf16"):
+        assert "rocm_wmma_gemm_" + suffix in names
+
+
+def test_library_exports_every_declared_symbol(built_library):
+    lib = ctypes.CDLL(built_library)
+    for name in declared_symbols():
+        assert hasattr(lib, name), f"{name} declared in include/rocm_wmma_gemm_c.h but not exported"
+    lib.rocm_wmma_gemm_arch.restype = ctypes.c_char_p
+    assert lib.rocm_wmma_gemm_arch() == b"gfx950"
+
+
+def test_loader_mirror_opens_named_arch_and_lists_variants(built_library):
+    import rocm_wmma_gemm_amd as R
+
+    L = R.Loader(arch="gfx950")
+    vs = L.variants()
+    assert len(vs) >= 2
+    for v in vs:
+        assert v.block_m == v.warps_m * v.warp_tile_m * 32
+        assert v.block_n == v.warps_n * v.warp_tile_n * 32
+        assert v.threads == 64 * v.warps_m * v.warps_n
+        assert v.lds_bytes <= 160 * 1024
+
+
+def test_loader_mirror_failure_modes(tmp_path, built_library):
+    import rocm_wmma_gemm_amd as R
+
+    # missing library: raises, naming the file (reference kernel_loader.hpp:104-108)
+    with pytest.raises(R.GemmLibraryError, match="librocm_wmma_gemm_gfx000.so"):
+        R.Loader(arch="gfx000")
+    # a library without the symbols: raises "symbol not found" (reference :62-71)
+    src = tmp_path / "empty.c"
+    src.write_text("int nothing_here(void) { return 0; }\n")
+    so = tmp_path / "librocm_wmma_gemm_gfx999.so"
+    subprocess.run(["gcc", "-shared", "-fPIC", str(src), "-o", str(so)], check=True)
+    with pytest.raises(R.GemmLibraryError, match="symbol not found: rocm_wmma_gemm_f16_f16"):
+        R.Loader(arch="gfx999", lib_dir=str(tmp_path))
+    # no GPU in the machine: probing device 0 fails like hipGetDeviceProperties would
+    import torch
+
+    if not torch.cuda.is_available():
+        with pytest.raises(R.GemmLibraryError):
+            R.Loader()
+
+
+def _host_tool(tmp_path_factory):
+    out = tmp_path_factory.mktemp("hosttool") / "host_checks"
+    src = os.path.join(ROOT, "tests", "host_checks.cpp")
+    csrc = os.path.join(ROOT, "rocm_wmma_gemm_amd", "csrc")
+    subprocess.run(["g++", "-O1", "-std=c++17", "-I", csrc, src,
+                    os.path.join(csrc, "config_select.cpp"), "-o", str(out)], check=True)
+    return str(out)
+
+
+@pytest.fixture(scope="module")
+def host_tool(tmp_path_factory, built_library):
+    return _host_tool(tmp_path_factory)
+
+
+def test_tile_map_is_a_bijection_for_every_grid(host_tool):
+    r = subprocess.run([host_tool, "tilemap"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+
+
+def test_xcd_groups_own_compact_rectangles(host_tool):
+    r = subprocess.run([host_tool, "xcd"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+
+
+def test_config_selection_order(host_tool):
+    r = subprocess.run([host_tool, "select"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+
+
+def test_generator_rejects_unknown_variant_and_roundtrips(tmp_path):
+    sys.path.insert(0, os.path.join(ROOT, "rocm_wmma_gemm_amd", "config"))
+    import generate_config as G
+
+    variants = G.read_variants(os.path.join(ROOT, "rocm_wmma_gemm_amd", "csrc", "variants.def"))
+    assert [v["index"] for v in variants] == list(range(len(variants)))
+    v0 = variants[0]
+    cfg = dict(warps_m=v0["warps_m"], warps_n=v0["warps_n"],
+               warp_tile_m=v0["block_m"] // v0["warps_m"] // 32,
+               warp_tile_n=v0["block_n"] // v0["warps_n"] // 32, swizzle=8, bits=128,
+               block_k=v0["block_k"], pipeline=v0["pipeline"])
+    assert G.variant_of(cfg, variants) == 0
+    with pytest.raises(ValueError):
+        G.variant_of(dict(cfg, warps_m=7), variants)
+    import json
+
+    doc = {"configurations": [
+        {"range": {"M": 64, "N": 64, "K": 64},
+         "layout": {"A": "row_major", "B": "col_major", "C": "row_major"}, "config": cfg},
+        {"range": {"M": 64, "N": 64, "K": 64},
+         "layout": {"A": "row_major", "B": "col_major", "C": "row_major"},
+         "config": dict(cfg, swizzle=16)}]}
+    p = tmp_path / "gemm_config_gfx950_f16.json"
+    p.write_text(json.dumps(doc))
+    rows = G.build_table(str(p), None, variants)
+    assert rows == [(64, 64, 64, 0, 0, 1, 0, 0, 16, 1)]  # later duplicate wins
+    text = G.render(rows, [str(p)])
+    assert "{64, 64, 64, 0, 0, 1, 0, {0, 16, 1}}" in text
+
+
+def test_shipped_json_matches_reference_schema():
+    import json
+
+    cfg_dir = os.path.join(ROOT, "rocm_wmma_gemm_amd", "config")
+    doc = json.load(open(os.path.join(cfg_dir, "gemm_config_gfx950_f16.json")))
+    assert doc["configurations"]
+    for conf in doc["configurations"]:
+        assert set(conf) == {"range", "layout", "config"}
+        assert set(conf["range"]) == {"M", "N", "K"}
+        assert set(conf["layout"]) == {"A", "B", "C"}
+        assert all(v in ("row_major", "col_major") for v in conf["layout"].values())
+        assert {"warps_m", "warps_n", "warp_tile_m", "warp_tile_n", "swizzle", "bits"} <= set(conf["config"])
