@@ -19,8 +19,11 @@ namespace rocm_wmma_gemm
 namespace host
 {
 
+// LDS per workgroup: the staged pipeline double-buffers one tile pair; the direct
+// pipeline keeps a ring of 2 (BLOCK_K 64) or 4 (BLOCK_K 32) tile pairs.
 #define RWG_VARIANT(IDX, BM, BN, BK, WM, WN, PIPE)                                         \
-    {BM, BN, BK, WM, WN, PIPE, 2 * (BM + BN) * (BK / 8) * 16, 64 * WM * WN},
+    {BM, BN, BK, WM, WN, PIPE, ((PIPE) == 1 && (BK) == 32 ? 4 : 2) * (BM + BN) * BK * 2,   \
+     64 * WM * WN},
 const variant_desc variant_table[num_variants] = {
 #include "variants.def"
 };
@@ -173,12 +176,47 @@ void zero_fill(void* C, size_t count, hipStream_t stream)
                                                                      static_cast<long long>(count));
 }
 
-template<class OutT>
-int launch(int type_idx, const launch_plan& plan, const kernel_problem& p, hipStream_t stream)
+// Variant that serves shapes a direct-to-LDS variant cannot take: the staged
+// variant with the same workgroup tile, else the small general tile.
+int staged_fallback(const variant_desc& v)
 {
+    for(int i = 0; i < num_variants; ++i)
+    {
+        const variant_desc& w = variant_table[i];
+        if(w.pipeline == 0 && w.block_m == v.block_m && w.block_n == v.block_n)
+        {
+            return i;
+        }
+    }
+    return 0;
+}
+
+// The direct pipeline addresses a tile with 32-bit byte offsets from its origin.
+bool direct_eligible(const kernel_problem& p, const variant_desc& v, int mode)
+{
+    if(mode != static_cast<int>(device::load_mode::vec_unguarded))
+    {
+        return false;
+    }
+    const unsigned long long a_ld = p.a_kmajor ? p.K : p.M, b_ld = p.b_kmajor ? p.K : p.N;
+    const unsigned long long a_span = (p.a_kmajor ? v.block_m : v.block_k) * a_ld * 2;
+    const unsigned long long b_span = (p.b_kmajor ? v.block_n : v.block_k) * b_ld * 2;
+    return a_span < (1ull << 32) && b_span < (1ull << 32);
+}
+
+template<class OutT>
+int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hipStream_t stream)
+{
+    launch_plan plan = plan_in;
     if(plan.variant < 0 || plan.variant >= num_variants)
     {
         return -1;
+    }
+    if(variant_table[plan.variant].pipeline == 1
+       && !direct_eligible(p, variant_table[plan.variant],
+                           pick_mode(p, variant_table[plan.variant], plan.split_k)))
+    {
+        plan.variant = staged_fallback(variant_table[plan.variant]);
     }
     const variant_desc& v = variant_table[plan.variant];
     if(p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull)

@@ -1,0 +1,497 @@
+// Direct-to-LDS MFMA GEMM kernel for gfx950: the fast path for shapes that are
+// whole multiples of the workgroup tile.
+//
+// Differences from the register-staged kernel (gemm_kernel.hpp):
+//   * operand tiles go global -> LDS with global_load_lds_dwordx4 (16 bytes per
+//     lane, no VGPR round trip); a wave-level load always fills 1024 contiguous
+//     LDS bytes in lane order, so each lane picks the GLOBAL address whose data
+//     belongs in its fixed LDS slot (the swizzle is applied on the global side);
+//   * an operand that is contiguous along M or N stays in that orientation in LDS
+//     and is transposed on the way to registers by ds_read_b64_tr_b16;
+//   * the LDS holds a ring of STAGES tiles; the loads of tile i+STAGES are issued as
+//     soon as tile i's stage has been drained, so a load has STAGES-1 tile times to
+//     land (measured: with one tile time the waves spend most of their cycles in
+//     s_waitcnt vmcnt, and a pure load loop runs 25 % faster with two tiles in
+//     flight than with one);
+//   * MFMA operand registers are double-buffered across the 16-wide K steps of a
+//     tile, and the one barrier per tile sits in front of the last K step, so its
+//     cost and the next tile's first LDS reads hide under that step's MFMAs.
+//
+// LDS layouts (one operand tile = ROWS x BK 16-bit elements):
+//   K-contiguous operand: row r = BK/8 chunks of 16 bytes; chunk c sits in slot
+//     c ^ swizzle(r) (see swizzle_of_row).  Wave-level load t fills rows
+//     t*512/BK .. (t+1)*512/BK - 1.
+//   M/N-contiguous operand: 1024-byte blocks of 4 k-rows x 128 rows-of-the-tile;
+//     block (kg, mh) at index kg * (ROWS/128) + mh; inside a block, k-row j holds
+//     16 chunks of 8 elements, chunk c in slot c ^ (4*j).  Wave-level load t fills
+//     block t.  ds_read_b64_tr_b16 then reads 4 k-rows x 32 elements per 32 lanes
+//     without bank conflicts (measured: 355 B/ns/CU vs 152 unswizzled).
+//
+// Same role as the staged kernel with respect to the reference (its gemm_impl,
+// prefetch_fragment, load_matrix: reference kernel/kernel.hpp:108-556,
+// kernel/load.hpp:348-966, kernel/fragment.hpp:191-274).
+#ifndef ROCM_WMMA_GEMM_DIRECT_KERNEL_HPP
+#define ROCM_WMMA_GEMM_DIRECT_KERNEL_HPP
+
+#include "gemm_kernel.hpp"
+
+namespace rocm_wmma_gemm
+{
+namespace device
+{
+
+typedef __fp16 fp16x4_raw __attribute__((__vector_size__(4 * sizeof(__fp16))));
+using lds_char_ptr = __attribute__((address_space(3))) char*;
+
+// One operand (A or B) of the direct pipeline.
+//   ROWS   tile extent along M (for A) or N (for B)
+//   WT     rows of the tile owned by one wave (wave tile extent)
+//   WAVES  waves in the workgroup (all of them cooperate on every tile load)
+template<bool KMAJOR, int ROWS, int BK, int WT, int WAVES>
+struct direct_operand
+{
+    static_assert(BK == 64 || BK == 32, "direct pipeline supports BK of 32 and 64");
+    static constexpr int CH         = BK / 8; // 16-byte chunks per K-contiguous row
+    static constexpr int KK         = BK / 16; // MFMA K steps per tile
+    static constexpr int TILE_BYTES = ROWS * BK * 2;
+    static constexpr int LOADS      = TILE_BYTES / 1024; // wave-level loads per tile
+    static_assert(LOADS % WAVES == 0, "tile loads must divide over the waves");
+    static constexpr int PER_WAVE = LOADS / WAVES;
+    static constexpr int T        = WT / 32; // 32-row MFMA operand tiles per wave
+    static constexpr int MH       = ROWS / 128; // 128-row halves (M/N-contiguous layout)
+    static constexpr int DS_PER_FRAGMENT = KMAJOR ? 1 : 2; // LDS reads behind one fragment()
+    static_assert(KMAJOR || ROWS % 128 == 0, "M/N-contiguous layout works in 128-row halves");
+    static_assert(T <= 4, "frag_off holds at most 4 entries");
+
+    // Per-lane element offset (from the tile origin at k = 0) of the 16 bytes this
+    // lane fetches in the wave's i-th load; advancing a tile adds BK * stride_k.
+    unsigned int lane_off[PER_WAVE];
+    // Per-lane LDS byte offsets for fragment reads (within an operand tile).
+    int frag_off[4]; // K-contiguous: one per K step; M/N-contiguous: one per operand tile i
+
+    __device__ __forceinline__ void init(int wave, int lane, long long ld, int wave_row0)
+    {
+#pragma unroll
+        for(int i = 0; i < PER_WAVE; ++i)
+        {
+            const int t = wave + i * WAVES; // wave-level load index within the tile
+            if constexpr(KMAJOR)
+            {
+                const int r    = (64 / CH) * t + lane / CH;
+                const int slot = lane % CH;
+                const int c    = slot ^ swizzle_of_row<CH>(r);
+                lane_off[i]    = (unsigned int)(r * ld + c * 8);
+            }
+            else
+            {
+                const int kg = t / MH, mh = t % MH;
+                const int j = lane / 16, cphys = lane % 16;
+                const int c = cphys ^ (4 * j);
+                lane_off[i] = (unsigned int)((long long)(kg * 4 + j) * ld + mh * 128 + c * 8);
+            }
+        }
+        if constexpr(KMAJOR)
+        {
+            const int lo = lane & 31, hi = lane >> 5;
+            const int row = wave_row0 + lo; // swizzle_of_row(row + 32*i) == swizzle_of_row(row)
+#pragma unroll
+            for(int kk = 0; kk < KK; ++kk)
+            {
+                frag_off[kk] = row * (16 * CH) + (((kk * 2 + hi) ^ swizzle_of_row<CH>(row)) * 16);
+            }
+        }
+        else
+        {
+            const int b = lane / 16, s = lane % 16, j = s / 4;
+#pragma unroll
+            for(int i = 0; i < T; ++i)
+            {
+                const int m  = wave_row0 + i * 32 + 16 * (b % 2) + (s % 4) * 4;
+                const int mh = m / 128, mm = m % 128;
+                const int c  = mm / 8;
+                // k group of K step 0, first half: kg = 2*(b/2); other (kk, h) add
+                // (kk*4 + h) * MH * 1024 bytes
+                frag_off[i] = ((2 * (b / 2)) * MH + mh) * 1024 + (j * 16 + (c ^ (4 * j))) * 16
+                              + (mm % 8) * 2;
+            }
+        }
+    }
+
+    // Enqueue this wave's share of one tile: global (tile_origin + lane_off) -> LDS.
+    template<class InT>
+    __device__ __forceinline__ void issue(const InT* tile_origin, lds_char_ptr lds_tile, int wave) const
+    {
+#pragma unroll
+        for(int i = 0; i < PER_WAVE; ++i)
+        {
+            const int t = wave + i * WAVES;
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(tile_origin + lane_off[i]),
+                (__attribute__((address_space(3))) void*)(lds_tile + t * 1024),
+                16,
+                0,
+                0);
+        }
+    }
+
+    // MFMA operand registers of operand tile i for K step kk.
+    __device__ __forceinline__ u32x4 fragment(lds_char_ptr lds_tile, int i, int kk) const
+    {
+        if constexpr(KMAJOR)
+        {
+            return *reinterpret_cast<__attribute__((address_space(3))) u32x4*>(
+                lds_tile + frag_off[kk] + i * (32 * 16 * CH));
+        }
+        else
+        {
+            auto* p0 = reinterpret_cast<__attribute__((address_space(3))) fp16x4_raw*>(
+                lds_tile + frag_off[i] + (kk * 4 + 0) * MH * 1024);
+            auto* p1 = reinterpret_cast<__attribute__((address_space(3))) fp16x4_raw*>(
+                lds_tile + frag_off[i] + (kk * 4 + 1) * MH * 1024);
+            const fp16x4_raw lo = __builtin_amdgcn_ds_read_tr16_b64_v4f16(p0);
+            const fp16x4_raw hi = __builtin_amdgcn_ds_read_tr16_b64_v4f16(p1);
+            const uint2      l2 = __builtin_bit_cast(uint2, lo);
+            const uint2      h2 = __builtin_bit_cast(uint2, hi);
+            return u32x4{l2.x, l2.y, h2.x, h2.y};
+        }
+    }
+};
+
+template<in_kind IN,
+         class OutT,
+         bool A_KMAJOR,
+         bool B_KMAJOR,
+         int  BM,
+         int  BN,
+         int  BK,
+         int  WAVES_M,
+         int  WAVES_N,
+         int  STAGES>
+struct direct_gemm
+{
+    using InT = typename std::conditional<IN == in_kind::f16, _Float16, __bf16>::type;
+
+    static constexpr int WAVES     = WAVES_M * WAVES_N;
+    static constexpr int THREADS   = 64 * WAVES;
+    static constexpr int WTM       = BM / WAVES_M;
+    static constexpr int WTN       = BN / WAVES_N;
+    static constexpr int TM        = WTM / 32;
+    static constexpr int TN        = WTN / 32;
+    static constexpr int KK        = BK / 16;
+    static constexpr int A_BYTES   = BM * BK * 2;
+    static constexpr int B_BYTES   = BN * BK * 2;
+    static constexpr int STAGE     = A_BYTES + B_BYTES;
+    static constexpr int LDS_BYTES = STAGES * STAGE;
+    static_assert(STAGES == 2 || STAGES == 4, "stage ring must be a power of two");
+    static_assert(KK % 2 == 0, "operand double-buffer parity must repeat every tile");
+    static_assert(LDS_BYTES <= 160 * 1024, "tile ring does not fit the 160 KB LDS");
+
+    using op_a = direct_operand<A_KMAJOR, BM, BK, WTM, WAVES>;
+    using op_b = direct_operand<B_KMAJOR, BN, BK, WTN, WAVES>;
+
+    static constexpr int VM_LOADS = op_a::PER_WAVE + op_b::PER_WAVE; // per wave, per tile
+    static constexpr int DS_READS = TM * op_a::DS_PER_FRAGMENT + TN * op_b::DS_PER_FRAGMENT;
+    static_assert((STAGES - 1) * VM_LOADS < 64, "vmcnt is a 6-bit counter");
+
+    // s_waitcnt immediate: lgkmcnt(0), expcnt untouched, vmcnt(n)
+    static constexpr int waitcnt_imm(int vmcnt)
+    {
+        return (vmcnt & 15) | (7 << 4) | (0 << 8) | ((vmcnt >> 4) << 14);
+    }
+
+    __device__ __forceinline__ static void load_fragments(const op_a& oa,
+                                                          const op_b& ob,
+                                                          lds_char_ptr stage,
+                                                          int          kk,
+                                                          u32x4 (&fa)[TM],
+                                                          u32x4 (&fb)[TN])
+    {
+#pragma unroll
+        for(int i = 0; i < TM; ++i)
+        {
+            fa[i] = oa.fragment(stage, i, kk);
+        }
+#pragma unroll
+        for(int j = 0; j < TN; ++j)
+        {
+            fb[j] = ob.fragment(stage + A_BYTES, j, kk);
+        }
+    }
+
+    __device__ __forceinline__ static void
+        multiply(const u32x4 (&fa)[TM], const u32x4 (&fb)[TN], f32x16 (&acc)[TM][TN])
+    {
+#pragma unroll
+        for(int i = 0; i < TM; ++i)
+        {
+#pragma unroll
+            for(int j = 0; j < TN; ++j)
+            {
+                acc[i][j] = mfma_32x32x16<IN>(fa[i], fb[j], acc[i][j]);
+            }
+        }
+    }
+
+    // Ask the scheduler for "one MFMA, then a slice of the memory instructions" so
+    // the LDS reads and global loads of a phase ride under its MFMAs instead of
+    // running ahead of or behind them.  LDS reads go under the first MFMAs, global
+    // -> LDS loads under the rest (they follow the reads in program order: the
+    // compiler keeps LDS reads and LDS-writing loads in source order).
+    template<int N_DS, int N_VMEM>
+    __device__ __forceinline__ static void interleave_hint()
+    {
+        constexpr int MFMAS    = TM * TN;
+        constexpr int DS_SLOTS = N_DS == 0 ? 0 : (N_VMEM > 0 ? MFMAS / 2 : MFMAS);
+        constexpr int DS_PER   = DS_SLOTS > 0 ? (N_DS + DS_SLOTS - 1) / DS_SLOTS : 1;
+        constexpr int VM_SLOTS = N_VMEM == 0 ? 0 : MFMAS - DS_SLOTS;
+        constexpr int VM_PER   = VM_SLOTS > 0 ? (N_VMEM + VM_SLOTS - 1) / VM_SLOTS : 1;
+        constexpr int REST     = MFMAS - DS_SLOTS - VM_SLOTS;
+#pragma unroll
+        for(int d = 0; d < DS_SLOTS; ++d)
+        {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // 1 MFMA
+            if(d * DS_PER < N_DS)
+            {
+                __builtin_amdgcn_sched_group_barrier(0x100, DS_PER, 0); // LDS reads
+            }
+        }
+        // loads are spread evenly: every VM_GAP-th MFMA slot carries VM_PER of them
+        constexpr int VM_GAP = (N_VMEM > 0 && VM_SLOTS >= 2 * N_VMEM) ? VM_SLOTS / N_VMEM : 1;
+#pragma unroll
+        for(int v = 0; v < VM_SLOTS; ++v)
+        {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if(v % VM_GAP == 0 && (v / VM_GAP) * VM_PER < N_VMEM)
+            {
+                __builtin_amdgcn_sched_group_barrier(0x020, VM_PER, 0); // global -> LDS
+            }
+        }
+        if constexpr(REST > 0)
+        {
+            __builtin_amdgcn_sched_group_barrier(0x008, REST, 0);
+        }
+    }
+
+    // One BK-wide tile out of stage (it % STAGES).  Every tile runs the same
+    // straight-line code, so that the scheduler can interleave it and no register
+    // shuffling is needed between variants of the step:
+    //   * (4-deep ring only) before the barrier, operand B of tile it+STAGES-1 is
+    //     enqueued; its operand A went out after the previous tile's barrier;
+    //   * after the barrier, tile it+STAGES is enqueued into the stage just drained
+    //     (2-deep ring: both operands; 4-deep ring: operand A only);
+    //   * K step 0 of tile it+1 is pre-read under the last K step's MFMAs.
+    // Past the end of K the caller keeps the source pointers on the last tile: the
+    // redundant loads land in stages nobody reads again, and the pre-read values are
+    // never used.  That keeps the number of loads in flight behind tile it+1 a
+    // compile-time constant, which s_waitcnt needs.
+    // Splitting a tile's loads over two phases keeps the rate at which the waves
+    // hand loads to the texture addresser (16 cycles per 1 KiB load, one addresser
+    // per CU) below what it drains, so MFMA issue does not stall behind them.
+    static constexpr bool SPLIT_ISSUE = STAGES == 4;
+    static constexpr int  WAIT_VM     = (STAGES - 2) * VM_LOADS;
+
+    __device__ __forceinline__ static void tile_step(const op_a&  oa,
+                                                     const op_b&  ob,
+                                                     lds_char_ptr lds,
+                                                     int          it,
+                                                     int          wave,
+                                                     const InT*   a_src,
+                                                     const InT*   b_src,
+                                                     u32x4 (&fa)[2][TM],
+                                                     u32x4 (&fb)[2][TN],
+                                                     f32x16 (&acc)[TM][TN])
+    {
+        lds_char_ptr cur = lds + (it & (STAGES - 1)) * STAGE;
+        lds_char_ptr nxt = lds + ((it + 1) & (STAGES - 1)) * STAGE;
+#pragma unroll
+        for(int kk = 0; kk + 1 < KK; ++kk)
+        {
+            const int use = kk & 1, fill = use ^ 1;
+            load_fragments(oa, ob, cur, kk + 1, fa[fill], fb[fill]);
+            if constexpr(SPLIT_ISSUE)
+            {
+                if(kk == 0)
+                {
+                    ob.issue(b_src, lds + ((it + STAGES - 1) & (STAGES - 1)) * STAGE + A_BYTES, wave);
+                }
+            }
+            multiply(fa[use], fb[use], acc);
+            if(SPLIT_ISSUE && kk == 0)
+            {
+                interleave_hint<DS_READS, op_b::PER_WAVE>();
+            }
+            else
+            {
+                interleave_hint<DS_READS, 0>();
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // Every read of `cur` has been issued; once they have landed and this wave's
+        // share of tile it+1 is in LDS, meet the other waves.  After the barrier
+        // `cur` may be overwritten and `nxt` may be read.
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(WAIT_VM));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        constexpr int use = (KK - 1) & 1, fill = use ^ 1;
+        load_fragments(oa, ob, nxt, 0, fa[fill], fb[fill]);
+        oa.issue(a_src, cur, wave);
+        if constexpr(!SPLIT_ISSUE)
+        {
+            ob.issue(b_src, cur + A_BYTES, wave);
+        }
+        multiply(fa[use], fb[use], acc);
+        interleave_hint<DS_READS, SPLIT_ISSUE ? op_a::PER_WAVE : VM_LOADS>();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    __device__ static void run(const gemm_args& args)
+    {
+        __shared__ __attribute__((aligned(1024))) char lds_raw[LDS_BYTES];
+        lds_char_ptr lds = (lds_char_ptr)lds_raw;
+
+        const int tid     = threadIdx.x;
+        const int lane    = tid & 63;
+        const int wave    = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int wave_m  = wave / WAVES_N;
+        const int wave_n  = wave % WAVES_N;
+        const int lane_lo = lane & 31;
+        const int lane_hi = lane >> 5;
+
+        const int tiles   = args.grid_m * args.grid_n;
+        const int slice   = blockIdx.x / tiles;
+        const int tile_id = blockIdx.x - slice * tiles;
+        const tile_coord t = map_tile(tile_id, args.grid_m, args.grid_n, args.group);
+        const int row0 = t.m * BM;
+        const int col0 = t.n * BN;
+
+        const int k_steps_total = args.K / BK;
+        const int steps_per     = (k_steps_total + args.k_slices - 1) / args.k_slices;
+        const int step_begin    = slice * steps_per;
+        int       step_end      = step_begin + steps_per;
+        if(step_end > k_steps_total)
+        {
+            step_end = k_steps_total;
+        }
+        const int nk = step_end - step_begin;
+
+        const long long batch = blockIdx.y;
+        const InT* A = static_cast<const InT*>(args.A) + batch * args.batch_stride_a;
+        const InT* B = static_cast<const InT*>(args.B) + batch * args.batch_stride_b;
+
+        const long long a_ld = A_KMAJOR ? args.K : args.M;
+        const long long b_ld = B_KMAJOR ? args.K : args.N;
+        const long long a_sr = A_KMAJOR ? a_ld : 1, a_sk = A_KMAJOR ? 1 : a_ld;
+        const long long b_sr = B_KMAJOR ? b_ld : 1, b_sk = B_KMAJOR ? 1 : b_ld;
+
+        op_a oa;
+        op_b ob;
+        oa.init(wave, lane, a_ld, wave_m * WTM);
+        ob.init(wave, lane, b_ld, wave_n * WTN);
+
+        // tile origins at this slice's first K step; advanced by BK per tile
+        const InT* a_src = A + row0 * a_sr + (long long)step_begin * BK * a_sk;
+        const InT* b_src = B + col0 * b_sr + (long long)step_begin * BK * b_sk;
+        const long long a_step = BK * a_sk, b_step = BK * b_sk;
+
+        f32x16 acc[TM][TN];
+#pragma unroll
+        for(int i = 0; i < TM; ++i)
+        {
+#pragma unroll
+            for(int j = 0; j < TN; ++j)
+            {
+#pragma unroll
+                for(int v = 0; v < 16; ++v)
+                {
+                    acc[i][j][v] = 0.0f;
+                }
+            }
+        }
+
+        if(nk > 0)
+        {
+            u32x4 fa[2][TM], fb[2][TN];
+
+            // Source pointers never move past the last tile of this K range.
+            const InT* a_last = a_src + (long long)(nk - 1) * a_step;
+            const InT* b_last = b_src + (long long)(nk - 1) * b_step;
+
+            // Prologue: fill the ring and wait for tile 0.  The 2-deep ring takes tiles
+            // 0 and 1 whole; the 4-deep ring takes tiles 0..2 whole and operand A of
+            // tile 3, whose operand B goes out during tile 0.
+#pragma unroll
+            for(int s = 0; s < STAGES; ++s)
+            {
+                oa.issue(a_src, lds + s * STAGE, wave);
+                a_src = a_src + a_step > a_last ? a_last : a_src + a_step;
+                if(!(SPLIT_ISSUE && s == STAGES - 1))
+                {
+                    ob.issue(b_src, lds + s * STAGE + A_BYTES, wave);
+                    b_src = b_src + b_step > b_last ? b_last : b_src + b_step;
+                }
+            }
+            __builtin_amdgcn_s_waitcnt(
+                waitcnt_imm((STAGES - 1) * VM_LOADS - (SPLIT_ISSUE ? op_b::PER_WAVE : 0)));
+            __builtin_amdgcn_s_barrier();
+            load_fragments(oa, ob, lds, 0, fa[0], fb[0]);
+
+            for(int it = 0; it < nk; ++it)
+            {
+                tile_step(oa, ob, lds, it, wave, a_src, b_src, fa, fb, acc);
+                a_src = a_src + a_step > a_last ? a_last : a_src + a_step;
+                b_src = b_src + b_step > b_last ? b_last : b_src + b_step;
+            }
+            // redundant tail loads may still be in flight
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+        }
+
+        // Epilogue: accumulator register v of a 32x32 tile is row
+        // 8*(v/4) + 4*(lane/32) + v%4, column lane%32.
+        if(args.k_slices == 1)
+        {
+            OutT* C = static_cast<OutT*>(args.C) + batch * args.batch_stride_c;
+#pragma unroll
+            for(int i = 0; i < TM; ++i)
+            {
+#pragma unroll
+                for(int j = 0; j < TN; ++j)
+                {
+                    const int col = col0 + wave_n * WTN + j * 32 + lane_lo;
+#pragma unroll
+                    for(int v = 0; v < 16; ++v)
+                    {
+                        const int row
+                            = row0 + wave_m * WTM + i * 32 + 8 * (v / 4) + 4 * lane_hi + (v % 4);
+                        C[(long long)row * args.N + col] = to_out<OutT>(acc[i][j][v]);
+                    }
+                }
+            }
+        }
+        else
+        {
+            float* P = args.partials
+                       + ((long long)batch * args.k_slices + slice) * (long long)args.M * args.N;
+#pragma unroll
+            for(int i = 0; i < TM; ++i)
+            {
+#pragma unroll
+                for(int j = 0; j < TN; ++j)
+                {
+                    const int col = col0 + wave_n * WTN + j * 32 + lane_lo;
+#pragma unroll
+                    for(int v = 0; v < 16; ++v)
+                    {
+                        const int row
+                            = row0 + wave_m * WTM + i * 32 + 8 * (v / 4) + 4 * lane_hi + (v % 4);
+                        P[(long long)row * args.N + col] = acc[i][j][v];
+                    }
+                }
+            }
+        }
+    }
+};
+
+} // namespace device
+} // namespace rocm_wmma_gemm
+
+#endif // ROCM_WMMA_GEMM_DIRECT_KERNEL_HPP

@@ -7,6 +7,7 @@
 #ifndef ROCM_WMMA_GEMM_KERNEL_TABLE_HPP
 #define ROCM_WMMA_GEMM_KERNEL_TABLE_HPP
 
+#include "kernel/direct_kernel.hpp"
 #include "kernel/gemm_kernel.hpp"
 
 namespace rocm_wmma_gemm

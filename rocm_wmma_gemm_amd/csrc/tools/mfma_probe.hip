@@ -178,6 +178,140 @@ __global__ void __launch_bounds__(256) copy_kernel(u32x4* __restrict__ dst, cons
     }
 }
 
+
+// ---- 6. LDS read throughput under a given per-lane address pattern ------------
+// Every lane issues `iters` x 8 reads at its own fixed byte address (plus a per-read
+// immediate offset); the time against the linear pattern shows bank conflicts.
+template<bool TR>
+__global__ void __launch_bounds__(512) lds_pattern(const int* lane_addr, float* out, int iters)
+{
+    __shared__ u32x4 lds[4096]; // 64 KiB
+    for(int i = threadIdx.x; i < 4096; i += blockDim.x)
+    {
+        lds[i] = u32x4{1u, 2u, 3u, 4u};
+    }
+    __syncthreads();
+    const unsigned addr = (unsigned)lane_addr[threadIdx.x & 63]
+                          + (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    for(int it = 0; it < iters; ++it)
+    {
+        if constexpr(TR)
+        {
+            uint2 v[16];
+            asm volatile(
+                "ds_read_b64_tr_b16 %0, %16\n ds_read_b64_tr_b16 %1, %16 offset:4096\n"
+                "ds_read_b64_tr_b16 %2, %16 offset:8192\n ds_read_b64_tr_b16 %3, %16 offset:12288\n"
+                "ds_read_b64_tr_b16 %4, %16 offset:16384\n ds_read_b64_tr_b16 %5, %16 offset:20480\n"
+                "ds_read_b64_tr_b16 %6, %16 offset:24576\n ds_read_b64_tr_b16 %7, %16 offset:28672\n"
+                "ds_read_b64_tr_b16 %8, %16 offset:32768\n ds_read_b64_tr_b16 %9, %16 offset:36864\n"
+                "ds_read_b64_tr_b16 %10, %16 offset:40960\n ds_read_b64_tr_b16 %11, %16 offset:45056\n"
+                "ds_read_b64_tr_b16 %12, %16 offset:49152\n ds_read_b64_tr_b16 %13, %16 offset:53248\n"
+                "ds_read_b64_tr_b16 %14, %16 offset:57344\n ds_read_b64_tr_b16 %15, %16 offset:61440\n"
+                "s_waitcnt lgkmcnt(0)"
+                : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]),
+                  "=&v"(v[6]), "=&v"(v[7]), "=&v"(v[8]), "=&v"(v[9]), "=&v"(v[10]), "=&v"(v[11]),
+                  "=&v"(v[12]), "=&v"(v[13]), "=&v"(v[14]), "=&v"(v[15])
+                : "v"(addr));
+            for(int i = 0; i < 16; ++i)
+                acc.x ^= v[i].x ^ v[i].y;
+        }
+        else
+        {
+            u32x4 v[16];
+            asm volatile(
+                "ds_read_b128 %0, %16\n ds_read_b128 %1, %16 offset:4096\n"
+                "ds_read_b128 %2, %16 offset:8192\n ds_read_b128 %3, %16 offset:12288\n"
+                "ds_read_b128 %4, %16 offset:16384\n ds_read_b128 %5, %16 offset:20480\n"
+                "ds_read_b128 %6, %16 offset:24576\n ds_read_b128 %7, %16 offset:28672\n"
+                "ds_read_b128 %8, %16 offset:32768\n ds_read_b128 %9, %16 offset:36864\n"
+                "ds_read_b128 %10, %16 offset:40960\n ds_read_b128 %11, %16 offset:45056\n"
+                "ds_read_b128 %12, %16 offset:49152\n ds_read_b128 %13, %16 offset:53248\n"
+                "ds_read_b128 %14, %16 offset:57344\n ds_read_b128 %15, %16 offset:61440\n"
+                "s_waitcnt lgkmcnt(0)"
+                : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]),
+                  "=&v"(v[6]), "=&v"(v[7]), "=&v"(v[8]), "=&v"(v[9]), "=&v"(v[10]), "=&v"(v[11]),
+                  "=&v"(v[12]), "=&v"(v[13]), "=&v"(v[14]), "=&v"(v[15])
+                : "v"(addr));
+            for(int i = 0; i < 16; ++i)
+                acc.x ^= v[i].x ^ v[i].w;
+        }
+    }
+    if(acc.x == 0x12345678u)
+    {
+        out[0] = 1.0f;
+    }
+}
+
+
+// ---- 7. LDS reads and global->LDS loads side by side ----------------------------
+// MODE 0: 16 ds_read_b128 per step; MODE 1: 4 global_load_lds_dwordx4 per step (from
+// a window of global memory small enough to stay in L2); MODE 2: both.  Shows what
+// the LDS sustains when the MFMA operand reads and the tile loads share it.
+template<int MODE, int DMA_BYTES>
+__global__ void __launch_bounds__(512) lds_dma_mix(const char* src, float* out, int iters)
+{
+    __shared__ __attribute__((aligned(1024))) char lds[131072];
+    for(int i = threadIdx.x; i < 131072 / 16; i += blockDim.x)
+    {
+        ((u32x4*)lds)[i] = u32x4{1u, 2u, 3u, 4u};
+    }
+    __syncthreads();
+    const int      lane  = threadIdx.x & 63;
+    const int      wave  = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned raddr = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds
+                           + (unsigned)(((lane % 32) * 128 + (((lane / 32) ^ ((lane >> 1) & 7)) * 16)));
+    // each workgroup walks its own 64 KiB window; each wave its own 1 KiB stripes
+    const char* base = src + (size_t)(blockIdx.x % 64) * 65536 + lane * DMA_BYTES;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    for(int it = 0; it < iters; ++it)
+    {
+        if constexpr(MODE != 0)
+        {
+#pragma unroll
+            for(int q = 0; q < 4; ++q)
+            {
+                const int stripe = ((it * 4 + q) * 8 + wave) & 63;
+                auto* g = (const __attribute__((address_space(1))) void*)(base + stripe * (64 * DMA_BYTES));
+                auto* l = (__attribute__((address_space(3))) void*)(lds + 65536 + stripe * 1024);
+                if constexpr(DMA_BYTES == 16)
+                    __builtin_amdgcn_global_load_lds(g, l, 16, 0, 0);
+                else
+                    __builtin_amdgcn_global_load_lds(g, l, 4, 0, 0);
+            }
+        }
+        if constexpr(MODE != 1)
+        {
+            u32x4 v[16];
+            asm volatile(
+                "ds_read_b128 %0, %16\n ds_read_b128 %1, %16 offset:4096\n"
+                "ds_read_b128 %2, %16 offset:8192\n ds_read_b128 %3, %16 offset:12288\n"
+                "ds_read_b128 %4, %16 offset:16384\n ds_read_b128 %5, %16 offset:20480\n"
+                "ds_read_b128 %6, %16 offset:24576\n ds_read_b128 %7, %16 offset:28672\n"
+                "ds_read_b128 %8, %16 offset:32768\n ds_read_b128 %9, %16 offset:36864\n"
+                "ds_read_b128 %10, %16 offset:40960\n ds_read_b128 %11, %16 offset:45056\n"
+                "ds_read_b128 %12, %16 offset:49152\n ds_read_b128 %13, %16 offset:53248\n"
+                "ds_read_b128 %14, %16 offset:57344\n ds_read_b128 %15, %16 offset:61440\n"
+                "s_waitcnt lgkmcnt(0)"
+                : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]),
+                  "=&v"(v[6]), "=&v"(v[7]), "=&v"(v[8]), "=&v"(v[9]), "=&v"(v[10]), "=&v"(v[11]),
+                  "=&v"(v[12]), "=&v"(v[13]), "=&v"(v[14]), "=&v"(v[15])
+                : "v"(raddr));
+            for(int i = 0; i < 16; ++i)
+                acc.x ^= v[i].x ^ v[i].w;
+        }
+        if constexpr(MODE != 0)
+        {
+            __builtin_amdgcn_s_waitcnt(0x0070 | 4 | (0 << 8)); // vmcnt(4): one step in flight
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    if(acc.x == 0x12345678u)
+    {
+        out[0] = 1.0f;
+    }
+}
+
 static float time_ms(hipEvent_t a, hipEvent_t b)
 {
     float ms = 0.0f;
@@ -349,6 +483,76 @@ int main(int argc, char** argv)
             std::printf("mfma ceiling, %d waves/CU: %.1f TFLOP/s  (=> %.0f MHz at 1024 FLOP/clk/SIMD)\n", 4 * wg_per_cu, tf,
                         tf * 1e12 / (prop.multiProcessorCount * 4.0 * 1024.0) / 1e6);
         }
+    }
+
+
+    // LDS read patterns (4 waves per CU, all CUs)
+    {
+        struct pat { const char* name; bool tr; int (*f)(int); };
+        static const pat pats[] = {
+            {"b128 linear lane*16", false, [](int l) { return l * 16; }},
+            {"b128 row*128, chunk=hi (no swizzle)", false, [](int l) { return (l % 32) * 128 + (l / 32) * 16; }},
+            {"b128 slot = c ^ (r&7)", false, [](int l) { int r = l % 32, c = l / 32; return r * 128 + ((c ^ (r & 7)) * 16); }},
+            {"b128 slot = c ^ ((r>>1)&7)", false, [](int l) { int r = l % 32, c = l / 32; return r * 128 + ((c ^ ((r >> 1) & 7)) * 16); }},
+            {"b128 slot = c ^ (r&7) ^ ((r>>3)&1)", false, [](int l) { int r = l % 32, c = l / 32; return r * 128 + ((c ^ (r & 7) ^ ((r >> 3) & 1)) * 16); }},
+            {"b128 row*64 (BK=32), slot = c ^ ((r>>1)&3)", false, [](int l) { int r = l % 32, c = l / 32; return r * 64 + ((c ^ ((r >> 1) & 3)) * 16); }},
+            {"tr64 linear lane*8", true, [](int l) { return l * 8; }},
+            {"tr64 [k][m] rows of 512 B, no swizzle", true, [](int l) { int b = l / 16, s = l % 16; return (8 * (b / 2) + s / 4) * 512 + (16 * (b % 2) + (s % 4) * 4) * 2; }},
+            {"tr64 4k x 128m blocks, chunk ^ 4j", true, [](int l) { int b = l / 16, s = l % 16, j = s / 4; int mm = 16 * (b % 2) + (s % 4) * 4; int c = mm / 8; return (2 * (b / 2)) * 2048 + (j * 16 + (c ^ (4 * j))) * 16 + (mm % 8) * 2; }},
+            {"tr64 4k x 128m blocks, no swizzle", true, [](int l) { int b = l / 16, s = l % 16, j = s / 4; int mm = 16 * (b % 2) + (s % 4) * 4; int c = mm / 8; return (2 * (b / 2)) * 2048 + (j * 16 + c) * 16 + (mm % 8) * 2; }},
+        };
+        int*   dAddr;
+        float* dOut;
+        CHECK(hipMalloc(&dAddr, 256));
+        CHECK(hipMalloc(&dOut, 4));
+        const int iters = 5000;
+        for(const pat& p : pats)
+        {
+            std::vector<int> addr(64);
+            for(int l = 0; l < 64; ++l)
+                addr[l] = p.f(l);
+            CHECK(hipMemcpy(dAddr, addr.data(), 256, hipMemcpyHostToDevice));
+            const int blocks = prop.multiProcessorCount;
+            for(int threads = 256; threads <= 512; threads *= 2)
+            {
+                if(p.tr) lds_pattern<true><<<blocks, threads>>>(dAddr, dOut, 100); else lds_pattern<false><<<blocks, threads>>>(dAddr, dOut, 100);
+                CHECK(hipDeviceSynchronize());
+                CHECK(hipEventRecord(e0));
+                if(p.tr) lds_pattern<true><<<blocks, threads>>>(dAddr, dOut, iters); else lds_pattern<false><<<blocks, threads>>>(dAddr, dOut, iters);
+                CHECK(hipEventRecord(e1));
+                CHECK(hipEventSynchronize(e1));
+                const float  ms    = time_ms(e0, e1);
+                const double bytes = (double)iters * 16 * threads * (p.tr ? 8 : 16); // per CU
+                std::printf("lds %-46s %d waves/CU %8.3f ms  %7.1f B/ns/CU\n", p.name, threads / 64, ms, bytes / (ms * 1e6));
+            }
+        }
+    }
+
+
+    // LDS reads vs global->LDS loads (8 waves per CU, all CUs, source resident in L2)
+    {
+        char*  dSrc;
+        float* dOut;
+        CHECK(hipMalloc(&dSrc, 64 * 65536 + 65536));
+        CHECK(hipMemset(dSrc, 1, 64 * 65536 + 65536));
+        CHECK(hipMalloc(&dOut, 4));
+        const int iters = 4000, blocks = prop.multiProcessorCount;
+        auto run = [&](const char* name, auto kernel, double rd_bytes, double dma_bytes) {
+            kernel<<<blocks, 512>>>(dSrc, dOut, 50);
+            CHECK(hipDeviceSynchronize());
+            CHECK(hipEventRecord(e0));
+            kernel<<<blocks, 512>>>(dSrc, dOut, iters);
+            CHECK(hipEventRecord(e1));
+            CHECK(hipEventSynchronize(e1));
+            const float ms = time_ms(e0, e1);
+            std::printf("mix %-34s %8.3f ms  reads %7.1f B/ns/CU  loads %7.1f B/ns/CU\n", name, ms,
+                        rd_bytes * iters / (ms * 1e6), dma_bytes * iters / (ms * 1e6));
+        };
+        run("ds_read_b128 only", lds_dma_mix<0, 16>, 8.0 * 16 * 1024, 0.0);
+        run("global_load_lds_dwordx4 only", lds_dma_mix<1, 16>, 0.0, 8.0 * 4 * 1024);
+        run("both (dwordx4)", lds_dma_mix<2, 16>, 8.0 * 16 * 1024, 8.0 * 4 * 1024);
+        run("global_load_lds_dword only", lds_dma_mix<1, 4>, 0.0, 8.0 * 4 * 256);
+        run("both (dword)", lds_dma_mix<2, 4>, 8.0 * 16 * 1024, 8.0 * 4 * 256);
     }
 
     // HBM copy ceiling
