@@ -197,6 +197,33 @@ def test_runs_on_the_callers_stream(loader):
     check_against_oracle(to_host(dC, O.F16), A, B, M, N, K, 0, 0, 1, O.F16, O.F16)
 
 
+def test_cpp_client_through_this_repositorys_loader_header():
+    """A C++ client of rocm_wmma_gemm::loader (all type pairs, all layouts, batched),
+    bit-exact against a host loop on inputs whose sums are exact."""
+    import os
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(__file__), "..", "rocm_wmma_gemm_amd", "lib", "dropin_check")
+    assert os.path.exists(exe), "build the tools first (make -C rocm_wmma_gemm_amd/csrc)"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and "DROP-IN CHECK PASSED" in r.stdout, r.stdout + r.stderr
+
+
+def test_cpp_client_through_the_references_own_loader_header():
+    """The same client compiled against the REFERENCE's kernel_loader.hpp (built where the
+    reference tree is present, see oracle/Makefile target `ref`): the reference's loader
+    finds librocm_wmma_gemm_gfx950.so by architecture name and drives it unchanged."""
+    import os
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(__file__), "..", "oracle", "_ref",
+                       "dropin_check_reference_loader")
+    if not os.path.exists(exe):
+        pytest.skip("oracle/_ref/dropin_check_reference_loader was not built (no reference tree)")
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and "DROP-IN CHECK PASSED" in r.stdout, r.stdout + r.stderr
+
+
 # ---------------------------------------------------------------- full-size configurations
 def _full_size_case(loader, M, N, K, lc, la, lb, tname, row_bands, **gen):
     din, dout = TYPE_PAIRS[tname]
