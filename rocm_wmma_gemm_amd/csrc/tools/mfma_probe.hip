@@ -312,6 +312,99 @@ __global__ void __launch_bounds__(512) lds_dma_mix(const char* src, float* out, 
     }
 }
 
+
+// ---- 8. MFMA throughput with a memory stream running beside it ---------------------
+// Each wave runs 16 independent MFMAs per step on pseudo-random operands and, beside
+// them, LOADS memory operations of one kind:
+//   KIND 0 none, 1 global_load_lds_dwordx4 (L2-resident source), 2 global_load_dwordx4
+//   into VGPRs, 3 ds_read_b128, 4 global_load_lds from a large (HBM-resident) source
+template<int KIND, int LOADS>
+__global__ void __launch_bounds__(256) mfma_with_stream(const char* src, size_t src_bytes, float* out, int iters)
+{
+    __shared__ __attribute__((aligned(1024))) char lds[65536];
+    for(int i = threadIdx.x; i < 65536 / 16; i += blockDim.x)
+        ((u32x4*)lds)[i] = u32x4{(unsigned)i * 2654435761u, 0x3c003c00u ^ (unsigned)i, 0xbc00u * (unsigned)i, 0x12345u * (unsigned)i};
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    f32x16    acc[16];
+    for(int c = 0; c < 16; ++c)
+        for(int v = 0; v < 16; ++v)
+            acc[c][v] = 0.0f;
+    u32x4 fa[4], fb[4];
+    for(int i = 0; i < 4; ++i)
+    {
+        fa[i] = ((u32x4*)lds)[(lane * 4 + i) & 4095];
+        fb[i] = ((u32x4*)lds)[(lane * 4 + i + 1024) & 4095];
+    }
+    const unsigned long long clk0 = __builtin_amdgcn_s_memtime();
+    const unsigned long long rt0  = __builtin_amdgcn_s_memrealtime();
+    const size_t window = KIND == 4 ? src_bytes : (size_t)(4 << 20);
+    size_t       pos    = ((size_t)blockIdx.x * 65536 + (size_t)wave * 16384) % window;
+    u32x4        sink   = {0u, 0u, 0u, 0u};
+    const unsigned raddr = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds + lane * 16;
+    for(int it = 0; it < iters; ++it)
+    {
+#pragma unroll
+        for(int q = 0; q < LOADS; ++q)
+        {
+            const char* g = src + pos + q * 1024 + lane * 16;
+            if constexpr(KIND == 6)
+            {
+                // buffer form: 128-bit resource in SGPRs, 32-bit per-lane offset, scalar offset
+                auto rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, 0x7fffffff, 0x00020000);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc,
+                                                         (__attribute__((address_space(3))) void*)(lds + 32768 + ((wave * LOADS + q) & 31) * 1024),
+                                                         16, lane * 16, (int)(pos + q * 1024), 0, 0);
+            }
+            else if constexpr(KIND == 5)
+            {
+                // uniform 64-bit base in SGPRs + 32-bit per-lane byte offset
+                const char* ubase = src + pos + q * 1024;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ubase + (unsigned)(lane * 16)),
+                                                 (__attribute__((address_space(3))) void*)(lds + 32768 + ((wave * LOADS + q) & 31) * 1024),
+                                                 16, 0, 0);
+            }
+            else if constexpr(KIND == 1 || KIND == 4)
+            {
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                                 (__attribute__((address_space(3))) void*)(lds + 32768 + ((wave * LOADS + q) & 31) * 1024),
+                                                 16, 0, 0);
+            }
+            else if constexpr(KIND == 2)
+            {
+                u32x4 v = __builtin_nontemporal_load((const u32x4*)g);
+                sink ^= v;
+            }
+            else if constexpr(KIND == 3)
+            {
+                u32x4 v;
+                asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(raddr + q * 1024));
+                sink ^= v;
+            }
+        }
+        pos = (pos + 256 * 1024) % window;
+#pragma unroll
+        for(int c = 0; c < 16; ++c)
+            acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fa[c / 4]), __builtin_bit_cast(f16x8, fb[c % 4]), acc[c], 0, 0, 0);
+        if constexpr(KIND == 1 || KIND == 4 || KIND == 5 || KIND == 6)
+            __builtin_amdgcn_s_waitcnt(0x0070 | (3 * LOADS > 15 ? 15 : 3 * LOADS)); // keep ~3 steps in flight
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    float s = 0.0f;
+    for(int c = 0; c < 16; ++c)
+        for(int v = 0; v < 16; ++v)
+            s += acc[c][v];
+    if(s == 12345.678f || sink.x == 0x7654321u)
+        out[0] = s;
+    if(blockIdx.x == 0 && threadIdx.x == 0)
+    {
+        // shader-clock ticks and constant 100 MHz ticks over the loop -> average core clock
+        out[1] = (float)(__builtin_amdgcn_s_memtime() - clk0);
+        out[2] = (float)(__builtin_amdgcn_s_memrealtime() - rt0);
+    }
+}
+
 static float time_ms(hipEvent_t a, hipEvent_t b)
 {
     float ms = 0.0f;
@@ -553,6 +646,42 @@ int main(int argc, char** argv)
         run("both (dwordx4)", lds_dma_mix<2, 16>, 8.0 * 16 * 1024, 8.0 * 4 * 1024);
         run("global_load_lds_dword only", lds_dma_mix<1, 4>, 0.0, 8.0 * 4 * 256);
         run("both (dword)", lds_dma_mix<2, 4>, 8.0 * 16 * 1024, 8.0 * 4 * 256);
+    }
+
+
+    // MFMA beside a memory stream (4 waves per CU, all CUs)
+    {
+        const size_t big = size_t{1} << 30;
+        char*        dSrc;
+        float*       dOut;
+        CHECK(hipMalloc(&dSrc, big + (1 << 20)));
+        CHECK(hipMemset(dSrc, 0x3c, big + (1 << 20)));
+        CHECK(hipMalloc(&dOut, 16));
+        const int iters = 4000, blocks = prop.multiProcessorCount;
+        auto run = [&](const char* name, auto kernel, int loads) {
+            kernel<<<blocks, 256>>>(dSrc, big, dOut, 50);
+            CHECK(hipDeviceSynchronize());
+            CHECK(hipEventRecord(e0));
+            kernel<<<blocks, 256>>>(dSrc, big, dOut, iters);
+            CHECK(hipEventRecord(e1));
+            CHECK(hipEventSynchronize(e1));
+            const float  ms = time_ms(e0, e1);
+            const double tf = 2.0 * 32 * 32 * 16 * 16 * (double)iters * 4 * blocks / (ms * 1e-3) / 1e12;
+            float clk[3];
+            CHECK(hipMemcpy(clk, dOut, 12, hipMemcpyDeviceToHost));
+            const double mhz = clk[2] > 0 ? clk[1] / clk[2] * 100.0 : 0.0;
+            std::printf("mfma+%-44s %8.3f ms %8.1f TFLOP/s  stream %6.1f B/ns/CU  core clock %5.0f MHz  MFMA busy %4.1f %%\n", name, ms, tf,
+                        loads * 1024.0 * 4 * iters / (ms * 1e6), mhz,
+                        mhz > 0 ? 100.0 * tf * 1e12 / (prop.multiProcessorCount * 4.0 * 1024.0 * mhz * 1e6) : 0.0);
+        };
+        run("nothing (random operands)", mfma_with_stream<0, 0>, 0);
+        run("global_load_lds x4 per 16 MFMA, L2-resident", mfma_with_stream<1, 4>, 4);
+        run("global_load_lds x2 per 16 MFMA, L2-resident", mfma_with_stream<1, 2>, 2);
+        run("global_load_lds x4, SGPR base + 32-bit offset", mfma_with_stream<5, 4>, 4);
+        run("buffer_load ... lds x4 (32-bit voffset + soffset)", mfma_with_stream<6, 4>, 4);
+        run("global_load_lds x4 per 16 MFMA, 1 GiB source", mfma_with_stream<4, 4>, 4);
+        run("global_load_dwordx4 x4 per 16 MFMA, L2-resident", mfma_with_stream<2, 4>, 4);
+        run("ds_read_b128 x8 per 16 MFMA", mfma_with_stream<3, 8>, 8);
     }
 
     // HBM copy ceiling
