@@ -22,7 +22,7 @@ namespace host
 // LDS per workgroup: the staged pipeline double-buffers one tile pair; the direct
 // pipeline keeps a ring of 2 (BLOCK_K 64) or 4 (BLOCK_K 32) tile pairs.
 #define RWG_VARIANT(IDX, BM, BN, BK, WM, WN, PIPE)                                         \
-    {BM, BN, BK, WM, WN, PIPE, ((PIPE) == 1 && (BK) == 32 ? 4 : 2) * (BM + BN) * BK * 2,   \
+    {BM, BN, BK, WM, WN, PIPE, ((PIPE) != 0 && (BK) == 32 ? 4 : 2) * (BM + BN) * BK * 2,   \
      64 * WM * WN},
 const variant_desc variant_table[num_variants] = {
 #include "variants.def"
@@ -212,7 +212,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
     {
         return -1;
     }
-    if(variant_table[plan.variant].pipeline == 1
+    if(variant_table[plan.variant].pipeline != 0
        && !direct_eligible(p, variant_table[plan.variant],
                            pick_mode(p, variant_table[plan.variant], plan.split_k)))
     {

@@ -226,12 +226,6 @@ struct direct_gemm
     __device__ __forceinline__ static void
         multiply(const u32x4 (&fa)[TM], const u32x4 (&fb)[TN], f32x16 (&acc)[TM][TN])
     {
-#ifdef RWG_EXP_BURST
-        __builtin_amdgcn_sched_barrier(0);
-#endif
-#ifdef RWG_EXP_PRIO
-        __builtin_amdgcn_s_setprio(3);
-#endif
 #pragma unroll
         for(int i = 0; i < TM; ++i)
         {
@@ -241,9 +235,6 @@ struct direct_gemm
                 acc[i][j] = mfma_32x32x16<IN>(fa[i], fb[j], acc[i][j]);
             }
         }
-#ifdef RWG_EXP_PRIO
-        __builtin_amdgcn_s_setprio(0);
-#endif
     }
 
     // Ask the scheduler for "one MFMA, then a slice of the memory instructions" so
@@ -254,9 +245,6 @@ struct direct_gemm
     template<int N_DS, int N_VMEM>
     __device__ __forceinline__ static void interleave_hint()
     {
-#ifdef RWG_EXP_BURST
-        return;
-#endif
         constexpr int MFMAS    = TM * TN;
         constexpr int DS_SLOTS = N_DS == 0 ? 0 : (N_VMEM > 0 ? MFMAS / 2 : MFMAS);
         constexpr int DS_PER   = DS_SLOTS > 0 ? (N_DS + DS_SLOTS - 1) / DS_SLOTS : 1;
@@ -324,9 +312,7 @@ struct direct_gemm
         for(int kk = 0; kk + 1 < KK; ++kk)
         {
             const int use = kk & 1, fill = use ^ 1;
-#ifndef RWG_EXP_NOLDS
             load_fragments(oa, ob, cur, kk + 1, fa[fill], fb[fill]);
-#endif
             if constexpr(SPLIT_ISSUE)
             {
                 if(kk == 0)
@@ -352,11 +338,7 @@ struct direct_gemm
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         constexpr int use = (KK - 1) & 1, fill = use ^ 1;
-#ifndef RWG_EXP_NOLDS
         load_fragments(oa, ob, nxt, 0, fa[fill], fb[fill]);
-#else
-        asm volatile("" : "+v"(fa[0][0]), "+v"(fb[0][0]), "+v"(fa[1][0]), "+v"(fb[1][0]));
-#endif
         oa.issue(a_src, cur, wave);
         if constexpr(!SPLIT_ISSUE)
         {
@@ -457,9 +439,6 @@ struct direct_gemm
                 waitcnt_imm((STAGES - 1) * VM_LOADS - (SPLIT_ISSUE ? op_b::PER_WAVE : 0)));
             __builtin_amdgcn_s_barrier();
             load_fragments(oa, ob, lds, 0, fa[0], fb[0]);
-#ifdef RWG_EXP_NOLDS
-            load_fragments(oa, ob, lds, 1, fa[1], fb[1]);
-#endif
 
             for(int it = 0; it < nk; ++it)
             {

@@ -23,17 +23,23 @@ using out_t = std::conditional<RWG_TYPE == 0, _Float16,
 template<int BM, int BN, int BK, int WM, int WN, int PIPE, device::load_mode MODE>
 constexpr kernel_fn entry()
 {
-    static_assert(PIPE == 0 || PIPE == 1, "unknown pipeline");
+    static_assert(PIPE == 0 || PIPE == 1 || PIPE == 2, "unknown pipeline");
     if constexpr(PIPE == 0)
     {
         return &device::gemm_entry<
             device::staged_gemm<kIn, out_t, RWG_AK != 0, RWG_BK != 0, BM, BN, BK, WM, WN, MODE>>;
     }
-    else if constexpr(MODE == device::load_mode::vec_unguarded)
+    else if constexpr(MODE == device::load_mode::vec_unguarded && PIPE == 1)
     {
         return &device::gemm_entry<
             device::direct_gemm<kIn, out_t, RWG_AK != 0, RWG_BK != 0, BM, BN, BK, WM, WN,
                                 (BK == 64 ? 2 : 4)>>;
+    }
+    else if constexpr(MODE == device::load_mode::vec_unguarded && PIPE == 2)
+    {
+        return &device::gemm_entry<
+            device::pingpong_gemm<kIn, out_t, RWG_AK != 0, RWG_BK != 0, BM, BN, BK, WM, WN,
+                                  (BK == 64 ? 2 : 4)>>;
     }
     else
     {

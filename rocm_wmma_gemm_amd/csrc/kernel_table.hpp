@@ -8,6 +8,7 @@
 #define ROCM_WMMA_GEMM_KERNEL_TABLE_HPP
 
 #include "kernel/direct_kernel.hpp"
+#include "kernel/pingpong_kernel.hpp"
 #include "kernel/gemm_kernel.hpp"
 
 namespace rocm_wmma_gemm

@@ -405,6 +405,70 @@ __global__ void __launch_bounds__(256) mfma_with_stream(const char* src, size_t 
     }
 }
 
+
+// ---- 9. MFMA shape vs sustained rate on pseudo-random operands ----------------------
+// SHAPE 0: v_mfma_f32_32x32x16_f16 (16 accumulator registers per instruction),
+// SHAPE 1: v_mfma_f32_16x16x32_f16 (4 accumulator registers per instruction).
+// Long enough for the clock governor to settle; reports TFLOP/s and the core clock.
+template<int SHAPE>
+__global__ void __launch_bounds__(256) mfma_shape_rate(const unsigned* seed, float* out, int iters)
+{
+    const int lane = threadIdx.x & 63;
+    u32x4     fa[4], fb[4];
+    for(int i = 0; i < 4; ++i)
+    {
+        unsigned h = seed[(threadIdx.x * 8 + i) & 4095];
+        fa[i] = u32x4{h, h * 2654435761u, h ^ 0x3c003c00u, h * 40503u};
+        fb[i] = u32x4{h * 69069u, h ^ 0xbc00bc00u, h * 1664525u, h + 0x12345u};
+        // keep exponents in a sane range: clear the top exponent bit of every half
+        fa[i] &= u32x4{0xbfffbfffu, 0xbfffbfffu, 0xbfffbfffu, 0xbfffbfffu};
+        fb[i] &= u32x4{0xbfffbfffu, 0xbfffbfffu, 0xbfffbfffu, 0xbfffbfffu};
+    }
+    const unsigned long long clk0 = __builtin_amdgcn_s_memtime();
+    const unsigned long long rt0  = __builtin_amdgcn_s_memrealtime();
+    float s = 0.0f;
+    if constexpr(SHAPE == 0)
+    {
+        f32x16 acc[16];
+        for(int c = 0; c < 16; ++c)
+            for(int v = 0; v < 16; ++v)
+                acc[c][v] = 0.0f;
+        for(int it = 0; it < iters; ++it)
+        {
+#pragma unroll
+            for(int c = 0; c < 16; ++c)
+                acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fa[c / 4]), __builtin_bit_cast(f16x8, fb[c % 4]), acc[c], 0, 0, 0);
+        }
+        for(int c = 0; c < 16; ++c)
+            for(int v = 0; v < 16; ++v)
+                s += acc[c][v];
+    }
+    else
+    {
+        f32x4 acc[64];
+        for(int c = 0; c < 64; ++c)
+            for(int v = 0; v < 4; ++v)
+                acc[c][v] = 0.0f;
+        for(int it = 0; it < iters; ++it)
+        {
+#pragma unroll
+            for(int c = 0; c < 32; ++c) // 32 x (16x16x32) = the FLOPs of 16 x (32x32x16)
+                acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fa[c % 4]), __builtin_bit_cast(f16x8, fb[(c / 4) % 4]), acc[c], 0, 0, 0);
+        }
+        for(int c = 0; c < 64; ++c)
+            for(int v = 0; v < 4; ++v)
+                s += acc[c][v];
+    }
+    if(s == 12345.678f)
+        out[0] = s;
+    if(blockIdx.x == 0 && threadIdx.x == 0)
+    {
+        out[1] = (float)(__builtin_amdgcn_s_memtime() - clk0);
+        out[2] = (float)(__builtin_amdgcn_s_memrealtime() - rt0);
+    }
+    (void)lane;
+}
+
 static float time_ms(hipEvent_t a, hipEvent_t b)
 {
     float ms = 0.0f;
@@ -682,6 +746,43 @@ int main(int argc, char** argv)
         run("global_load_lds x4 per 16 MFMA, 1 GiB source", mfma_with_stream<4, 4>, 4);
         run("global_load_dwordx4 x4 per 16 MFMA, L2-resident", mfma_with_stream<2, 4>, 4);
         run("ds_read_b128 x8 per 16 MFMA", mfma_with_stream<3, 8>, 8);
+    }
+
+
+    // MFMA shape vs sustained rate (4 waves per CU, ~30 ms each)
+    {
+        std::vector<unsigned> seed(4096);
+        unsigned              x = 0x2545F491u;
+        for(auto& v : seed)
+        {
+            x ^= x << 13;
+            x ^= x >> 17;
+            x ^= x << 5;
+            v = x;
+        }
+        unsigned* dSeed;
+        float*    dOut;
+        CHECK(hipMalloc(&dSeed, 4096 * 4));
+        CHECK(hipMemcpy(dSeed, seed.data(), 4096 * 4, hipMemcpyHostToDevice));
+        CHECK(hipMalloc(&dOut, 16));
+        const int iters = 100000, blocks = prop.multiProcessorCount;
+        auto run = [&](const char* name, auto kernel) {
+            kernel<<<blocks, 256>>>(dSeed, dOut, 1000);
+            CHECK(hipDeviceSynchronize());
+            CHECK(hipEventRecord(e0));
+            kernel<<<blocks, 256>>>(dSeed, dOut, iters);
+            CHECK(hipEventRecord(e1));
+            CHECK(hipEventSynchronize(e1));
+            const float  ms = time_ms(e0, e1);
+            const double tf = 2.0 * 32 * 32 * 16 * 16 * (double)iters * 4 * blocks / (ms * 1e-3) / 1e12;
+            float clk[3];
+            CHECK(hipMemcpy(clk, dOut, 12, hipMemcpyDeviceToHost));
+            std::printf("shape %-28s %8.2f ms %8.1f TFLOP/s  core clock %5.0f MHz\n", name, ms, tf, clk[2] > 0 ? clk[1] / clk[2] * 100.0 : 0.0);
+        };
+        run("32x32x16 f16, random operands", mfma_shape_rate<0>);
+        run("16x16x32 f16, random operands", mfma_shape_rate<1>);
+        run("32x32x16 f16, random operands", mfma_shape_rate<0>);
+        run("16x16x32 f16, random operands", mfma_shape_rate<1>);
     }
 
     // HBM copy ceiling
