@@ -54,6 +54,25 @@ def load_traffic():
         return None
 
 
+def mfma_ceiling():
+    """Sustained v_mfma_f32_32x32x16_f16 rate of this GPU on pseudo-random operands with
+    nothing else running (registers only, ~35 ms): what the power and clock management
+    leaves of the published peak for data like the benchmark's.  Context only."""
+    import subprocess
+
+    exe = os.path.join(ROOT, "rocm_wmma_gemm_amd", "lib", "mfma_probe")
+    try:
+        r = subprocess.run([exe, "--ceiling"], capture_output=True, text=True, timeout=60)
+        for line in r.stdout.splitlines():
+            if line.startswith("ceiling "):
+                _, tf, mhz = line.split()
+                return {"tflops": float(tf), "core_clock_mhz": float(mhz),
+                        "what": "MFMA-only loop, random fp16 operands, 4 waves/CU, all CUs"}
+    except (OSError, subprocess.SubprocessError, ValueError):
+        pass
+    return None
+
+
 def cpu_baseline(torch, A, B, M, N, K, gpu_c, la, lb, lc):
     """The oracle (a port of the reference's hgemm_cpu) on the host cores, whole
     4096^3 problem in one layout, one run; also used to spot-check the GPU result."""
@@ -104,10 +123,12 @@ def main() -> int:
     gen.manual_seed(1)
     A = (torch.rand(M * K, device="cuda", generator=gen) * 2 - 1).to(torch.float16)
     B = (torch.rand(K * N, device="cuda", generator=gen) * 2 - 1).to(torch.float16)
-    Cs = [torch.empty(M * N, dtype=torch.float16, device="cuda") for _ in LAYOUTS]
+    # one output buffer: every GEMM overwrites C, as every call of the library does
+    C = torch.empty(M * N, dtype=torch.float16, device="cuda")
+    Cs = [C for _ in LAYOUTS]
 
     def step():
-        for C, (la, lb, lc) in zip(Cs, LAYOUTS):
+        for (la, lb, lc) in LAYOUTS:
             loader.gemm(C, A, B, M, N, K, lc, la, lb)
 
     for _ in range(a.warmup):
@@ -136,7 +157,8 @@ def main() -> int:
         "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": round(2.0 * M * N * K / avg_launch_s / 1e12 / PEAK_TFLOPS, 4),
         "traffic": traffic.get("hbm_bytes_per_launch") if traffic else None,
-        "kernel": "direct_gemm<256x256x64> (one launch = one 4096^3 GEMM, 2*M*N*K FLOP)",
+        "kernel": "256x256 direct-to-LDS MFMA GEMM kernels (direct_gemm / pingpong_gemm as tuned per "
+                  "layout; one launch = one GEMM = 2*M*N*K FLOP)",
         "avg_launch_us": round(avg_launch_s * 1e6, 2),
         "algorithmic_bytes_per_launch": (M * K + K * N + M * N) * 2,
     }
@@ -169,6 +191,10 @@ def main() -> int:
         out["vendor_context"] = {"torch_matmul_fp16_4096_tflops":
                                  round(2.0 * M * N * K * a.steps / s / 1e12, 1)}
         del A2, B2, C2
+        ceil = mfma_ceiling()
+        if ceil:
+            out["mfma_ceiling_random_operands"] = ceil
+            out["pct_of_measured_mfma_ceiling"] = round(100.0 * tflops / ceil["tflops"], 2)
 
     if not a.no_cpu:
         la, lb, lc = 0, 1, 0

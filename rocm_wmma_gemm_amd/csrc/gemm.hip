@@ -6,6 +6,7 @@
 #include <rocm_wmma_gemm/gemm.hpp>
 #include <rocm_wmma_gemm_c.h>
 
+#include <algorithm>
 #include <mutex>
 #include <stdexcept>
 #include <string>
@@ -72,31 +73,44 @@ size_t out_bytes(int type_idx)
     return (type_idx == 1 || type_idx == 3) ? 4 : 2;
 }
 
-// Split-K workspace: one fp32 buffer per device, allocated on first use and kept
-// for the life of the process.  Calls that need more than the cap run with fewer
-// slices instead.
-constexpr size_t workspace_cap_bytes = size_t{256} << 20;
-constexpr int    max_devices         = 64;
+// Library-owned scratch memory, one buffer per device: fp32 partial planes of split-K
+// and zero-padded copies of ragged or misaligned operands.  Allocated on first use,
+// grown when a call needs more (after a device-wide synchronisation, since kernels of
+// earlier calls may still be reading the old buffer), never shrunk.
+constexpr size_t workspace_first_bytes = size_t{256} << 20;
+constexpr size_t workspace_limit_bytes = size_t{16} << 30;
+constexpr int    max_devices           = 64;
 std::mutex       workspace_mutex;
-float*           workspace_ptr[max_devices] = {};
+char*            workspace_ptr[max_devices]  = {};
+size_t           workspace_size[max_devices] = {};
 
-float* workspace_for_current_device()
+char* workspace_for_current_device(size_t bytes)
 {
     int dev = 0;
-    if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= max_devices)
+    if(bytes > workspace_limit_bytes || hipGetDevice(&dev) != hipSuccess || dev < 0
+       || dev >= max_devices)
     {
         return nullptr;
     }
     std::lock_guard<std::mutex> lock(workspace_mutex);
-    if(workspace_ptr[dev] == nullptr)
+    if(workspace_size[dev] < bytes)
     {
+        size_t want = std::max(bytes + bytes / 4, workspace_first_bytes);
+        if(workspace_ptr[dev] != nullptr)
+        {
+            (void)hipDeviceSynchronize();
+            (void)hipFree(workspace_ptr[dev]);
+            workspace_ptr[dev]  = nullptr;
+            workspace_size[dev] = 0;
+        }
         void* p = nullptr;
-        if(hipMalloc(&p, workspace_cap_bytes) != hipSuccess)
+        if(hipMalloc(&p, want) != hipSuccess)
         {
             (void)hipGetLastError();
             return nullptr;
         }
-        workspace_ptr[dev] = static_cast<float*>(p);
+        workspace_ptr[dev]  = static_cast<char*>(p);
+        workspace_size[dev] = want;
     }
     return workspace_ptr[dev];
 }
@@ -191,17 +205,26 @@ int staged_fallback(const variant_desc& v)
     return 0;
 }
 
-// The direct pipeline addresses a tile with 32-bit byte offsets from its origin.
-bool direct_eligible(const kernel_problem& p, const variant_desc& v, int mode)
+size_t round_up(size_t x, size_t to)
 {
-    if(mode != static_cast<int>(device::load_mode::vec_unguarded))
-    {
-        return false;
-    }
-    const unsigned long long a_ld = p.a_kmajor ? p.K : p.M, b_ld = p.b_kmajor ? p.K : p.N;
-    const unsigned long long a_span = (p.a_kmajor ? v.block_m : v.block_k) * a_ld * 2;
-    const unsigned long long b_span = (p.b_kmajor ? v.block_n : v.block_k) * b_ld * 2;
+    return (x + to - 1) / to * to;
+}
+
+// The direct pipelines address a tile with 32-bit byte offsets from its origin.
+bool spans_fit(const variant_desc& v, bool a_kmajor, bool b_kmajor, size_t lda, size_t ldb)
+{
+    const unsigned long long a_span = (a_kmajor ? v.block_m : v.block_k) * lda * 2ull;
+    const unsigned long long b_span = (b_kmajor ? v.block_n : v.block_k) * ldb * 2ull;
     return a_span < (1ull << 32) && b_span < (1ull << 32);
+}
+
+// Padding pays when the GEMM is large next to the copy: the copy moves every operand
+// element twice, the GEMM does 2*M*N*K/(M*K + K*N) FLOP per operand element.
+bool padding_pays(const kernel_problem& p)
+{
+    const double flop_per_elem
+        = 2.0 * p.M * p.N * p.K / (static_cast<double>(p.M) * p.K + static_cast<double>(p.K) * p.N);
+    return flop_per_elem >= 256.0 && p.M >= 128 && p.N >= 128 && p.K >= 128;
 }
 
 template<class OutT>
@@ -212,17 +235,57 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
     {
         return -1;
     }
-    if(variant_table[plan.variant].pipeline != 0
-       && !direct_eligible(p, variant_table[plan.variant],
-                           pick_mode(p, variant_table[plan.variant], plan.split_k)))
-    {
-        plan.variant = staged_fallback(variant_table[plan.variant]);
-    }
-    const variant_desc& v = variant_table[plan.variant];
     if(p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull)
     {
         throw std::runtime_error("rocm_wmma_gemm: M, N and K must each fit in 31 bits");
     }
+
+    // Operand views the kernel will see; may be replaced by padded copies below.
+    const void* a_ptr    = p.A;
+    const void* b_ptr    = p.B;
+    size_t      lda      = p.a_kmajor ? p.K : p.M;
+    size_t      ldb      = p.b_kmajor ? p.K : p.N;
+    size_t      k_kernel = p.K;
+    size_t      stride_a = p.stride_a, stride_b = p.stride_b;
+    int         mode     = pick_mode(p, variant_table[plan.variant], plan.split_k);
+    size_t      pack_bytes = 0;
+    bool        packed     = false;
+
+    if(variant_table[plan.variant].pipeline != 0)
+    {
+        const variant_desc& dv = variant_table[plan.variant];
+        const bool direct_ok = mode == static_cast<int>(device::load_mode::vec_unguarded)
+                               && spans_fit(dv, p.a_kmajor, p.b_kmajor, lda, ldb);
+        if(!direct_ok)
+        {
+            // Ragged or misaligned: run the direct kernel on zero-padded copies when the
+            // problem is big enough to pay for the copy, else take the staged kernel.
+            const size_t m_pad = round_up(p.M, dv.block_m), n_pad = round_up(p.N, dv.block_n),
+                         k_pad = round_up(p.K, dv.block_k);
+            const size_t pa = m_pad * k_pad, pb = k_pad * n_pad;
+            const size_t plda = p.a_kmajor ? k_pad : m_pad, pldb = p.b_kmajor ? k_pad : n_pad;
+            pack_bytes = round_up((pa + pb) * p.batch * in_bytes, 256);
+            if(padding_pays(p) && spans_fit(dv, p.a_kmajor, p.b_kmajor, plda, pldb)
+               && pack_bytes <= workspace_limit_bytes / 2)
+            {
+                packed   = true;
+                lda      = plda;
+                ldb      = pldb;
+                k_kernel = k_pad;
+                stride_a = pa;
+                stride_b = pb;
+                mode     = static_cast<int>(device::load_mode::vec_guarded); // guarded C stores
+            }
+            else
+            {
+                pack_bytes   = 0;
+                plan.variant = staged_fallback(dv);
+                mode         = pick_mode(p, variant_table[plan.variant], plan.split_k);
+            }
+        }
+    }
+    const variant_desc& v = variant_table[plan.variant];
+
     const size_t grid_m = (p.M + v.block_m - 1) / v.block_m;
     const size_t grid_n = (p.N + v.block_n - 1) / v.block_n;
     if(grid_m * grid_n > 0x7fffffffull)
@@ -231,45 +294,83 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
     }
 
     int       split_k = plan.split_k < 1 ? 1 : plan.split_k;
-    const int k_steps = static_cast<int>((p.K + v.block_k - 1) / v.block_k);
+    const int k_steps = static_cast<int>((k_kernel + v.block_k - 1) / v.block_k);
     if(split_k > k_steps)
     {
         split_k = k_steps;
     }
-    float* partials = nullptr;
-    if(split_k > 1)
-    {
-        // shrink the split until one chunk of batches fits the workspace
-        const size_t plane = p.M * p.N * sizeof(float);
-        while(split_k > 1 && plane * split_k > workspace_cap_bytes)
-        {
-            --split_k;
-        }
-        partials = split_k > 1 ? workspace_for_current_device() : nullptr;
-        if(partials == nullptr)
-        {
-            split_k = 1;
-        }
-    }
-    if(grid_m * grid_n * split_k > 0x7fffffffull)
+    if(grid_m * grid_n * static_cast<size_t>(split_k) > 0x7fffffffull)
     {
         split_k = 1;
     }
+    // Batches per launch: bounded by grid.y and, under split-K, by a 1 GiB budget for
+    // the partial planes.
+    const size_t plane_bytes        = p.M * p.N * sizeof(float);
+    size_t       batches_per_launch = std::min<size_t>(p.batch, 65535);
+    while(split_k > 1 && plane_bytes * split_k > (size_t{1} << 30))
+    {
+        --split_k;
+    }
+    if(split_k > 1)
+    {
+        batches_per_launch
+            = std::min(batches_per_launch, std::max<size_t>((size_t{1} << 30) / (plane_bytes * split_k), 1));
+    }
+    const size_t partial_bytes = split_k > 1 ? plane_bytes * split_k * batches_per_launch : 0;
 
-    const int mode = pick_mode(p, v, split_k);
-    kernel_fn fn   = lookup_kernel(type_idx, p.a_kmajor, p.b_kmajor, plan.variant, mode);
+    char* workspace = nullptr;
+    if(pack_bytes + partial_bytes > 0)
+    {
+        workspace = workspace_for_current_device(pack_bytes + partial_bytes);
+        if(workspace == nullptr)
+        {
+            if(packed)
+            {
+                // no memory for the padded copies: take the general kernel instead
+                launch_plan retry = plan;
+                retry.variant     = staged_fallback(v);
+                return launch<OutT>(type_idx, retry, p, stream);
+            }
+            split_k = 1;
+        }
+    }
+    float* partials = split_k > 1 ? reinterpret_cast<float*>(workspace + pack_bytes) : nullptr;
+
+    if(packed)
+    {
+        auto* wa = reinterpret_cast<unsigned short*>(workspace);
+        auto* wb = wa + stride_a * p.batch;
+        // operand as a 2-D array: `outer` rows of `inner` contiguous elements
+        const size_t a_outer = p.a_kmajor ? p.M : p.K, a_inner = p.a_kmajor ? p.K : p.M;
+        const size_t b_outer = p.b_kmajor ? p.N : p.K, b_inner = p.b_kmajor ? p.K : p.N;
+        const size_t a_outer_pad = stride_a / lda, b_outer_pad = stride_b / ldb;
+        for(size_t b0 = 0; b0 < p.batch; b0 += 65535)
+        {
+            const unsigned nb = static_cast<unsigned>(std::min<size_t>(65535, p.batch - b0));
+            const dim3 ga(static_cast<unsigned>(std::min<size_t>((lda / 2 + 255) / 256, 64)),
+                          static_cast<unsigned>(std::min<size_t>(a_outer_pad, 65535)), nb);
+            device::pack_padded<unsigned short><<<ga, dim3(256), 0, stream>>>(
+                static_cast<const unsigned short*>(p.A) + b0 * p.stride_a, wa + b0 * stride_a,
+                static_cast<int>(a_outer), static_cast<int>(a_inner), static_cast<int>(a_outer_pad),
+                static_cast<int>(lda), static_cast<long long>(p.stride_a),
+                static_cast<long long>(stride_a));
+            const dim3 gb(static_cast<unsigned>(std::min<size_t>((ldb / 2 + 255) / 256, 64)),
+                          static_cast<unsigned>(std::min<size_t>(b_outer_pad, 65535)), nb);
+            device::pack_padded<unsigned short><<<gb, dim3(256), 0, stream>>>(
+                static_cast<const unsigned short*>(p.B) + b0 * p.stride_b, wb + b0 * stride_b,
+                static_cast<int>(b_outer), static_cast<int>(b_inner), static_cast<int>(b_outer_pad),
+                static_cast<int>(ldb), static_cast<long long>(p.stride_b),
+                static_cast<long long>(stride_b));
+        }
+        a_ptr = wa;
+        b_ptr = wb;
+    }
+
+    kernel_fn fn = lookup_kernel(type_idx, p.a_kmajor, p.b_kmajor, plan.variant, mode);
     if(fn == nullptr)
     {
         // reference kernel_launcher.hpp:119-125 throws the same way
         throw std::runtime_error("No kernel available for the requested configuration and layout");
-    }
-
-    // Batches per launch: bounded by grid.y and, under split-K, by the workspace.
-    size_t batches_per_launch = 65535;
-    if(split_k > 1)
-    {
-        const size_t fit = workspace_cap_bytes / (p.M * p.N * sizeof(float) * split_k);
-        batches_per_launch = std::min(batches_per_launch, std::max<size_t>(fit, 1));
     }
 
     for(size_t b0 = 0; b0 < p.batch; b0 += batches_per_launch)
@@ -277,13 +378,15 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         const size_t nb = std::min(batches_per_launch, p.batch - b0);
         device::gemm_args args;
         args.C = static_cast<char*>(p.C) + b0 * p.stride_c * sizeof(OutT);
-        args.A = static_cast<const char*>(p.A) + b0 * p.stride_a * in_bytes;
-        args.B = static_cast<const char*>(p.B) + b0 * p.stride_b * in_bytes;
+        args.A = static_cast<const char*>(a_ptr) + b0 * stride_a * in_bytes;
+        args.B = static_cast<const char*>(b_ptr) + b0 * stride_b * in_bytes;
         args.M = static_cast<int>(p.M);
         args.N = static_cast<int>(p.N);
-        args.K = static_cast<int>(p.K);
-        args.batch_stride_a = static_cast<long long>(p.stride_a);
-        args.batch_stride_b = static_cast<long long>(p.stride_b);
+        args.K = static_cast<int>(k_kernel);
+        args.lda = static_cast<long long>(lda);
+        args.ldb = static_cast<long long>(ldb);
+        args.batch_stride_a = static_cast<long long>(stride_a);
+        args.batch_stride_b = static_cast<long long>(stride_b);
         args.batch_stride_c = static_cast<long long>(p.stride_c);
         args.grid_m         = static_cast<int>(grid_m);
         args.grid_n         = static_cast<int>(grid_n);

@@ -56,6 +56,8 @@ struct gemm_args
     const void* A;
     const void* B;
     int         M, N, K; // C is M x N row-major in kernel space
+    long long   lda, ldb; // leading dimension of each operand along its contiguous axis:
+                          // K (or the padded K) if K-contiguous, else the row count
     long long   batch_stride_a, batch_stride_b, batch_stride_c; // elements
     int         grid_m, grid_n; // tiles along M and N
     int         group; // tile-row band height of the tile map
@@ -403,10 +405,10 @@ struct staged_gemm
         const InT* B = static_cast<const InT*>(args.B) + batch * args.batch_stride_b;
 
         // Element (row, k) of A at A[row*a_sr + k*a_sk]; element (k, col) of B at B[col*b_sr + k*b_sk].
-        const long long a_sr = A_KMAJOR ? args.K : 1;
-        const long long a_sk = A_KMAJOR ? 1 : args.M;
-        const long long b_sr = B_KMAJOR ? args.K : 1;
-        const long long b_sk = B_KMAJOR ? 1 : args.N;
+        const long long a_sr = A_KMAJOR ? args.lda : 1;
+        const long long a_sk = A_KMAJOR ? 1 : args.lda;
+        const long long b_sr = B_KMAJOR ? args.ldb : 1;
+        const long long b_sk = B_KMAJOR ? 1 : args.ldb;
 
         const InT* a_tile = A + row0 * a_sr;
         const InT* b_tile = B + col0 * b_sr;
@@ -547,6 +549,47 @@ __global__ void __launch_bounds__(256) reduce_partials(OutT* __restrict__ C,
             s += P[k * plane + i];
         }
         out[i] = to_out<OutT>(s);
+    }
+}
+
+// Copies a dense 2-D array of 16-bit elements (`outer` rows of `inner` contiguous
+// elements, any alignment) into a zero-padded one whose rows are `inner_pad` long and
+// 16-byte aligned and which has `outer_pad` rows.  Lets ragged or misaligned operands
+// take the direct-to-LDS kernels, which need whole tiles and aligned rows; the zero
+// padding along K adds nothing to the products.
+template<class Elem16>
+__global__ void __launch_bounds__(256) pack_padded(const Elem16* __restrict__ src,
+                                                   Elem16* __restrict__ dst,
+                                                   int       outer,
+                                                   int       inner,
+                                                   int       outer_pad,
+                                                   int       inner_pad,
+                                                   long long src_batch_stride,
+                                                   long long dst_batch_stride)
+{
+    static_assert(sizeof(Elem16) == 2, "16-bit elements only");
+    const Elem16* s = src + blockIdx.z * src_batch_stride;
+    unsigned int*         d = reinterpret_cast<unsigned int*>(dst + blockIdx.z * dst_batch_stride);
+    const int             pairs = inner_pad / 2; // inner_pad is even
+    for(int o = blockIdx.y; o < outer_pad; o += gridDim.y)
+    {
+        const Elem16* row = s + (long long)o * inner;
+        for(int i = blockIdx.x * blockDim.x + threadIdx.x; i < pairs; i += gridDim.x * blockDim.x)
+        {
+            unsigned int lo = 0u, hi = 0u;
+            if(o < outer)
+            {
+                if(2 * i < inner)
+                {
+                    lo = row[2 * i];
+                }
+                if(2 * i + 1 < inner)
+                {
+                    hi = row[2 * i + 1];
+                }
+            }
+            d[(long long)o * pairs + i] = lo | (hi << 16);
+        }
     }
 }
 

@@ -48,7 +48,8 @@ template<in_kind IN,
          int  BK,
          int  WAVES_M,
          int  WAVES_N,
-         int  STAGES>
+         int  STAGES,
+         bool GUARD_C = false>
 struct pingpong_gemm
 {
     using InT = typename std::conditional<IN == in_kind::f16, _Float16, __bf16>::type;
@@ -114,8 +115,8 @@ struct pingpong_gemm
         const InT* A = static_cast<const InT*>(args.A) + batch * args.batch_stride_a;
         const InT* B = static_cast<const InT*>(args.B) + batch * args.batch_stride_b;
 
-        const long long a_ld = A_KMAJOR ? args.K : args.M;
-        const long long b_ld = B_KMAJOR ? args.K : args.N;
+        const long long a_ld = args.lda;
+        const long long b_ld = args.ldb;
         const long long a_sr = A_KMAJOR ? a_ld : 1, a_sk = A_KMAJOR ? 1 : a_ld;
         const long long b_sr = B_KMAJOR ? b_ld : 1, b_sk = B_KMAJOR ? 1 : b_ld;
 
@@ -239,7 +240,10 @@ struct pingpong_gemm
                     {
                         const int row
                             = row0 + wave_m * WTM + i * 32 + 8 * (v / 4) + 4 * lane_hi + (v % 4);
-                        C[(long long)row * args.N + col] = to_out<OutT>(acc[i][j][v]);
+                        if(!GUARD_C || (row < args.M && col < args.N))
+                        {
+                            C[(long long)row * args.N + col] = to_out<OutT>(acc[i][j][v]);
+                        }
                     }
                 }
             }
@@ -260,7 +264,10 @@ struct pingpong_gemm
                     {
                         const int row
                             = row0 + wave_m * WTM + i * 32 + 8 * (v / 4) + 4 * lane_hi + (v % 4);
-                        P[(long long)row * args.N + col] = acc[i][j][v];
+                        if(!GUARD_C || (row < args.M && col < args.N))
+                        {
+                            P[(long long)row * args.N + col] = acc[i][j][v];
+                        }
                     }
                 }
             }

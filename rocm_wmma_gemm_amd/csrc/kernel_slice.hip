@@ -29,21 +29,23 @@ constexpr kernel_fn entry()
         return &device::gemm_entry<
             device::staged_gemm<kIn, out_t, RWG_AK != 0, RWG_BK != 0, BM, BN, BK, WM, WN, MODE>>;
     }
-    else if constexpr(MODE == device::load_mode::vec_unguarded && PIPE == 1)
+    else if constexpr(MODE != device::load_mode::scalar && PIPE == 1)
     {
+        // vec_guarded here means: operands are whole aligned tiles (the host padded
+        // them if need be) but C is ragged, so the stores are guarded
         return &device::gemm_entry<
             device::direct_gemm<kIn, out_t, RWG_AK != 0, RWG_BK != 0, BM, BN, BK, WM, WN,
-                                (BK == 64 ? 2 : 4)>>;
+                                (BK == 64 ? 2 : 4), MODE == device::load_mode::vec_guarded>>;
     }
-    else if constexpr(MODE == device::load_mode::vec_unguarded && PIPE == 2)
+    else if constexpr(MODE != device::load_mode::scalar && PIPE == 2)
     {
         return &device::gemm_entry<
             device::pingpong_gemm<kIn, out_t, RWG_AK != 0, RWG_BK != 0, BM, BN, BK, WM, WN,
-                                  (BK == 64 ? 2 : 4)>>;
+                                  (BK == 64 ? 2 : 4), MODE == device::load_mode::vec_guarded>>;
     }
     else
     {
-        return nullptr; // the direct pipeline only runs whole, aligned tiles
+        return nullptr; // the direct pipelines never load 2 bytes at a time
     }
 }
 } // namespace

@@ -6,6 +6,8 @@
 //   mfma_probe --dump     additionally print raw lane dumps of the LDS paths
 //   mfma_probe --copy N   run only the copy kernel over N MiB (reference point for
 //                         scaling FETCH_SIZE / WRITE_SIZE counters)
+//   mfma_probe --ceiling  run only the sustained MFMA-rate measurement on pseudo-random
+//                         fp16 operands and print one line: "ceiling <TFLOP/s> <MHz>"
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -510,11 +512,14 @@ static bool check_product(const char* name, int M, int N, int K, F launch)
 int main(int argc, char** argv)
 {
     bool   dump     = false;
+    bool   ceiling  = false;
     size_t copy_mib = 0;
     for(int i = 1; i < argc; ++i)
     {
         if(!std::strcmp(argv[i], "--dump"))
             dump = true;
+        if(!std::strcmp(argv[i], "--ceiling"))
+            ceiling = true;
         if(!std::strcmp(argv[i], "--copy") && i + 1 < argc)
             copy_mib = std::strtoull(argv[++i], nullptr, 10);
     }
@@ -523,6 +528,37 @@ int main(int argc, char** argv)
     hipEvent_t e0, e1;
     CHECK(hipEventCreate(&e0));
     CHECK(hipEventCreate(&e1));
+
+    if(ceiling)
+    {
+        std::vector<unsigned> seed(4096);
+        unsigned              x = 0x2545F491u;
+        for(auto& v : seed)
+        {
+            x ^= x << 13;
+            x ^= x >> 17;
+            x ^= x << 5;
+            v = x;
+        }
+        unsigned* dSeed;
+        float*    dOut;
+        CHECK(hipMalloc(&dSeed, 4096 * 4));
+        CHECK(hipMemcpy(dSeed, seed.data(), 4096 * 4, hipMemcpyHostToDevice));
+        CHECK(hipMalloc(&dOut, 16));
+        const int iters = 100000, blocks = prop.multiProcessorCount;
+        mfma_shape_rate<0><<<blocks, 256>>>(dSeed, dOut, 20000); // lets the clock governor settle
+        CHECK(hipDeviceSynchronize());
+        CHECK(hipEventRecord(e0));
+        mfma_shape_rate<0><<<blocks, 256>>>(dSeed, dOut, iters);
+        CHECK(hipEventRecord(e1));
+        CHECK(hipEventSynchronize(e1));
+        const float  ms = time_ms(e0, e1);
+        const double tf = 2.0 * 32 * 32 * 16 * 16 * (double)iters * 4 * blocks / (ms * 1e-3) / 1e12;
+        float        clk[3];
+        CHECK(hipMemcpy(clk, dOut, 12, hipMemcpyDeviceToHost));
+        std::printf("ceiling %.1f %.0f\n", tf, clk[2] > 0 ? clk[1] / clk[2] * 100.0 : 0.0);
+        return 0;
+    }
 
     if(copy_mib)
     {
