@@ -110,6 +110,29 @@ def test_ragged_and_tiny_shapes(loader, type_name, lc, la, lb):
         check_against_oracle(gpu, A, B, M, N, K, lc, la, lb, din, dout)
 
 
+@pytest.mark.parametrize("type_name", ["f16_f16", "f32_bf16"])
+def test_unaligned_base_pointers(loader, type_name):
+    """A, B and C starting one element past a 16-byte boundary: vector loads are not
+    legal, so small problems take the 2-byte-load path and large ones the padded copies."""
+    import torch
+
+    din, dout = TYPE_PAIRS[type_name]
+    for (M, N, K) in ((100, 72, 56), (520, 776, 328)):
+        for (lc, la, lb) in [(0, 0, 1), (1, 1, 0), (0, 1, 1), (0, 0, 0)]:
+            A, B = make_inputs(M, N, K, la, lb, din, seed_a=5, seed_b=6)
+            bufA = torch.zeros(M * K + 9, dtype=torch_dtype(din), device="cuda")
+            bufB = torch.zeros(K * N + 9, dtype=torch_dtype(din), device="cuda")
+            bufC = torch.full((M * N + 9,), float("nan"), dtype=torch_dtype(dout), device="cuda")
+            dA, dB, dC = bufA[1:1 + M * K], bufB[1:1 + K * N], bufC[1:1 + M * N]
+            dA.copy_(to_device(A, din))
+            dB.copy_(to_device(B, din))
+            assert dA.data_ptr() % 16 != 0 and dB.data_ptr() % 16 != 0
+            loader.gemm(dC, dA, dB, M, N, K, lc, la, lb)
+            torch.cuda.synchronize()
+            assert torch.isnan(bufC[0]) and torch.isnan(bufC[1 + M * N:]).all()
+            check_against_oracle(to_host(dC.contiguous(), dout), A, B, M, N, K, lc, la, lb, din, dout)
+
+
 def test_does_not_write_outside_c(loader):
     """Guard rows/columns around C stay untouched for ragged shapes."""
     import torch
@@ -254,8 +277,12 @@ def test_llm_projection_shapes(loader, M, N, K):
         _full_size_case(loader, M, N, K, lc, la, lb, "f32_f16", (0, max(0, M - 32)))
 
 
-@pytest.mark.parametrize("M,N,K", [(4095, 5121, 3001), (1000, 1000, 1000), (1024, 1024, 65536)])
+@pytest.mark.parametrize("M,N,K", [(4095, 5121, 3001), (1000, 1000, 1000), (1024, 1024, 65536),
+                                   (8191, 8191, 8191)])
 def test_edge_tile_and_long_k(loader, M, N, K):
-    for (lc, la, lb) in [(0, 0, 1), (1, 0, 0), (0, 1, 0), (1, 1, 1)]:
+    """Non-tile-multiple and long-K shapes; 8191^3 needs padded copies larger than the
+    workspace's first allocation, so it also covers the workspace growing."""
+    layouts = [(0, 0, 1), (1, 0, 0), (0, 1, 0), (1, 1, 1)] if M < 8000 else [(0, 0, 1), (1, 1, 0)]
+    for (lc, la, lb) in layouts:
         _full_size_case(loader, M, N, K, lc, la, lb, "bf16_bf16", (0, max(0, M - 32)),
                         lo=-0.5, hi=0.5)
