@@ -445,6 +445,28 @@ __global__ void __launch_bounds__(256) mfma_shape_rate(const unsigned* seed, flo
             for(int v = 0; v < 16; ++v)
                 s += acc[c][v];
     }
+    else if constexpr(SHAPE == 2)
+    {
+        // same instruction, but each accumulator is updated 4 times in a row (the K-inner
+        // order of a GEMM tile), so the hardware can forward it instead of re-reading it
+        f32x16 acc[16];
+        for(int c = 0; c < 16; ++c)
+            for(int v = 0; v < 16; ++v)
+                acc[c][v] = 0.0f;
+        for(int it = 0; it < iters; it += 4)
+        {
+#pragma unroll
+            for(int c = 0; c < 16; ++c)
+            {
+#pragma unroll
+                for(int r = 0; r < 4; ++r)
+                    acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fa[(c / 4 + r) % 4]), __builtin_bit_cast(f16x8, fb[(c + r) % 4]), acc[c], 0, 0, 0);
+            }
+        }
+        for(int c = 0; c < 16; ++c)
+            for(int v = 0; v < 16; ++v)
+                s += acc[c][v];
+    }
     else
     {
         f32x4 acc[64];
@@ -815,10 +837,11 @@ int main(int argc, char** argv)
             CHECK(hipMemcpy(clk, dOut, 12, hipMemcpyDeviceToHost));
             std::printf("shape %-28s %8.2f ms %8.1f TFLOP/s  core clock %5.0f MHz\n", name, ms, tf, clk[2] > 0 ? clk[1] / clk[2] * 100.0 : 0.0);
         };
-        run("32x32x16 f16, random operands", mfma_shape_rate<0>);
-        run("16x16x32 f16, random operands", mfma_shape_rate<1>);
-        run("32x32x16 f16, random operands", mfma_shape_rate<0>);
-        run("16x16x32 f16, random operands", mfma_shape_rate<1>);
+        run("32x32x16 f16, round-robin accs", mfma_shape_rate<0>);
+        run("32x32x16 f16, chains of 4", mfma_shape_rate<2>);
+        run("16x16x32 f16, round-robin accs", mfma_shape_rate<1>);
+        run("32x32x16 f16, round-robin accs", mfma_shape_rate<0>);
+        run("32x32x16 f16, chains of 4", mfma_shape_rate<2>);
     }
 
     // HBM copy ceiling
