@@ -256,7 +256,16 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         const variant_desc& dv = variant_table[plan.variant];
         const bool direct_ok = mode == static_cast<int>(device::load_mode::vec_unguarded)
                                && spans_fit(dv, p.a_kmajor, p.b_kmajor, lda, ldb);
-        if(!direct_ok)
+        if(direct_ok)
+        {
+            // The 16x16x32 kernels store 4 elements of C at a time when unguarded.
+            const bool c_vec = aligned16(p.C) && (p.batch == 1 || p.stride_c % 8 == 0);
+            if(dv.pipeline >= 3 && !c_vec)
+            {
+                mode = static_cast<int>(device::load_mode::vec_guarded);
+            }
+        }
+        else
         {
             // Ragged or misaligned: run the direct kernel on zero-padded copies when the
             // problem is big enough to pay for the copy, else take the staged kernel.
@@ -281,6 +290,12 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
                 pack_bytes   = 0;
                 plan.variant = staged_fallback(dv);
                 mode         = pick_mode(p, variant_table[plan.variant], plan.split_k);
+                if(mode == static_cast<int>(device::load_mode::scalar))
+                {
+                    // The 2-byte-load path keeps far more values in flight per thread;
+                    // the small tile is the variant built to hold them without spilling.
+                    plan.variant = 0;
+                }
             }
         }
     }
@@ -329,6 +344,11 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
                 // no memory for the padded copies: take the general kernel instead
                 launch_plan retry = plan;
                 retry.variant     = staged_fallback(v);
+                if(pick_mode(p, variant_table[retry.variant], retry.split_k)
+                   == static_cast<int>(device::load_mode::scalar))
+                {
+                    retry.variant = 0;
+                }
                 return launch<OutT>(type_idx, retry, p, stream);
             }
             split_k = 1;
@@ -428,10 +448,11 @@ int run(int type_idx, const launch_plan* forced, void* C, void* A, void* B, size
     const kernel_problem p = to_kernel_space(C, A, B, M, N, K, batch, layout_c, layout_a, layout_b);
     launch_plan          plan
         = forced ? *forced : select_plan(M, N, K, type_idx, layout_c, layout_a, layout_b);
-    if(!forced)
+    if(!forced && variant_table[plan.variant].pipeline == 0)
     {
-        // The 2-byte-load fallback keeps far more values in flight per thread; the
-        // small tile is the variant built to hold them without spilling.
+        // Same rule as in launch() for a staged variant picked directly: misaligned
+        // operands go through the small tile.  A direct variant is left alone here:
+        // launch() decides between padded copies and the staged kernels.
         const int mode = pick_mode(p, variant_table[plan.variant], plan.split_k);
         if(mode == static_cast<int>(device::load_mode::scalar))
         {

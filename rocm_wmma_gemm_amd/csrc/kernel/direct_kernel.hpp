@@ -23,9 +23,11 @@
 //     t*512/BK .. (t+1)*512/BK - 1.
 //   M/N-contiguous operand: 1024-byte blocks of 4 k-rows x 128 rows-of-the-tile;
 //     block (kg, mh) at index kg * (ROWS/128) + mh; inside a block, k-row j holds
-//     16 chunks of 8 elements, chunk c in slot c ^ (4*j).  Wave-level load t fills
-//     block t.  ds_read_b64_tr_b16 then reads 4 k-rows x 32 elements per 32 lanes
-//     without bank conflicts (measured: 355 B/ns/CU vs 152 unswizzled).
+//     16 chunks of 8 elements, chunk c in slot c ^ (4*j) ^ (2*((kg/2)%2)).  Wave-level
+//     load t fills block t.  ds_read_b64_tr_b16 then reads, per 32 lanes, either 4
+//     k-rows x 32 elements of one block (32x32x16 MFMA) or 4 k-rows x 16 elements of
+//     two blocks two k groups apart (16x16x32 MFMA) without bank conflicts
+//     (measured for the first: 355 B/ns/CU vs 152 unswizzled).
 //
 // Same role as the staged kernel with respect to the reference (its gemm_impl,
 // prefetch_fragment, load_matrix: reference kernel/kernel.hpp:108-556,
@@ -52,27 +54,31 @@ using lds_char_ptr = __attribute__((address_space(3))) char*;
 //   ROWS   tile extent along M (for A) or N (for B)
 //   WT     rows of the tile owned by one wave (wave tile extent)
 //   WAVES  waves in the workgroup (all of them cooperate on every tile load)
-template<bool KMAJOR, int ROWS, int BK, int WT, int WAVES>
+//   MI     MFMA shape: 32 = v_mfma_f32_32x32x16 (lane l feeds row l%32, k 8*(l/32)..+7),
+//                      16 = v_mfma_f32_16x16x32 (lane l feeds row l%16, k 8*(l/16)..+7)
+template<bool KMAJOR, int ROWS, int BK, int WT, int WAVES, int MI = 32>
 struct direct_operand
 {
     static_assert(BK == 64 || BK == 32, "direct pipeline supports BK of 32 and 64");
+    static_assert(MI == 32 || MI == 16, "MFMA shapes: 32x32x16 and 16x16x32");
     static constexpr int CH         = BK / 8; // 16-byte chunks per K-contiguous row
-    static constexpr int KK         = BK / 16; // MFMA K steps per tile
+    static constexpr int KSTEP      = MI == 32 ? 16 : 32; // K extent of one MFMA
+    static constexpr int KK         = BK / KSTEP; // MFMA K steps per tile
     static constexpr int TILE_BYTES = ROWS * BK * 2;
     static constexpr int LOADS      = TILE_BYTES / 1024; // wave-level loads per tile
     static_assert(LOADS % WAVES == 0, "tile loads must divide over the waves");
     static constexpr int PER_WAVE = LOADS / WAVES;
-    static constexpr int T        = WT / 32; // 32-row MFMA operand tiles per wave
+    static constexpr int T        = WT / MI; // MI-row MFMA operand tiles per wave
     static constexpr int MH       = ROWS / 128; // 128-row halves (M/N-contiguous layout)
     static constexpr int DS_PER_FRAGMENT = KMAJOR ? 1 : 2; // LDS reads behind one fragment()
+    static constexpr int NOFF     = KMAJOR ? KK : T;
     static_assert(KMAJOR || ROWS % 128 == 0, "M/N-contiguous layout works in 128-row halves");
-    static_assert(T <= 4, "frag_off holds at most 4 entries");
 
     // Per-lane element offset (from the tile origin at k = 0) of the 16 bytes this
     // lane fetches in the wave's i-th load; advancing a tile adds BK * stride_k.
     unsigned int lane_off[PER_WAVE];
     // Per-lane LDS byte offsets for fragment reads (within an operand tile).
-    int frag_off[4]; // K-contiguous: one per K step; M/N-contiguous: one per operand tile i
+    int frag_off[NOFF]; // K-contiguous: one per K step; M/N-contiguous: one per operand tile i
 
     __device__ __forceinline__ void init(int wave, int lane, long long ld, int wave_row0)
     {
@@ -91,21 +97,23 @@ struct direct_operand
             {
                 const int kg = t / MH, mh = t % MH;
                 const int j = lane / 16, cphys = lane % 16;
-                const int c = cphys ^ (4 * j);
+                const int c = cphys ^ (4 * j) ^ (2 * ((kg >> 1) & 1));
                 lane_off[i] = (unsigned int)((long long)(kg * 4 + j) * ld + mh * 128 + c * 8);
             }
         }
         if constexpr(KMAJOR)
         {
-            const int lo = lane & 31, hi = lane >> 5;
-            const int row = wave_row0 + lo; // swizzle_of_row(row + 32*i) == swizzle_of_row(row)
+            // swizzle_of_row(row + 16*i) == swizzle_of_row(row)
+            const int row = wave_row0 + (lane & (MI - 1));
+            const int hi  = lane / MI; // which 8 k values of the K step this lane feeds
 #pragma unroll
             for(int kk = 0; kk < KK; ++kk)
             {
-                frag_off[kk] = row * (16 * CH) + (((kk * 2 + hi) ^ swizzle_of_row<CH>(row)) * 16);
+                frag_off[kk] = row * (16 * CH)
+                               + (((kk * (KSTEP / 8) + hi) ^ swizzle_of_row<CH>(row)) * 16);
             }
         }
-        else
+        else if constexpr(MI == 32)
         {
             const int b = lane / 16, s = lane % 16, j = s / 4;
 #pragma unroll
@@ -115,9 +123,24 @@ struct direct_operand
                 const int mh = m / 128, mm = m % 128;
                 const int c  = mm / 8;
                 // k group of K step 0, first half: kg = 2*(b/2); other (kk, h) add
-                // (kk*4 + h) * MH * 1024 bytes
-                frag_off[i] = ((2 * (b / 2)) * MH + mh) * 1024 + (j * 16 + (c ^ (4 * j))) * 16
-                              + (mm % 8) * 2;
+                // (kk*4 + h) * MH * 1024 bytes and leave (kg >> 1) & 1 == b/2
+                frag_off[i] = ((2 * (b / 2)) * MH + mh) * 1024
+                              + (j * 16 + (c ^ (4 * j) ^ (2 * (b / 2)))) * 16 + (mm % 8) * 2;
+            }
+        }
+        else
+        {
+            // 16-lane block g reads k = 8g + 4h + j (h: which of the two reads), rows
+            // 16i .. 16i+15 of the wave tile: kg = kk*8 + 2g + h, (kg >> 1) & 1 == g & 1
+            const int g = lane / 16, s = lane % 16, j = s / 4;
+#pragma unroll
+            for(int i = 0; i < T; ++i)
+            {
+                const int m  = wave_row0 + i * 16 + (s % 4) * 4;
+                const int mh = m / 128, mm = m % 128;
+                const int c  = mm / 8;
+                frag_off[i] = ((2 * g) * MH + mh) * 1024
+                              + (j * 16 + (c ^ (4 * j) ^ (2 * (g & 1)))) * 16 + (mm % 8) * 2;
             }
         }
     }
@@ -145,14 +168,14 @@ struct direct_operand
         if constexpr(KMAJOR)
         {
             return *reinterpret_cast<__attribute__((address_space(3))) u32x4*>(
-                lds_tile + frag_off[kk] + i * (32 * 16 * CH));
+                lds_tile + frag_off[kk] + i * (MI * 16 * CH));
         }
         else
         {
             auto* p0 = reinterpret_cast<__attribute__((address_space(3))) fp16x4_raw*>(
-                lds_tile + frag_off[i] + (kk * 4 + 0) * MH * 1024);
+                lds_tile + frag_off[i] + (kk * (KSTEP / 4) + 0) * MH * 1024);
             auto* p1 = reinterpret_cast<__attribute__((address_space(3))) fp16x4_raw*>(
-                lds_tile + frag_off[i] + (kk * 4 + 1) * MH * 1024);
+                lds_tile + frag_off[i] + (kk * (KSTEP / 4) + 1) * MH * 1024);
             const fp16x4_raw lo = __builtin_amdgcn_ds_read_tr16_b64_v4f16(p0);
             const fp16x4_raw hi = __builtin_amdgcn_ds_read_tr16_b64_v4f16(p1);
             const uint2      l2 = __builtin_bit_cast(uint2, lo);
@@ -161,6 +184,98 @@ struct direct_operand
         }
     }
 };
+
+// Accumulator registers of one MFMA tile: 32x32 -> 16 per lane, 16x16 -> 4.
+template<int MI>
+using mfma_acc = typename std::conditional<MI == 32, f32x16, f32x4>::type;
+
+// acc += A-fragment x B-fragment for one MI x MI tile of C.  With the 16x16x32 shape
+// the operands go in swapped: the MFMA then computes the transposed tile, and a lane
+// ends up with 4 consecutive columns of one row of C.
+template<in_kind IN, int MI>
+__device__ __forceinline__ mfma_acc<MI> mfma_tile(u32x4 fa, u32x4 fb, mfma_acc<MI> acc)
+{
+    if constexpr(MI == 32)
+    {
+        return mfma_32x32x16<IN>(fa, fb, acc);
+    }
+    else
+    {
+        return mfma_16x16x32<IN>(fb, fa, acc);
+    }
+}
+
+// Store this wave's accumulators to a row-major M x N matrix of DstT (C itself, or
+// one fp32 plane of split-K partial sums) whose wave tile starts at (row_w, col_w).
+template<int MI, bool GUARD_C, int TM, int TN, class AccT, class DstT>
+__device__ __forceinline__ void write_out(
+const AccT (&acc)[TM][TN], DstT* D, int M, int N, int row_w, int col_w, int lane)
+{
+    if constexpr(MI == 32)
+    {
+        // Accumulator register v of a 32x32 tile is row 8*(v/4) + 4*(lane/32) + v%4,
+        // column lane%32.
+        const int lane_lo = lane & 31, lane_hi = lane >> 5;
+#pragma unroll
+        for(int i = 0; i < TM; ++i)
+        {
+#pragma unroll
+            for(int j = 0; j < TN; ++j)
+            {
+                const int col = col_w + j * 32 + lane_lo;
+#pragma unroll
+                for(int v = 0; v < 16; ++v)
+                {
+                    const int row = row_w + i * 32 + 8 * (v / 4) + 4 * lane_hi + (v % 4);
+                    if(!GUARD_C || (row < M && col < N))
+                    {
+                        D[(long long)row * N + col] = to_out<DstT>(acc[i][j][v]);
+                    }
+                }
+            }
+        }
+    }
+    else
+    {
+        // Transposed 16x16 tiles (the kernels feed the MFMA with B's fragment first): register v of tile (i, j) is row
+        // lane%16 of the tile, column 4*(lane/16) + v.  Whole tiles with an aligned
+        // destination take one 8- or 16-byte store per tile and lane.
+        const int r16 = lane & 15, g = lane >> 4;
+#pragma unroll
+        for(int i = 0; i < TM; ++i)
+        {
+            const int row = row_w + i * 16 + r16;
+#pragma unroll
+            for(int j = 0; j < TN; ++j)
+            {
+                const int       col = col_w + j * 16 + 4 * g;
+                const long long at  = (long long)row * N + col;
+                if constexpr(GUARD_C)
+                {
+#pragma unroll
+                    for(int v = 0; v < 4; ++v)
+                    {
+                        if(row < M && col + v < N)
+                        {
+                            D[at + v] = to_out<DstT>(acc[i][j][v]);
+                        }
+                    }
+                }
+                else
+                {
+                    typedef DstT dst4 __attribute__((ext_vector_type(4)));
+                    dst4 o;
+#pragma unroll
+                    for(int v = 0; v < 4; ++v)
+                    {
+                        o[v] = to_out<DstT>(acc[i][j][v]);
+                    }
+                    *reinterpret_cast<dst4*>(D + at) = o;
+                }
+            }
+        }
+    }
+}
 
 template<in_kind IN,
          class OutT,
@@ -172,7 +287,8 @@ template<in_kind IN,
          int  WAVES_M,
          int  WAVES_N,
          int  STAGES,
-         bool GUARD_C = false>
+         bool GUARD_C = false,
+         int  MI      = 32>
 struct direct_gemm
 {
     using InT = typename std::conditional<IN == in_kind::f16, _Float16, __bf16>::type;
@@ -181,9 +297,9 @@ struct direct_gemm
     static constexpr int THREADS   = 64 * WAVES;
     static constexpr int WTM       = BM / WAVES_M;
     static constexpr int WTN       = BN / WAVES_N;
-    static constexpr int TM        = WTM / 32;
-    static constexpr int TN        = WTN / 32;
-    static constexpr int KK        = BK / 16;
+    static constexpr int TM        = WTM / MI;
+    static constexpr int TN        = WTN / MI;
+    static constexpr int KK        = BK / (MI == 32 ? 16 : 32);
     static constexpr int A_BYTES   = BM * BK * 2;
     static constexpr int B_BYTES   = BN * BK * 2;
     static constexpr int STAGE     = A_BYTES + B_BYTES;
@@ -192,8 +308,10 @@ struct direct_gemm
     static_assert(KK % 2 == 0, "operand double-buffer parity must repeat every tile");
     static_assert(LDS_BYTES <= 160 * 1024, "tile ring does not fit the 160 KB LDS");
 
-    using op_a = direct_operand<A_KMAJOR, BM, BK, WTM, WAVES>;
-    using op_b = direct_operand<B_KMAJOR, BN, BK, WTN, WAVES>;
+    using op_a = direct_operand<A_KMAJOR, BM, BK, WTM, WAVES, MI>;
+    using op_b = direct_operand<B_KMAJOR, BN, BK, WTN, WAVES, MI>;
+    using acc_t = mfma_acc<MI>;
+    static constexpr int ACC_REGS = MI == 32 ? 16 : 4;
 
     static constexpr int VM_LOADS = op_a::PER_WAVE + op_b::PER_WAVE; // per wave, per tile
     static constexpr int DS_READS = TM * op_a::DS_PER_FRAGMENT + TN * op_b::DS_PER_FRAGMENT;
@@ -225,7 +343,7 @@ struct direct_gemm
     }
 
     __device__ __forceinline__ static void
-        multiply(const u32x4 (&fa)[TM], const u32x4 (&fb)[TN], f32x16 (&acc)[TM][TN])
+        multiply(const u32x4 (&fa)[TM], const u32x4 (&fb)[TN], acc_t (&acc)[TM][TN])
     {
 #pragma unroll
         for(int i = 0; i < TM; ++i)
@@ -233,7 +351,7 @@ struct direct_gemm
 #pragma unroll
             for(int j = 0; j < TN; ++j)
             {
-                acc[i][j] = mfma_32x32x16<IN>(fa[i], fb[j], acc[i][j]);
+                acc[i][j] = mfma_tile<IN, MI>(fa[i], fb[j], acc[i][j]);
             }
         }
     }
@@ -305,7 +423,7 @@ struct direct_gemm
                                                      const InT*   b_src,
                                                      u32x4 (&fa)[2][TM],
                                                      u32x4 (&fb)[2][TN],
-                                                     f32x16 (&acc)[TM][TN])
+                                                     acc_t (&acc)[TM][TN])
     {
         lds_char_ptr cur = lds + (it & (STAGES - 1)) * STAGE;
         lds_char_ptr nxt = lds + ((it + 1) & (STAGES - 1)) * STAGE;
@@ -360,8 +478,6 @@ struct direct_gemm
         const int wave    = __builtin_amdgcn_readfirstlane(tid >> 6);
         const int wave_m  = wave / WAVES_N;
         const int wave_n  = wave % WAVES_N;
-        const int lane_lo = lane & 31;
-        const int lane_hi = lane >> 5;
 
         const int tiles   = args.grid_m * args.grid_n;
         const int slice   = blockIdx.x / tiles;
@@ -399,7 +515,7 @@ struct direct_gemm
         const InT* b_src = B + col0 * b_sr + (long long)step_begin * BK * b_sk;
         const long long a_step = BK * a_sk, b_step = BK * b_sk;
 
-        f32x16 acc[TM][TN];
+        acc_t acc[TM][TN];
 #pragma unroll
         for(int i = 0; i < TM; ++i)
         {
@@ -407,7 +523,7 @@ struct direct_gemm
             for(int j = 0; j < TN; ++j)
             {
 #pragma unroll
-                for(int v = 0; v < 16; ++v)
+                for(int v = 0; v < ACC_REGS; ++v)
                 {
                     acc[i][j][v] = 0.0f;
                 }
@@ -451,54 +567,16 @@ struct direct_gemm
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
         }
 
-        // Epilogue: accumulator register v of a 32x32 tile is row
-        // 8*(v/4) + 4*(lane/32) + v%4, column lane%32.
         if(args.k_slices == 1)
         {
             OutT* C = static_cast<OutT*>(args.C) + batch * args.batch_stride_c;
-#pragma unroll
-            for(int i = 0; i < TM; ++i)
-            {
-#pragma unroll
-                for(int j = 0; j < TN; ++j)
-                {
-                    const int col = col0 + wave_n * WTN + j * 32 + lane_lo;
-#pragma unroll
-                    for(int v = 0; v < 16; ++v)
-                    {
-                        const int row
-                            = row0 + wave_m * WTM + i * 32 + 8 * (v / 4) + 4 * lane_hi + (v % 4);
-                        if(!GUARD_C || (row < args.M && col < args.N))
-                        {
-                            C[(long long)row * args.N + col] = to_out<OutT>(acc[i][j][v]);
-                        }
-                    }
-                }
-            }
+            write_out<MI, GUARD_C>(acc, C, args.M, args.N, row0 + wave_m * WTM, col0 + wave_n * WTN, lane);
         }
         else
         {
             float* P = args.partials
                        + ((long long)batch * args.k_slices + slice) * (long long)args.M * args.N;
-#pragma unroll
-            for(int i = 0; i < TM; ++i)
-            {
-#pragma unroll
-                for(int j = 0; j < TN; ++j)
-                {
-                    const int col = col0 + wave_n * WTN + j * 32 + lane_lo;
-#pragma unroll
-                    for(int v = 0; v < 16; ++v)
-                    {
-                        const int row
-                            = row0 + wave_m * WTM + i * 32 + 8 * (v / 4) + 4 * lane_hi + (v % 4);
-                        if(!GUARD_C || (row < args.M && col < args.N))
-                        {
-                            P[(long long)row * args.N + col] = acc[i][j][v];
-                        }
-                    }
-                }
-            }
+            write_out<MI, GUARD_C>(acc, P, args.M, args.N, row0 + wave_m * WTM, col0 + wave_n * WTN, lane);
         }
     }
 };

@@ -35,6 +35,7 @@ using u32x4  = unsigned int __attribute__((ext_vector_type(4)));
 using f16x8  = _Float16 __attribute__((ext_vector_type(8)));
 using bf16x8 = __bf16 __attribute__((ext_vector_type(8)));
 using f32x16 = float __attribute__((ext_vector_type(16)));
+using f32x4  = float __attribute__((ext_vector_type(4)));
 
 enum class in_kind
 {
@@ -76,6 +77,23 @@ __device__ __forceinline__ f32x16 mfma_32x32x16(u32x4 a, u32x4 b, f32x16 c)
     else
     {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+}
+
+// 16x16x32: lane l feeds row (column) l%16, k 8*(l/16)..+7 of the first (second)
+// operand; result register v is row 4*(l/16) + v, column l%16.
+template<in_kind IN>
+__device__ __forceinline__ f32x4 mfma_16x16x32(u32x4 a, u32x4 b, f32x4 c)
+{
+    if constexpr(IN == in_kind::f16)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(
+            __builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    else
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(
             __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     }
 }

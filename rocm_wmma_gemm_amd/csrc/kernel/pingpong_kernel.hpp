@@ -49,7 +49,8 @@ template<in_kind IN,
          int  WAVES_M,
          int  WAVES_N,
          int  STAGES,
-         bool GUARD_C = false>
+         bool GUARD_C = false,
+         int  MI      = 32>
 struct pingpong_gemm
 {
     using InT = typename std::conditional<IN == in_kind::f16, _Float16, __bf16>::type;
@@ -58,9 +59,9 @@ struct pingpong_gemm
     static constexpr int THREADS   = 64 * WAVES;
     static constexpr int WTM       = BM / WAVES_M;
     static constexpr int WTN       = BN / WAVES_N;
-    static constexpr int TM        = WTM / 32;
-    static constexpr int TN        = WTN / 32;
-    static constexpr int KK        = BK / 16;
+    static constexpr int TM        = WTM / MI;
+    static constexpr int TN        = WTN / MI;
+    static constexpr int KK        = BK / (MI == 32 ? 16 : 32);
     static constexpr int A_BYTES   = BM * BK * 2;
     static constexpr int B_BYTES   = BN * BK * 2;
     static constexpr int STAGE     = A_BYTES + B_BYTES;
@@ -69,8 +70,9 @@ struct pingpong_gemm
     static_assert(STAGES == 4 || STAGES == 2, "stage ring must be a power of two");
     static_assert(LDS_BYTES <= 160 * 1024, "tile ring does not fit the 160 KB LDS");
 
-    using op_a = direct_operand<A_KMAJOR, BM, BK, WTM, WAVES>;
-    using op_b = direct_operand<B_KMAJOR, BN, BK, WTN, WAVES>;
+    using op_a  = direct_operand<A_KMAJOR, BM, BK, WTM, WAVES, MI>;
+    using op_b  = direct_operand<B_KMAJOR, BN, BK, WTN, WAVES, MI>;
+    using acc_t = mfma_acc<MI>;
 
     static constexpr int VM_LOADS = op_a::PER_WAVE + op_b::PER_WAVE; // per wave, per tile
     static_assert((STAGES - 1) * VM_LOADS < 64, "vmcnt is a 6-bit counter");
@@ -91,8 +93,6 @@ struct pingpong_gemm
         const int group   = wave >> 2; // waves w and w+4 share a SIMD
         const int wave_m  = wave / WAVES_N;
         const int wave_n  = wave % WAVES_N;
-        const int lane_lo = lane & 31;
-        const int lane_hi = lane >> 5;
 
         const int tiles   = args.grid_m * args.grid_n;
         const int slice   = blockIdx.x / tiles;
@@ -129,7 +129,7 @@ struct pingpong_gemm
         const InT* b_src = B + col0 * b_sr + (long long)step_begin * BK * b_sk;
         const long long a_step = BK * a_sk, b_step = BK * b_sk;
 
-        f32x16 acc[TM][TN];
+        acc_t acc[TM][TN];
 #pragma unroll
         for(int i = 0; i < TM; ++i)
         {
@@ -137,7 +137,7 @@ struct pingpong_gemm
             for(int j = 0; j < TN; ++j)
             {
 #pragma unroll
-                for(int v = 0; v < 16; ++v)
+                for(int v = 0; v < (MI == 32 ? 16 : 4); ++v)
                 {
                     acc[i][j][v] = 0.0f;
                 }
@@ -207,7 +207,7 @@ struct pingpong_gemm
 #pragma unroll
                         for(int j = 0; j < TN; ++j)
                         {
-                            acc[i][j] = mfma_32x32x16<IN>(fa[kk][i], fb[kk][j], acc[i][j]);
+                            acc[i][j] = mfma_tile<IN, MI>(fa[kk][i], fb[kk][j], acc[i][j]);
                         }
                     }
                 }
@@ -223,54 +223,18 @@ struct pingpong_gemm
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(0)); // redundant tail loads
         }
 
-        // Epilogue: accumulator register v of a 32x32 tile is row
-        // 8*(v/4) + 4*(lane/32) + v%4, column lane%32.
         if(args.k_slices == 1)
         {
             OutT* C = static_cast<OutT*>(args.C) + batch * args.batch_stride_c;
-#pragma unroll
-            for(int i = 0; i < TM; ++i)
-            {
-#pragma unroll
-                for(int j = 0; j < TN; ++j)
-                {
-                    const int col = col0 + wave_n * WTN + j * 32 + lane_lo;
-#pragma unroll
-                    for(int v = 0; v < 16; ++v)
-                    {
-                        const int row
-                            = row0 + wave_m * WTM + i * 32 + 8 * (v / 4) + 4 * lane_hi + (v % 4);
-                        if(!GUARD_C || (row < args.M && col < args.N))
-                        {
-                            C[(long long)row * args.N + col] = to_out<OutT>(acc[i][j][v]);
-                        }
-                    }
-                }
-            }
+            write_out<MI, GUARD_C>(
+                acc, C, args.M, args.N, row0 + wave_m * WTM, col0 + wave_n * WTN, lane);
         }
         else
         {
             float* P = args.partials
                        + ((long long)batch * args.k_slices + slice) * (long long)args.M * args.N;
-#pragma unroll
-            for(int i = 0; i < TM; ++i)
-            {
-#pragma unroll
-                for(int j = 0; j < TN; ++j)
-                {
-                    const int col = col0 + wave_n * WTN + j * 32 + lane_lo;
-#pragma unroll
-                    for(int v = 0; v < 16; ++v)
-                    {
-                        const int row
-                            = row0 + wave_m * WTM + i * 32 + 8 * (v / 4) + 4 * lane_hi + (v % 4);
-                        if(!GUARD_C || (row < args.M && col < args.N))
-                        {
-                            P[(long long)row * args.N + col] = acc[i][j][v];
-                        }
-                    }
-                }
-            }
+            write_out<MI, GUARD_C>(
+                acc, P, args.M, args.N, row0 + wave_m * WTM, col0 + wave_n * WTN, lane);
         }
     }
 };

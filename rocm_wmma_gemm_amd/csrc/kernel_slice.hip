@@ -23,7 +23,7 @@ using out_t = std::conditional<RWG_TYPE == 0, _Float16,
 template<int BM, int BN, int BK, int WM, int WN, int PIPE, device::load_mode MODE>
 constexpr kernel_fn entry()
 {
-    static_assert(PIPE == 0 || PIPE == 1 || PIPE == 2, "unknown pipeline");
+    static_assert(PIPE >= 0 && PIPE <= 4, "unknown pipeline");
     if constexpr(PIPE == 0)
     {
         return &device::gemm_entry<
@@ -42,6 +42,18 @@ constexpr kernel_fn entry()
         return &device::gemm_entry<
             device::pingpong_gemm<kIn, out_t, RWG_AK != 0, RWG_BK != 0, BM, BN, BK, WM, WN,
                                   (BK == 64 ? 2 : 4), MODE == device::load_mode::vec_guarded>>;
+    }
+    else if constexpr(MODE != device::load_mode::scalar && PIPE == 3)
+    {
+        return &device::gemm_entry<
+            device::direct_gemm<kIn, out_t, RWG_AK != 0, RWG_BK != 0, BM, BN, BK, WM, WN,
+                                (BK == 64 ? 2 : 4), MODE == device::load_mode::vec_guarded, 16>>;
+    }
+    else if constexpr(MODE != device::load_mode::scalar && PIPE == 4)
+    {
+        return &device::gemm_entry<
+            device::pingpong_gemm<kIn, out_t, RWG_AK != 0, RWG_BK != 0, BM, BN, BK, WM, WN,
+                                  (BK == 64 ? 2 : 4), MODE == device::load_mode::vec_guarded, 16>>;
     }
     else
     {

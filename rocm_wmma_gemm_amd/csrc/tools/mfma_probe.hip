@@ -416,8 +416,8 @@ template<int SHAPE>
 __global__ void __launch_bounds__(256) mfma_shape_rate(const unsigned* seed, float* out, int iters)
 {
     const int lane = threadIdx.x & 63;
-    u32x4     fa[4], fb[4];
-    for(int i = 0; i < 4; ++i)
+    u32x4     fa[8], fb[8];
+    for(int i = 0; i < 8; ++i)
     {
         unsigned h = seed[(threadIdx.x * 8 + i) & 4095];
         fa[i] = u32x4{h, h * 2654435761u, h ^ 0x3c003c00u, h * 40503u};
@@ -469,17 +469,17 @@ __global__ void __launch_bounds__(256) mfma_shape_rate(const unsigned* seed, flo
     }
     else
     {
-        f32x4 acc[64];
-        for(int c = 0; c < 64; ++c)
+        f32x4 acc[32];
+        for(int c = 0; c < 32; ++c)
             for(int v = 0; v < 4; ++v)
                 acc[c][v] = 0.0f;
         for(int it = 0; it < iters; ++it)
         {
 #pragma unroll
             for(int c = 0; c < 32; ++c) // 32 x (16x16x32) = the FLOPs of 16 x (32x32x16)
-                acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fa[c % 4]), __builtin_bit_cast(f16x8, fb[(c / 4) % 4]), acc[c], 0, 0, 0);
+                asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[c]) : "v"(fa[c % 4]), "v"(fb[c / 4]));
         }
-        for(int c = 0; c < 64; ++c)
+        for(int c = 0; c < 32; ++c)
             for(int v = 0; v < 4; ++v)
                 s += acc[c][v];
     }
@@ -824,7 +824,8 @@ int main(int argc, char** argv)
         CHECK(hipMemcpy(dSeed, seed.data(), 4096 * 4, hipMemcpyHostToDevice));
         CHECK(hipMalloc(&dOut, 16));
         const int iters = 100000, blocks = prop.multiProcessorCount;
-        auto run = [&](const char* name, auto kernel) {
+        auto run = [&](const char* name, auto kernel, int per_cu = 1) {
+            const int blocks = prop.multiProcessorCount * per_cu;
             kernel<<<blocks, 256>>>(dSeed, dOut, 1000);
             CHECK(hipDeviceSynchronize());
             CHECK(hipEventRecord(e0));
@@ -840,6 +841,7 @@ int main(int argc, char** argv)
         run("32x32x16 f16, round-robin accs", mfma_shape_rate<0>);
         run("32x32x16 f16, chains of 4", mfma_shape_rate<2>);
         run("16x16x32 f16, round-robin accs", mfma_shape_rate<1>);
+        run("16x16x32 f16, 2 blocks per CU", mfma_shape_rate<1>, 2);
         run("32x32x16 f16, round-robin accs", mfma_shape_rate<0>);
         run("32x32x16 f16, chains of 4", mfma_shape_rate<2>);
     }
