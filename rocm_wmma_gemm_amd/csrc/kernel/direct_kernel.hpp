@@ -90,7 +90,7 @@ struct direct_operand
             {
                 const int r    = (64 / CH) * t + lane / CH;
                 const int slot = lane % CH;
-                const int c    = slot ^ swizzle_of_row<CH>(r);
+                const int c    = slot ^ swizzle_of_row<CH, MI>(r);
                 lane_off[i]    = (unsigned int)(r * ld + c * 8);
             }
             else
@@ -110,7 +110,7 @@ struct direct_operand
             for(int kk = 0; kk < KK; ++kk)
             {
                 frag_off[kk] = row * (16 * CH)
-                               + (((kk * (KSTEP / 8) + hi) ^ swizzle_of_row<CH>(row)) * 16);
+                               + (((kk * (KSTEP / 8) + hi) ^ swizzle_of_row<CH, MI>(row)) * 16);
             }
         }
         else if constexpr(MI == 32)
@@ -159,6 +159,36 @@ struct direct_operand
                 16,
                 0,
                 RWG_LOAD_AUX);
+        }
+    }
+
+    // fragment() as volatile inline assembly, for the hand-scheduled kernel: the reads
+    // stay where the source puts them and the compiler neither tracks them (the caller
+    // waits with s_waitcnt lgkmcnt before the first use) nor orders them against the
+    // global -> LDS loads (behind such a load it puts s_waitcnt vmcnt(0) in front of
+    // every ds_read_b64_tr_b16 it knows of).  lds_tile is the byte address of the
+    // operand tile in LDS.
+    template<int I, int KKI>
+    __device__ __forceinline__ u32x4 fragment_pinned(unsigned int lds_tile) const
+    {
+        if constexpr(KMAJOR)
+        {
+            u32x4              r;
+            const unsigned int addr = lds_tile + (unsigned int)frag_off[KKI];
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(I * (MI * 16 * CH)));
+            return r;
+        }
+        else
+        {
+            uint2              lo, hi;
+            const unsigned int addr = lds_tile + (unsigned int)frag_off[I];
+            asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2"
+                         : "=v"(lo)
+                         : "v"(addr), "n"((KKI * (KSTEP / 4) + 0) * MH * 1024));
+            asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2"
+                         : "=v"(hi)
+                         : "v"(addr), "n"((KKI * (KSTEP / 4) + 1) * MH * 1024));
+            return u32x4{lo.x, lo.y, hi.x, hi.y};
         }
     }
 

@@ -105,18 +105,31 @@ __device__ __forceinline__ OutT to_out(float v)
     return static_cast<OutT>(v);
 }
 
-// Chunk slot swizzle.  The LDS has 64 banks of 4 bytes (256 bytes per clock) and a
-// 16-byte-per-lane read is served 16 lanes at a time, so the 16 rows read together
-// (same chunk column) must land in 16 distinct 16-byte columns of a 256-byte line.
-// A row of CH chunks spans 16*CH bytes, 16/CH rows share a line, and rows that
-// share a line position must differ in slot: slot = chunk ^ ((row / (16/CH)) % CH).
-// Measured on MI355X: this gives the full ~505 B/ns/CU, "chunk ^ (row % 8)" only
-// ~297 B/ns/CU (two-way conflicts), no swizzle 76 B/ns/CU.
-template<int CH>
+// Chunk slot swizzle.  The LDS has 64 banks of 4 bytes (256 bytes per clock); a
+// 16-byte-per-lane read of a wave is served in 4 cycles of 16 lanes each.  Measured
+// on MI355X (two lanes alone on one bank column slow down iff they share a cycle): the
+// cycles take, of each 32-lane half, the lanes of 4-lane quads {0,3,5,6} and
+// {1,2,4,7}.  The 16 lanes of a cycle must hit 16 distinct 16-byte columns of a
+// 256-byte line.  A row of CH chunks spans 16*CH bytes and 16/CH rows share a line.
+//   * 32x32x16 MFMA (lane l reads row l%32, chunk l/32): a cycle reads one chunk of
+//     rows 4q..4q+3 for the 4 quads q; slot = chunk ^ ((row / (16/CH)) % CH) gives
+//     ~505 B/ns/CU, "chunk ^ (row % 8)" ~297 (two-way conflicts), no swizzle 76.
+//   * 16x16x32 MFMA (lane l reads row l%16, chunk l/16): a cycle reads chunk g of
+//     rows 0-3 and 12-15 and chunk g^1 of rows 4-11.  The slot above is conflict-free
+//     for CH = 8 (~520 B/ns/CU) but two-way conflicted for CH = 4 (~300); there
+//     slot = chunk ^ 2*((row / 8) % 2) separates the rows that share a line position.
+template<int CH, int MI = 32>
 __device__ __forceinline__ int swizzle_of_row(int row)
 {
     static_assert(CH == 8 || CH == 4 || CH == 2, "unsupported BK");
-    return (row * CH / 16) % CH;
+    if constexpr(MI == 16 && CH == 4)
+    {
+        return 2 * ((row >> 3) & 1);
+    }
+    else
+    {
+        return (row * CH / 16) % CH;
+    }
 }
 
 // 16-byte chunk index (in u32x4 units) of (row, chunk) inside a tile.

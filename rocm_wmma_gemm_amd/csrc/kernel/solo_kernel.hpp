@@ -1,0 +1,392 @@
+// One-wave-per-SIMD MFMA GEMM kernel for gfx950 (4 waves, 128 x 128 wave tiles).
+//
+// Same data path as the direct kernel (direct_kernel.hpp: global -> LDS with
+// global_load_lds_dwordx4, swizzled LDS layouts, ds_read_b64_tr_b16 for operands that
+// are contiguous along M or N) on the 16x16x32 MFMA, but with the largest wave tile
+// the register file allows: 128 x 128 per wave = 256 accumulator registers, all of
+// the AGPRs.  A wave then reads 16 operand fragments from LDS per 64 MFMAs, against
+// 12 per 32 for the 128 x 64 wave tiles of the 8-wave kernels: one third fewer LDS
+// bytes per FLOP, which is what the power-capped clock responds to.
+//
+// With one wave per SIMD nothing hides a stall, so the schedule is fixed by hand:
+// the MFMAs are volatile inline assembly (which also pins every accumulator to its
+// AGPRs: with the builtin the register allocator moved accumulators between the two
+// register files inside the loop), and the LDS reads and global -> LDS loads of a K
+// step sit between them in source order.
+//
+// Ring of 2 tiles of BLOCK_K 64 (two MFMA K steps per tile, one barrier per tile;
+// K-contiguous rows are 128 bytes, so every load fetches whole cache lines).  The
+// fragments of the next K step are always read one step ahead, so the stage of the
+// tile being multiplied is free for the next loads as soon as all waves have passed
+// the barrier in the middle of the tile.  Measured with the shader clock on 8192^3:
+// 1117 + 1186 cycles for the two steps of a tile (1024 each would be MFMA-bound) plus
+// about 70 in the wait and the barrier, where issuing a tile's loads back to back
+// had cost 1700-1900 cycles for the second step.
+//
+// Role with respect to the reference: as the other kernels, its gemm_impl (reference
+// rocm_wmma_gemm/include/rocm_wmma_gemm/kernel/kernel.hpp:108-556).
+#ifndef ROCM_WMMA_GEMM_SOLO_KERNEL_HPP
+#define ROCM_WMMA_GEMM_SOLO_KERNEL_HPP
+
+#include <utility>
+
+#include "direct_kernel.hpp"
+
+namespace rocm_wmma_gemm
+{
+namespace device
+{
+
+// acc += (B fragment) x (A fragment): the transposed 16x16 tile, see write_out.
+template<in_kind IN>
+__device__ __forceinline__ void mfma_16x16x32_pinned(f32x4& acc, const u32x4& fa, const u32x4& fb)
+{
+    if constexpr(IN == in_kind::f16)
+    {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(fb), "v"(fa));
+    }
+    else
+    {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(fb), "v"(fa));
+    }
+}
+
+template<in_kind IN,
+         class OutT,
+         bool A_KMAJOR,
+         bool B_KMAJOR,
+         int  BM,
+         int  BN,
+         int  BK,
+         int  WAVES_M,
+         int  WAVES_N,
+         int  STAGES,
+         bool GUARD_C = false>
+struct solo_gemm
+{
+    using InT = typename std::conditional<IN == in_kind::f16, _Float16, __bf16>::type;
+
+    static constexpr int MI        = 16;
+    static constexpr int WAVES     = WAVES_M * WAVES_N;
+    static constexpr int THREADS   = 64 * WAVES;
+    static constexpr int WTM       = BM / WAVES_M;
+    static constexpr int WTN       = BN / WAVES_N;
+    static constexpr int TM        = WTM / MI;
+    static constexpr int TN        = WTN / MI;
+    static constexpr int MFMAS     = TM * TN;
+    static constexpr int A_BYTES   = BM * BK * 2;
+    static constexpr int B_BYTES   = BN * BK * 2;
+    static constexpr int STAGE     = A_BYTES + B_BYTES;
+    static constexpr int LDS_BYTES = STAGES * STAGE;
+    static_assert(BK == 64 && STAGES == 2, "ring of 2 tiles of BLOCK_K 64");
+    static_assert(LDS_BYTES <= 160 * 1024, "tile ring does not fit the 160 KB LDS");
+
+    using op_a = direct_operand<A_KMAJOR, BM, BK, WTM, WAVES, MI>;
+    using op_b = direct_operand<B_KMAJOR, BN, BK, WTN, WAVES, MI>;
+
+    static constexpr int VM_LOADS = op_a::PER_WAVE + op_b::PER_WAVE; // per wave, per tile
+    static_assert((STAGES - 1) * VM_LOADS < 64, "vmcnt is a 6-bit counter");
+
+    static constexpr int KK    = BK / 32; // MFMA K steps per tile
+    static constexpr int FRAGS = TM + TN;
+    // Fragment u (A fragments first, then B) is read after MFMA u * FRAG_GAP.
+    static constexpr int FRAG_GAP = 2;
+    static_assert(FRAGS * FRAG_GAP <= MFMAS, "fragment reads must fit under the MFMAs of a step");
+
+    // s_waitcnt immediate: lgkmcnt(0), expcnt untouched, vmcnt(n)
+    static constexpr int waitcnt_imm(int vmcnt)
+    {
+        return (vmcnt & 15) | (7 << 4) | (0 << 8) | ((vmcnt >> 4) << 14);
+    }
+
+    // Wave-level load v of the tile (A's loads first, then B's), as a buffer load: the
+    // tile origin goes into a buffer descriptor in scalar registers and the lane's byte
+    // offset inside the tile is loop-invariant, so a load costs no vector ALU work
+    // (with a 64-bit address per lane it cost an add per load and twice the address
+    // traffic; measured 1-2 % in throughput at the power limit).
+    __device__ __forceinline__ static void issue_one(const op_a&  oa,
+                                                     const op_b&  ob,
+                                                     int          v,
+                                                     const InT*   a_src,
+                                                     const InT*   b_src,
+                                                     lds_char_ptr stage,
+                                                     int          wave)
+    {
+        // dword 3 of the descriptor: 32-bit raw buffer; every tile span fits 32 bits
+        // (the host checks), so the range check never fires
+        constexpr int RSRC_FLAGS = 0x00020000;
+        if(v < op_a::PER_WAVE)
+        {
+            const int t    = wave + v * WAVES;
+            auto      rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<InT*>(a_src), 0, 0xffffffff, RSRC_FLAGS);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                rsrc,
+                (__attribute__((address_space(3))) void*)(stage + t * 1024),
+                16,
+                (int)(oa.lane_off[v] * 2u),
+                0,
+                0,
+                RWG_LOAD_AUX);
+        }
+        else
+        {
+            const int w    = v - op_a::PER_WAVE;
+            const int t    = wave + w * WAVES;
+            auto      rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<InT*>(b_src), 0, 0xffffffff, RSRC_FLAGS);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                rsrc,
+                (__attribute__((address_space(3))) void*)(stage + A_BYTES + t * 1024),
+                16,
+                (int)(ob.lane_off[w] * 2u),
+                0,
+                0,
+                RWG_LOAD_AUX);
+        }
+    }
+
+    // Everything a step works on.
+    struct step_ctx
+    {
+        const op_a&  oa;
+        const op_b&  ob;
+        unsigned int rd; // LDS byte address of the stage the fragments are read from
+        lds_char_ptr fill; // stage the loads go to
+        int          wave;
+        const InT*   a_src;
+        const InT*   b_src;
+    };
+
+    // Which loads of a tile a step issues: loads BEGIN .. BEGIN+COUNT-1 (A's loads come
+    // first, then B's), load BEGIN+v after MFMA FIRST + v * GAP.  The texture addresser
+    // of the CU takes about 16 cycles per 1 KiB load; four waves that issue a load every
+    // few MFMAs fill its queue and then stall in front of it, MFMAs included, so the
+    // loads are spread as evenly as the ring allows.
+    template<int FIRST, int GAP, int BEGIN, int COUNT>
+    struct load_plan
+    {
+        static_assert(COUNT == 0 || FIRST + (COUNT - 1) * GAP < MFMAS, "loads must fit under the MFMAs of a step");
+        static constexpr int first = FIRST, gap = GAP, begin = BEGIN, count = COUNT;
+    };
+    using no_loads = load_plan<0, 1, 0, 0>;
+
+    // MFMA number M of a step and the memory instructions that follow it: fragment
+    // M / FRAG_GAP (A fragments first, then B) of K step READ_KK of the tile at c.rd
+    // into (na, nb), and the load PLAN puts here, bound for c.fill.
+    template<int M, int READ_KK, class PLAN>
+    __device__ __forceinline__ static void slot(const step_ctx& c,
+                                                const u32x4 (&fa)[TM],
+                                                const u32x4 (&fb)[TN],
+                                                u32x4 (&na)[TM],
+                                                u32x4 (&nb)[TN],
+                                                f32x4 (&acc)[TM][TN])
+    {
+        mfma_16x16x32_pinned<IN>(acc[M / TN][M % TN], fa[M / TN], fb[M % TN]);
+        if constexpr(M % FRAG_GAP == 0 && M / FRAG_GAP < FRAGS)
+        {
+            constexpr int U = M / FRAG_GAP;
+            if constexpr(U < TM)
+            {
+                na[U] = c.oa.template fragment_pinned<U, READ_KK>(c.rd);
+            }
+            else
+            {
+                nb[U - TM] = c.ob.template fragment_pinned<U - TM, READ_KK>(c.rd + A_BYTES);
+            }
+        }
+        if constexpr(PLAN::count > 0 && M >= PLAN::first && (M - PLAN::first) % PLAN::gap == 0
+                     && (M - PLAN::first) / PLAN::gap < PLAN::count)
+        {
+            issue_one(c.oa, c.ob, PLAN::begin + (M - PLAN::first) / PLAN::gap, c.a_src, c.b_src,
+                      c.fill, c.wave);
+        }
+    }
+
+    template<int READ_KK, class PLAN, int... M>
+    __device__ __forceinline__ static void slots(std::integer_sequence<int, M...>,
+                                                 const step_ctx& c,
+                                                 const u32x4 (&fa)[TM],
+                                                 const u32x4 (&fb)[TN],
+                                                 u32x4 (&na)[TM],
+                                                 u32x4 (&nb)[TN],
+                                                 f32x4 (&acc)[TM][TN])
+    {
+        (slot<M, READ_KK, PLAN>(c, fa, fb, na, nb, acc), ...);
+    }
+
+    // One K step: the MFMAs on (fa, fb) with the reads and loads between them.
+    template<int READ_KK, class PLAN>
+    __device__ __forceinline__ static void step(const step_ctx& c,
+                                                const u32x4 (&fa)[TM],
+                                                const u32x4 (&fb)[TN],
+                                                u32x4 (&na)[TM],
+                                                u32x4 (&nb)[TN],
+                                                f32x4 (&acc)[TM][TN])
+    {
+        __builtin_amdgcn_sched_barrier(0);
+        slots<READ_KK, PLAN>(
+            std::make_integer_sequence<int, MFMAS>{}, c, fa, fb, na, nb, acc);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // All fragments of K step 0 of the tile at LDS byte address rd.
+    template<int... I, int... J>
+    __device__ __forceinline__ static void read_first(std::integer_sequence<int, I...>,
+                                                      std::integer_sequence<int, J...>,
+                                                      const op_a&  oa,
+                                                      const op_b&  ob,
+                                                      unsigned int rd,
+                                                      u32x4 (&fa)[TM],
+                                                      u32x4 (&fb)[TN])
+    {
+        ((fa[I] = oa.template fragment_pinned<I, 0>(rd)), ...);
+        ((fb[J] = ob.template fragment_pinned<J, 0>(rd + A_BYTES)), ...);
+    }
+
+    __device__ static void run(const gemm_args& args)
+    {
+        __shared__ __attribute__((aligned(1024))) char lds_raw[LDS_BYTES];
+        lds_char_ptr lds = (lds_char_ptr)lds_raw;
+
+        const int tid    = threadIdx.x;
+        const int lane   = tid & 63;
+        const int wave   = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int wave_m = wave / WAVES_N;
+        const int wave_n = wave % WAVES_N;
+
+        const int tiles   = args.grid_m * args.grid_n;
+        const int slice   = blockIdx.x / tiles;
+        const int tile_id = blockIdx.x - slice * tiles;
+        const tile_coord t = map_tile(tile_id, args.grid_m, args.grid_n, args.group);
+        const int row0 = t.m * BM;
+        const int col0 = t.n * BN;
+
+        const int k_steps_total = args.K / BK;
+        const int steps_per     = (k_steps_total + args.k_slices - 1) / args.k_slices;
+        const int step_begin    = slice * steps_per;
+        int       step_end      = step_begin + steps_per;
+        if(step_end > k_steps_total)
+        {
+            step_end = k_steps_total;
+        }
+        const int nk = step_end - step_begin;
+
+        const long long batch = blockIdx.y;
+        const InT* A = static_cast<const InT*>(args.A) + batch * args.batch_stride_a;
+        const InT* B = static_cast<const InT*>(args.B) + batch * args.batch_stride_b;
+
+        const long long a_ld = args.lda;
+        const long long b_ld = args.ldb;
+        const long long a_sr = A_KMAJOR ? a_ld : 1, a_sk = A_KMAJOR ? 1 : a_ld;
+        const long long b_sr = B_KMAJOR ? b_ld : 1, b_sk = B_KMAJOR ? 1 : b_ld;
+
+        op_a oa;
+        op_b ob;
+        oa.init(wave, lane, a_ld, wave_m * WTM);
+        ob.init(wave, lane, b_ld, wave_n * WTN);
+
+        const InT* a_src = A + row0 * a_sr + (long long)step_begin * BK * a_sk;
+        const InT* b_src = B + col0 * b_sr + (long long)step_begin * BK * b_sk;
+        const long long a_step = BK * a_sk, b_step = BK * b_sk;
+
+        f32x4 acc[TM][TN];
+#pragma unroll
+        for(int i = 0; i < TM; ++i)
+        {
+#pragma unroll
+            for(int j = 0; j < TN; ++j)
+            {
+                acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+        }
+
+        if(nk > 0)
+        {
+            // Past the end of K the source pointers wrap to the first tile: the redundant
+            // loads land in stages nobody reads again and keep the number of loads in
+            // flight a compile-time constant.
+            const InT* const a_first = a_src;
+            const InT* const b_first = b_src;
+            const InT* const a_end   = a_src + (long long)nk * a_step;
+
+            u32x4 fa[2][TM], fb[2][TN];
+            const unsigned int lds_addr = (unsigned int)(size_t)lds;
+            auto advance = [&]() {
+                a_src += a_step;
+                b_src += b_step;
+                if(a_src == a_end)
+                {
+                    a_src = a_first;
+                    b_src = b_first;
+                }
+            };
+            // Ring of 2 tiles, two K steps per tile.  Tile t: first step on K step 0 with
+            // the reads of K step 1; then wait for the own loads of tile t+1 and the own
+            // reads of tile t, barrier; second step on K step 1 with the reads of tile
+            // t+1's K step 0.  Tile t's stage is free from that barrier on: the loads of
+            // tile t+2 go out under the second step (three quarters of them) and the
+            // first quarter of tile t+1's first step.
+            constexpr int LOADS_A = VM_LOADS / 4, LOADS_B = VM_LOADS - LOADS_A;
+            using plan_b = load_plan<2, (MFMAS - 2) / LOADS_B, 0, LOADS_B>;
+            using plan_a = load_plan<1, 4, LOADS_B, LOADS_A>;
+            // prologue: tile 0 and the first part of tile 1 on their way, tile 0 landed
+#pragma unroll
+            for(int v = 0; v < VM_LOADS; ++v)
+            {
+                issue_one(oa, ob, v, a_src, b_src, lds, wave);
+            }
+            advance();
+#pragma unroll
+            for(int v = 0; v < LOADS_B; ++v)
+            {
+                issue_one(oa, ob, v, a_src, b_src, lds + STAGE, wave);
+            }
+            const InT* a_prev = a_src;
+            const InT* b_prev = b_src;
+            advance();
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(LOADS_B));
+            __builtin_amdgcn_s_barrier();
+            read_first(std::make_integer_sequence<int, TM>{}, std::make_integer_sequence<int, TN>{},
+                       oa, ob, lds_addr, fa[0], fb[0]);
+            for(int it = 0; it < nk; ++it)
+            {
+                const step_ctx c0{oa, ob, lds_addr + (it & 1) * STAGE, lds + ((it + 1) & 1) * STAGE,
+                                  wave, a_prev, b_prev};
+                const step_ctx c1{oa, ob, lds_addr + ((it + 1) & 1) * STAGE, lds + (it & 1) * STAGE,
+                                  wave, a_src, b_src};
+                __builtin_amdgcn_s_waitcnt(waitcnt_imm(63)); // last step's fragment reads
+                step<1, plan_a>(c0, fa[0], fb[0], fa[1], fb[1], acc);
+                __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+                __builtin_amdgcn_s_barrier();
+                step<0, plan_b>(c1, fa[1], fb[1], fa[0], fb[0], acc);
+                a_prev = a_src;
+                b_prev = b_src;
+                advance();
+            }
+            // redundant tail loads and reads may still be in flight; the MFMAs are
+            // invisible to the compiler, so cover their result latency by hand
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+        }
+
+        if(args.k_slices == 1)
+        {
+            OutT* C = static_cast<OutT*>(args.C) + batch * args.batch_stride_c;
+            write_out<MI, GUARD_C>(
+                acc, C, args.M, args.N, row0 + wave_m * WTM, col0 + wave_n * WTN, lane);
+        }
+        else
+        {
+            float* P = args.partials
+                       + ((long long)batch * args.k_slices + slice) * (long long)args.M * args.N;
+            write_out<MI, GUARD_C>(
+                acc, P, args.M, args.N, row0 + wave_m * WTM, col0 + wave_n * WTN, lane);
+        }
+    }
+};
+
+} // namespace device
+} // namespace rocm_wmma_gemm
+
+#endif // ROCM_WMMA_GEMM_SOLO_KERNEL_HPP

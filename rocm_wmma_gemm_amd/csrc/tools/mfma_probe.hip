@@ -408,6 +408,59 @@ __global__ void __launch_bounds__(256) mfma_with_stream(const char* src, size_t 
 }
 
 
+// ---- 6b. ds_read_b128 with only some lanes active (address < 0 = lane sits out) -----
+template<bool B64>
+__global__ void __launch_bounds__(512) lds_pattern_masked(const int* lane_addr, float* out, int iters)
+{
+    __shared__ u32x4 lds[4096]; // 64 KiB
+    for(int i = threadIdx.x; i < 4096; i += blockDim.x)
+    {
+        lds[i] = u32x4{1u, 2u, 3u, 4u};
+    }
+    __syncthreads();
+    const int      la   = lane_addr[threadIdx.x & 63];
+    const unsigned addr = (unsigned)la + (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    if(la >= 0)
+    {
+        for(int it = 0; it < iters; ++it)
+        {
+            u32x4 v[8];
+            if constexpr(B64)
+            {
+                uint2 w[8];
+                asm volatile(
+                    "ds_read_b64_tr_b16 %0, %8\n ds_read_b64_tr_b16 %1, %8 offset:4096\n"
+                    "ds_read_b64_tr_b16 %2, %8 offset:8192\n ds_read_b64_tr_b16 %3, %8 offset:12288\n"
+                    "ds_read_b64_tr_b16 %4, %8 offset:16384\n ds_read_b64_tr_b16 %5, %8 offset:20480\n"
+                    "ds_read_b64_tr_b16 %6, %8 offset:24576\n ds_read_b64_tr_b16 %7, %8 offset:28672\n"
+                    "s_waitcnt lgkmcnt(0)"
+                    : "=&v"(w[0]), "=&v"(w[1]), "=&v"(w[2]), "=&v"(w[3]), "=&v"(w[4]), "=&v"(w[5]),
+                      "=&v"(w[6]), "=&v"(w[7])
+                    : "v"(addr));
+                for(int i = 0; i < 8; ++i)
+                    v[i] = u32x4{w[i].x, w[i].y, 0u, 0u};
+            }
+            else
+            {
+                asm volatile(
+                    "ds_read_b128 %0, %8\n ds_read_b128 %1, %8 offset:4096\n"
+                    "ds_read_b128 %2, %8 offset:8192\n ds_read_b128 %3, %8 offset:12288\n"
+                    "ds_read_b128 %4, %8 offset:16384\n ds_read_b128 %5, %8 offset:20480\n"
+                    "ds_read_b128 %6, %8 offset:24576\n ds_read_b128 %7, %8 offset:28672\n"
+                    "s_waitcnt lgkmcnt(0)"
+                    : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]),
+                      "=&v"(v[6]), "=&v"(v[7])
+                    : "v"(addr));
+            }
+            for(int i = 0; i < 8; ++i)
+                acc ^= v[i];
+        }
+    }
+    if(acc.x == 0x12345u)
+        out[0] = 1.0f;
+}
+
 // ---- 9. MFMA shape vs sustained rate on pseudo-random operands ----------------------
 // SHAPE 0: v_mfma_f32_32x32x16_f16 (16 accumulator registers per instruction),
 // SHAPE 1: v_mfma_f32_16x16x32_f16 (4 accumulator registers per instruction).
@@ -535,6 +588,7 @@ int main(int argc, char** argv)
 {
     bool   dump     = false;
     bool   ceiling  = false;
+    bool   lds_groups = false;
     size_t copy_mib = 0;
     for(int i = 1; i < argc; ++i)
     {
@@ -542,6 +596,8 @@ int main(int argc, char** argv)
             dump = true;
         if(!std::strcmp(argv[i], "--ceiling"))
             ceiling = true;
+        if(!std::strcmp(argv[i], "--lds-groups"))
+            lds_groups = true;
         if(!std::strcmp(argv[i], "--copy") && i + 1 < argc)
             copy_mib = std::strtoull(argv[++i], nullptr, 10);
     }
@@ -579,6 +635,136 @@ int main(int argc, char** argv)
         float        clk[3];
         CHECK(hipMemcpy(clk, dOut, 12, hipMemcpyDeviceToHost));
         std::printf("ceiling %.1f %.0f\n", tf, clk[2] > 0 ? clk[1] / clk[2] * 100.0 : 0.0);
+        return 0;
+    }
+
+    if(lds_groups)
+    {
+        // Which lanes of a ds_read_b128 are served in the same LDS cycle, and which
+        // address bits pick the bank: start from the conflict-free pattern lane*16 and
+        // move ONE lane j onto another row of lane 0's 16-byte column (experiment 1), or
+        // move lane 1 to byte offset X of another row (experiment 2); a slower run means
+        // the two lanes met in one cycle on one bank.
+        int*   dAddr;
+        float* dOut;
+        CHECK(hipMalloc(&dAddr, 256));
+        CHECK(hipMalloc(&dOut, 4));
+        const int iters = 3000, blocks = prop.multiProcessorCount;
+        auto run = [&](const std::vector<int>& addr) {
+            CHECK(hipMemcpy(dAddr, addr.data(), 256, hipMemcpyHostToDevice));
+            lds_pattern<false><<<blocks, 512>>>(dAddr, dOut, 100);
+            CHECK(hipDeviceSynchronize());
+            CHECK(hipEventRecord(e0));
+            lds_pattern<false><<<blocks, 512>>>(dAddr, dOut, iters);
+            CHECK(hipEventRecord(e1));
+            CHECK(hipEventSynchronize(e1));
+            return time_ms(e0, e1);
+        };
+        auto run_masked = [&](const std::vector<int>& addr) {
+            CHECK(hipMemcpy(dAddr, addr.data(), 256, hipMemcpyHostToDevice));
+            lds_pattern_masked<false><<<blocks, 512>>>(dAddr, dOut, 100);
+            CHECK(hipDeviceSynchronize());
+            CHECK(hipEventRecord(e0));
+            lds_pattern_masked<false><<<blocks, 512>>>(dAddr, dOut, iters);
+            CHECK(hipEventRecord(e1));
+            CHECK(hipEventSynchronize(e1));
+            return time_ms(e0, e1);
+        };
+        (void)run;
+        // Experiment 1: lanes i and j alone, same 16-byte bank column, different rows.
+        for(int i : {0, 8, 16, 32})
+        {
+            std::vector<int> one(64, -1);
+            one[i]         = 0;
+            const float t1 = run_masked(one);
+            std::printf("lanes %d and j active on one bank column (time relative to lane %d alone, %.3f ms):\n", i, i, t1);
+            for(int j = 0; j < 64; ++j)
+            {
+                if(j == i)
+                {
+                    std::printf("  --:----%s", j % 8 == 7 ? "\n" : "");
+                    continue;
+                }
+                std::vector<int> a(64, -1);
+                a[i] = 0;
+                a[j] = 2048;
+                std::printf("  %2d:%.2f%s", j, run_masked(a) / t1, j % 8 == 7 ? "\n" : "");
+            }
+        }
+        // Experiment 2: lanes 0 and 1 alone; lane 0 at byte 0, lane 1 at byte X.
+        {
+            std::vector<int> one(64, -1);
+            one[0]         = 0;
+            const float t1 = run_masked(one);
+            std::printf("lane 0 at byte 0, lane 1 at byte X (relative time):\n");
+            int n = 0;
+            for(int x : {16, 32, 64, 128, 256, 512, 1024, 2048, 4096, 8192, 256 + 16, 512 + 16, 1024 + 16, 2048 + 16, 4096 + 16, 128 + 256, 128 + 512, 64 + 1024})
+            {
+                std::vector<int> a(64, -1);
+                a[0] = 0;
+                a[1] = x;
+                std::printf("  %5d:%.2f%s", x, run_masked(a) / t1, ++n % 6 == 0 ? "\n" : "");
+            }
+            std::printf("\n");
+        }
+        // Experiment 1b/2b: the same for ds_read_b64_tr_b16 (8 bytes per lane)
+        auto run_masked64 = [&](const std::vector<int>& addr) {
+            CHECK(hipMemcpy(dAddr, addr.data(), 256, hipMemcpyHostToDevice));
+            lds_pattern_masked<true><<<blocks, 512>>>(dAddr, dOut, 100);
+            CHECK(hipDeviceSynchronize());
+            CHECK(hipEventRecord(e0));
+            lds_pattern_masked<true><<<blocks, 512>>>(dAddr, dOut, iters);
+            CHECK(hipEventRecord(e1));
+            CHECK(hipEventSynchronize(e1));
+            return time_ms(e0, e1);
+        };
+        for(int i : {0, 16, 32})
+        {
+            std::vector<int> one(64, -1);
+            one[i]         = 0;
+            const float t1 = run_masked64(one);
+            std::printf("b64_tr: lanes %d and j active on one 8-byte bank column (relative to lane %d alone, %.3f ms):\n", i, i, t1);
+            for(int j = 0; j < 64; ++j)
+            {
+                if(j == i)
+                {
+                    std::printf("  --:----%s", j % 8 == 7 ? "\n" : "");
+                    continue;
+                }
+                std::vector<int> a(64, -1);
+                a[i] = 0;
+                a[j] = 2048;
+                std::printf("  %2d:%.2f%s", j, run_masked64(a) / t1, j % 8 == 7 ? "\n" : "");
+            }
+        }
+        {
+            std::vector<int> one(64, -1);
+            one[0]         = 0;
+            const float t1 = run_masked64(one);
+            std::printf("b64_tr: lane 0 at byte 0, lane 1 at byte X (relative time):\n");
+            int n = 0;
+            for(int x : {8, 16, 32, 64, 128, 256, 512, 1024, 2048, 4096, 256 + 8, 512 + 8, 2048 + 8, 128 + 256})
+            {
+                std::vector<int> a(64, -1);
+                a[0] = 0;
+                a[1] = x;
+                std::printf("  %5d:%.2f%s", x, run_masked64(a) / t1, ++n % 7 == 0 ? "\n" : "");
+            }
+            std::printf("\n");
+        }
+        // Experiment 3: how many lanes of a 16-lane block can run before time goes up
+        {
+            std::printf("lanes 0..n-1 active at lane*16 (ms):");
+            for(int n : {1, 2, 4, 8, 16, 24, 32, 48, 64})
+            {
+                std::vector<int> a(64, -1);
+                for(int l = 0; l < n; ++l)
+                    a[l] = l * 16;
+                std::printf("  %d:%.3f", n, run_masked(a));
+            }
+            std::printf("\n");
+        }
+        std::printf("\n");
         return 0;
     }
 
@@ -711,6 +897,12 @@ int main(int argc, char** argv)
             {"b128 slot = c ^ ((r>>1)&7)", false, [](int l) { int r = l % 32, c = l / 32; return r * 128 + ((c ^ ((r >> 1) & 7)) * 16); }},
             {"b128 slot = c ^ (r&7) ^ ((r>>3)&1)", false, [](int l) { int r = l % 32, c = l / 32; return r * 128 + ((c ^ (r & 7) ^ ((r >> 3) & 1)) * 16); }},
             {"b128 row*64 (BK=32), slot = c ^ ((r>>1)&3)", false, [](int l) { int r = l % 32, c = l / 32; return r * 64 + ((c ^ ((r >> 1) & 3)) * 16); }},
+            {"b128 16x16x32: row*128, slot = g ^ ((r>>1)&7)", false, [](int l) { int r = l % 16, g = l / 16; return r * 128 + ((g ^ ((r >> 1) & 7)) * 16); }},
+            {"b128 16x16x32: row*64, slot = g ^ ((r>>2)&3)", false, [](int l) { int r = l % 16, g = l / 16; return r * 64 + ((g ^ ((r >> 2) & 3)) * 16); }},
+            {"b128 16 lanes linear, groups 4096 B apart", false, [](int l) { return (l % 16) * 16 + (l / 16) * 4096; }},
+            {"b128 16 lanes linear, groups 256 B apart", false, [](int l) { return (l % 16) * 16 + (l / 16) * 256; }},
+            {"b128 16x16x32: row*128, slot = (g + 4*(r&1)) ^ (r>>1)", false, [](int l) { int r = l % 16, g = l / 16; return r * 128 + (((g + 4 * (r & 1)) ^ ((r >> 1) & 7)) * 16); }},
+            {"b128 16x16x32: row*128, slot = (2g) ^ (r>>1), +16B odd g", false, [](int l) { int r = l % 16, g = l / 16; return r * 128 + (((2 * (g & 1) + (g >> 1)) ^ ((r >> 1) & 7)) * 16); }},
             {"tr64 linear lane*8", true, [](int l) { return l * 8; }},
             {"tr64 [k][m] rows of 512 B, no swizzle", true, [](int l) { int b = l / 16, s = l % 16; return (8 * (b / 2) + s / 4) * 512 + (16 * (b % 2) + (s % 4) * 4) * 2; }},
             {"tr64 4k x 128m blocks, chunk ^ 4j", true, [](int l) { int b = l / 16, s = l % 16, j = s / 4; int mm = 16 * (b % 2) + (s % 4) * 4; int c = mm / 8; return (2 * (b / 2)) * 2048 + (j * 16 + (c ^ (4 * j))) * 16 + (mm % 8) * 2; }},

@@ -179,7 +179,12 @@ def test_every_variant_and_split_k_agree_with_oracle(loader):
                         A, B = make_inputs(M, N, K, la, lb, din, seed_a=7, seed_b=8)
                         gpu = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout,
                                       variant=(v.index, 4, split_k))
-                        check_against_oracle(gpu, A, B, M, N, K, lc, la, lb, din, dout)
+                        try:
+                            check_against_oracle(gpu, A, B, M, N, K, lc, la, lb, din, dout)
+                        except AssertionError as e:
+                            raise AssertionError(
+                                f"variant {v.index} split_k {split_k} {M}x{N}x{K} layouts "
+                                f"C{lc} A{la} B{lb} {tname}: {e}") from None
 
 
 def test_degenerate_arguments(loader):
