@@ -32,6 +32,8 @@
 #ifndef ROCM_WMMA_GEMM_PINGPONG_KERNEL_HPP
 #define ROCM_WMMA_GEMM_PINGPONG_KERNEL_HPP
 
+#include <utility>
+
 #include "direct_kernel.hpp"
 
 namespace rocm_wmma_gemm
@@ -82,10 +84,28 @@ struct pingpong_gemm
         return (vmcnt & 15) | (7 << 4) | (0 << 8) | ((vmcnt >> 4) << 14);
     }
 
+    // All MFMA operands of the tile at LDS byte address `stage`, as pinned reads (see
+    // direct_operand::fragment_pinned): the s_waitcnt at the end of the memory
+    // interval covers them, and the compiler does not put a wait for all outstanding
+    // global -> LDS loads in front of them.
+    template<int... X, int... Y>
+    __device__ __forceinline__ static void read_fragments(std::integer_sequence<int, X...>,
+                                                          std::integer_sequence<int, Y...>,
+                                                          const op_a&  oa,
+                                                          const op_b&  ob,
+                                                          unsigned int stage,
+                                                          u32x4 (&fa)[KK][TM],
+                                                          u32x4 (&fb)[KK][TN])
+    {
+        ((fa[X / TM][X % TM] = oa.template fragment_pinned<X % TM, X / TM>(stage)), ...);
+        ((fb[Y / TN][Y % TN] = ob.template fragment_pinned<Y % TN, Y / TN>(stage + A_BYTES)), ...);
+    }
+
     __device__ static void run(const gemm_args& args)
     {
         __shared__ __attribute__((aligned(1024))) char lds_raw[LDS_BYTES];
-        lds_char_ptr lds = (lds_char_ptr)lds_raw;
+        lds_char_ptr       lds      = (lds_char_ptr)lds_raw;
+        const unsigned int lds_addr = (unsigned int)(size_t)lds;
 
         const int tid     = threadIdx.x;
         const int lane    = tid & 63;
@@ -171,23 +191,11 @@ struct pingpong_gemm
             u32x4 fa[KK][TM], fb[KK][TN];
             for(int u = 0; u < nk; ++u)
             {
-                lds_char_ptr cur  = lds + (u & (STAGES - 1)) * STAGE;
                 lds_char_ptr fill = lds + ((u + STAGES - 1) & (STAGES - 1)) * STAGE;
                 // ---- MEM(u)
-#pragma unroll
-                for(int kk = 0; kk < KK; ++kk)
-                {
-#pragma unroll
-                    for(int i = 0; i < TM; ++i)
-                    {
-                        fa[kk][i] = oa.fragment(cur, i, kk);
-                    }
-#pragma unroll
-                    for(int j = 0; j < TN; ++j)
-                    {
-                        fb[kk][j] = ob.fragment(cur + A_BYTES, j, kk);
-                    }
-                }
+                read_fragments(std::make_integer_sequence<int, KK * TM>{},
+                               std::make_integer_sequence<int, KK * TN>{}, oa, ob,
+                               lds_addr + (u & (STAGES - 1)) * STAGE, fa, fb);
                 oa.issue(a_src, fill, wave);
                 ob.issue(b_src, fill + A_BYTES, wave);
                 a_src = a_src + a_step > a_last ? a_last : a_src + a_step;

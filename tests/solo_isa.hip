@@ -1,0 +1,9 @@
+// Instantiates the hand-scheduled kernel for a few type/layout/guard combinations so
+// that the host test can look at the generated assembly (see test_host.py).
+#include "kernel_table.hpp"
+
+using namespace rocm_wmma_gemm;
+
+template __global__ void device::gemm_entry<device::solo_gemm<device::in_kind::f16, _Float16, true, true, 256, 256, 64, 2, 2, 2, false>>(device::gemm_args);
+template __global__ void device::gemm_entry<device::solo_gemm<device::in_kind::bf16, float, false, false, 256, 256, 64, 2, 2, 2, true>>(device::gemm_args);
+template __global__ void device::gemm_entry<device::solo_gemm<device::in_kind::f16, _Float16, true, false, 256, 256, 64, 2, 2, 2, false>>(device::gemm_args);

@@ -148,3 +148,57 @@ def test_shipped_json_matches_reference_schema():
         assert set(conf["layout"]) == {"A", "B", "C"}
         assert all(v in ("row_major", "col_major") for v in conf["layout"].values())
         assert {"warps_m", "warps_n", "warp_tile_m", "warp_tile_n", "swizzle", "bits"} <= set(conf["config"])
+
+
+def _mfma_loops(asm_text):
+    """(function, [lines]) for every loop (label .. backward branch to it) that holds an MFMA."""
+    out = []
+    func = None
+    lines = asm_text.split("\n")
+    label_at = {}
+    for n, line in enumerate(lines):
+        m = re.match(r"^(_Z\w+):", line)
+        if m:
+            func = m.group(1)
+            label_at = {}
+            continue
+        m = re.match(r"^(\.LBB\w+):", line)
+        if m:
+            label_at[m.group(1)] = n
+            continue
+        m = re.match(r"^\s+s_cbranch_\w+\s+(\.LBB\w+)", line)
+        if m and m.group(1) in label_at:
+            body = lines[label_at[m.group(1)]:n]
+            if any("v_mfma" in b for b in body):
+                out.append((func, body))
+    return out
+
+
+def test_hand_scheduled_kernel_keeps_accumulators_in_place(tmp_path):
+    """The one-wave-per-SIMD kernel issues its MFMAs as inline assembly, so the compiler
+    does not know when their results become readable.  That is safe only while it never
+    touches an accumulator between them: the MFMA loops must hold no accumulator
+    copies and no spills, and the first accumulator read after the last MFMA must sit
+    behind the explicit wait states."""
+    hipcc = "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not found")
+    asm = tmp_path / "solo_isa.s"
+    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature",
+           "-Xclang", "-packed-fp32-ops", "-I" + os.path.join(ROOT, "rocm_wmma_gemm_amd", "csrc"),
+           "-S", "--cuda-device-only", "-o", str(asm), os.path.join(ROOT, "tests", "solo_isa.hip")]
+    subprocess.run(cmd, check=True, capture_output=True, timeout=600)
+    text = asm.read_text()
+    loops = [(f, body) for f, body in _mfma_loops(text) if "solo_gemm" in f]
+    assert len(loops) == 3, "one MFMA loop per instantiated kernel expected"
+    for func, body in loops:
+        assert sum("v_mfma_f32_16x16x32" in b for b in body) == 128
+        bad = [b for b in body if re.search(r"v_accvgpr_|scratch_", b)]
+        assert not bad, f"{func}: accumulator traffic or spills inside the MFMA loop: {bad[:3]}"
+    # after the last MFMA of each kernel: two s_nop 15 before anything names an AGPR
+    for func in {f for f, _ in loops}:
+        body = text[text.index(func + ":"):]
+        body = body[:body.index(".Lfunc_end")]
+        tail = body[body.rindex("v_mfma"):].split("\n")
+        first_use = next(i for i, b in enumerate(tail) if i > 0 and re.search(r"[ ,]a\[?\d", b))
+        assert sum("s_nop 15" in b for b in tail[:first_use]) >= 2, func
