@@ -189,14 +189,22 @@ def test_hand_scheduled_kernel_keeps_accumulators_in_place(tmp_path):
            "-S", "--cuda-device-only", "-o", str(asm), os.path.join(ROOT, "tests", "solo_isa.hip")]
     subprocess.run(cmd, check=True, capture_output=True, timeout=600)
     text = asm.read_text()
-    loops = [(f, body) for f, body in _mfma_loops(text) if "solo_gemm" in f]
-    assert len(loops) == 3, "one MFMA loop per instantiated kernel expected"
-    for func, body in loops:
-        assert sum("v_mfma_f32_16x16x32" in b for b in body) == 128
+    loops = {}
+    for f, body in _mfma_loops(text):
+        # cold blocks laid out after the function body also branch backwards; the real
+        # loop is the shortest span that holds MFMAs
+        if "solo_gemm" in f and (f not in loops or len(body) < len(loops[f])):
+            loops[f] = body
+    assert len(loops) == 3, "an MFMA loop in each instantiated kernel expected"
+    for func, body in loops.items():
+        whole = text[text.index(func + ":"):]
+        whole = whole[:whole.index(".Lfunc_end")]
+        assert sum("v_mfma_f32_16x16x32" in b for b in body) == whole.count("v_mfma_f32_16x16x32") == 128, \
+            f"{func}: MFMAs outside the main loop (peeled or duplicated code)"
         bad = [b for b in body if re.search(r"v_accvgpr_|scratch_", b)]
         assert not bad, f"{func}: accumulator traffic or spills inside the MFMA loop: {bad[:3]}"
     # after the last MFMA of each kernel: two s_nop 15 before anything names an AGPR
-    for func in {f for f, _ in loops}:
+    for func in loops:
         body = text[text.index(func + ":"):]
         body = body[:body.index(".Lfunc_end")]
         tail = body[body.rindex("v_mfma"):].split("\n")
