@@ -74,13 +74,15 @@ int rocm_wmma_gemm_variant_info_get(int variant, rocm_wmma_gemm_variant_info* in
 
 /* Which variant the dispatcher would pick for this problem (the table built from
  * gemm_config_gfx950_*.json, then shape heuristics).  type_idx as above.
- * Also reports the swizzle (tile-row group height) and split-K factor. Returns the
- * variant index, or -1 for invalid arguments. */
+ * Also reports the swizzle (tile-row group height) and the split field: s > 1 = every
+ * tile's K range is cut into s slices; -s < -1 = only the tiles of the last, partial
+ * wave over the compute units are cut into s slices; 1 = no split.  Returns the variant
+ * index, or -1 for invalid arguments. */
 int rocm_wmma_gemm_select(size_t M, size_t N, size_t K, int type_idx, int layout_c, int layout_a,
                           int layout_b, int* swizzle, int* split_k);
 
 /* Same computation as the four entry points above, but with the tile variant,
- * swizzle and split-K factor forced (tuner hook).  Returns 0 on success, -1 if the
+ * swizzle and split field (see above) forced (tuner hook).  Returns 0 on success, -1 if the
  * variant cannot run this problem, -2 for invalid arguments. */
 int rocm_wmma_gemm_run_variant(int type_idx, int variant, int swizzle, int split_k, void* C,
                                void* A, void* B, size_t M, size_t N, size_t K,

@@ -28,6 +28,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.normpath(os.path.join(HERE, "..", "..")))
 
 LAYOUT_NAME = {0: "row_major", 1: "col_major"}
+CUS = 256  # compute units of an MI355X
 DEFAULT_SHAPES = [
     # the reference's tuned sizes (gemm_config_gfx1100_f16.json)
     (1024, 1024, 1024), (2048, 2048, 2048), (2048, 5120, 5120), (4096, 2048, 64),
@@ -39,6 +40,8 @@ DEFAULT_SHAPES = [
     (128, 8192, 8192), (4095, 5121, 3001), (1000, 1000, 1000), (1024, 1024, 65536),
     # small shapes of the parity suite
     (128, 128, 128), (256, 256, 256), (512, 512, 512),
+    # square sizes whose tile count does not divide by the CU count
+    (1536, 1536, 1536), (3072, 3072, 3072), (6144, 6144, 6144),
 ]
 
 
@@ -56,9 +59,13 @@ def key_of(entry: dict):
 
 
 def config_json(v, swizzle: int, split_k: int) -> dict:
-    return {"warps_m": v.warps_m, "warps_n": v.warps_n, "warp_tile_m": v.warp_tile_m,
-            "warp_tile_n": v.warp_tile_n, "swizzle": swizzle, "bits": 128,
-            "block_k": v.block_k, "pipeline": v.pipeline, "split_k": split_k}
+    """split_k as the library's hook takes it: s > 1 every tile split, -s only the tail wave."""
+    cfg = {"warps_m": v.warps_m, "warps_n": v.warps_n, "warp_tile_m": v.warp_tile_m,
+           "warp_tile_n": v.warp_tile_n, "swizzle": swizzle, "bits": 128,
+           "block_k": v.block_k, "pipeline": v.pipeline, "split_k": max(split_k, 1)}
+    if split_k < -1:
+        cfg["tail_split"] = -split_k
+    return cfg
 
 
 def candidates(variants, M, N, K, lc):
@@ -77,6 +84,12 @@ def candidates(variants, M, N, K, lc):
             for s in (2, 4, 8, 16, 32):
                 if tiles * s <= 2048 and k_steps // s >= 4:
                     splits.append(s)
+        # more tiles than CUs and a thin last wave: split only that wave (negative = tail)
+        tail = tiles % CUS
+        if tiles > CUS and 0 < tail <= CUS * 3 // 4 and k_steps >= 16:
+            for s in (2, 3, 4, 6, 8):
+                if tail * s <= CUS * 5 // 4 and k_steps // s >= 4:
+                    splits.append(-s)
         for sw in swizzles:
             for sk in splits:
                 out.append((v, sw, sk))

@@ -24,7 +24,7 @@ struct launch_plan
 {
     int variant; // index into the compiled variant table
     int swizzle; // tile-row band height of the tile map
-    int split_k; // K slices (1 = off)
+    int split_k; // K slices (1 = off); -s = split only the last, partial wave of tiles s ways
 };
 
 struct tuned_entry

@@ -7,6 +7,7 @@
 #include <rocm_wmma_gemm_c.h>
 
 #include <algorithm>
+#include <atomic>
 #include <mutex>
 #include <stdexcept>
 #include <string>
@@ -167,6 +168,27 @@ kernel_problem to_kernel_space(void* C, void* A, void* B, size_t M, size_t N, si
     return p;
 }
 
+// CUs of the current device (cached per device), 0 if unknown.
+size_t compute_units_of_current_device()
+{
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+    {
+        return 0;
+    }
+    int cus = cached[dev].load(std::memory_order_relaxed);
+    if(cus == 0)
+    {
+        if(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+        {
+            return 0;
+        }
+        cached[dev].store(cus, std::memory_order_relaxed);
+    }
+    return static_cast<size_t>(cus);
+}
+
 int pick_mode(const kernel_problem& p, const variant_desc& v, int split_k)
 {
     const bool batch_ok = p.batch == 1 || ((p.stride_a % 8 == 0) && (p.stride_b % 8 == 0));
@@ -308,23 +330,51 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         throw std::runtime_error("rocm_wmma_gemm: tile grid too large");
     }
 
-    int       split_k = plan.split_k < 1 ? 1 : plan.split_k;
-    const int k_steps = static_cast<int>((k_kernel + v.block_k - 1) / v.block_k);
+    // plan.split_k > 1: every tile is split (few tiles, long K).  plan.split_k < -1: only
+    // the tiles of the last, partial wave over the CUs are split, -split_k ways, so that
+    // their workgroups fill the machine too (tiles that do not divide by the CU count
+    // otherwise leave most CUs idle for a whole tile time at the end).
+    const int k_steps     = static_cast<int>((k_kernel + v.block_k - 1) / v.block_k);
+    const size_t tiles    = grid_m * grid_n;
+    size_t    tail_begin  = 0; // first split tile
+    int       split_k     = 1;
+    if(plan.split_k > 1)
+    {
+        split_k = plan.split_k;
+    }
+    else if(plan.split_k < -1)
+    {
+        const size_t cus = compute_units_of_current_device();
+        if(cus > 0 && tiles > cus && tiles % cus != 0)
+        {
+            tail_begin = tiles / cus * cus;
+            split_k    = -plan.split_k;
+        }
+    }
     if(split_k > k_steps)
     {
         split_k = k_steps;
     }
-    if(grid_m * grid_n * static_cast<size_t>(split_k) > 0x7fffffffull)
+    const size_t split_tiles = tiles - tail_begin;
+    if(tail_begin + split_tiles * static_cast<size_t>(split_k) > 0x7fffffffull)
     {
         split_k = 1;
     }
+    // fp32 partial sums of one batch entry: whole planes when every tile is split, else
+    // one block_m x block_n tile per split tile and slice
+    const size_t plane_bytes = tail_begin == 0
+                                   ? p.M * p.N * sizeof(float)
+                                   : split_tiles * v.block_m * v.block_n * sizeof(float);
     // Batches per launch: bounded by grid.y and, under split-K, by a 1 GiB budget for
-    // the partial planes.
-    const size_t plane_bytes        = p.M * p.N * sizeof(float);
-    size_t       batches_per_launch = std::min<size_t>(p.batch, 65535);
+    // the partial sums.
+    size_t batches_per_launch = std::min<size_t>(p.batch, 65535);
     while(split_k > 1 && plane_bytes * split_k > (size_t{1} << 30))
     {
         --split_k;
+    }
+    if(split_k == 1)
+    {
+        tail_begin = 0;
     }
     if(split_k > 1)
     {
@@ -351,7 +401,8 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
                 }
                 return launch<OutT>(type_idx, retry, p, stream);
             }
-            split_k = 1;
+            split_k    = 1;
+            tail_begin = 0;
         }
     }
     float* partials = split_k > 1 ? reinterpret_cast<float*>(workspace + pack_bytes) : nullptr;
@@ -412,17 +463,29 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         args.grid_n         = static_cast<int>(grid_n);
         args.group          = plan.swizzle < 1 ? 1 : plan.swizzle;
         args.k_slices       = split_k;
+        args.tail_begin     = static_cast<int>(tail_begin);
         args.partials       = partials;
 
-        const dim3 grid(static_cast<unsigned>(grid_m * grid_n * split_k), static_cast<unsigned>(nb));
+        const dim3 grid(static_cast<unsigned>(tail_begin + (tiles - tail_begin) * split_k),
+                        static_cast<unsigned>(nb));
         fn<<<grid, dim3(v.threads), 0, stream>>>(args);
-        if(split_k > 1)
+        if(split_k > 1 && tail_begin == 0)
         {
             const long long plane  = static_cast<long long>(p.M) * static_cast<long long>(p.N);
             const int       blocks = static_cast<int>(std::min<long long>((plane + 255) / 256, 4096));
             device::reduce_partials<OutT>
                 <<<dim3(blocks, static_cast<unsigned>(nb)), dim3(256), 0, stream>>>(
                     static_cast<OutT*>(args.C), partials, plane, split_k, args.batch_stride_c);
+        }
+        else if(split_k > 1)
+        {
+            device::reduce_split_tiles<OutT>
+                <<<dim3(static_cast<unsigned>((tiles - tail_begin)
+                                              * (v.block_m * v.block_n / device::reduce_chunk_elems)),
+                        static_cast<unsigned>(nb)),
+                   dim3(256), 0, stream>>>(static_cast<OutT*>(args.C), partials, args.M, args.N, v.block_m, v.block_n,
+                             args.grid_m, args.grid_n, args.group, args.tail_begin, split_k,
+                             args.batch_stride_c);
         }
     }
     return 0;

@@ -236,10 +236,17 @@ __device__ __forceinline__ mfma_acc<MI> mfma_tile(u32x4 fa, u32x4 fb, mfma_acc<M
 }
 
 // Store this wave's accumulators to a row-major M x N matrix of DstT (C itself, or
-// one fp32 plane of split-K partial sums) whose wave tile starts at (row_w, col_w).
+// fp32 split-K partial sums) whose rows are `pitch` elements apart and whose wave tile
+// starts at (row_w, col_w); M and N bound the guarded stores.
 template<int MI, bool GUARD_C, int TM, int TN, class AccT, class DstT>
-__device__ __forceinline__ void write_out(
-const AccT (&acc)[TM][TN], DstT* D, int M, int N, int row_w, int col_w, int lane)
+__device__ __forceinline__ void write_out(const AccT (&acc)[TM][TN],
+                                          DstT*     D,
+                                          int       M,
+                                          int       N,
+                                          long long pitch,
+                                          int       row_w,
+                                          int       col_w,
+                                          int       lane)
 {
     if constexpr(MI == 32)
     {
@@ -259,7 +266,7 @@ const AccT (&acc)[TM][TN], DstT* D, int M, int N, int row_w, int col_w, int lane
                     const int row = row_w + i * 32 + 8 * (v / 4) + 4 * lane_hi + (v % 4);
                     if(!GUARD_C || (row < M && col < N))
                     {
-                        D[(long long)row * N + col] = to_out<DstT>(acc[i][j][v]);
+                        D[(long long)row * pitch + col] = to_out<DstT>(acc[i][j][v]);
                     }
                 }
             }
@@ -279,7 +286,7 @@ const AccT (&acc)[TM][TN], DstT* D, int M, int N, int row_w, int col_w, int lane
             for(int j = 0; j < TN; ++j)
             {
                 const int       col = col_w + j * 16 + 4 * g;
-                const long long at  = (long long)row * N + col;
+                const long long at  = (long long)row * pitch + col;
                 if constexpr(GUARD_C)
                 {
 #pragma unroll
@@ -509,15 +516,14 @@ struct direct_gemm
         const int wave_m  = wave / WAVES_N;
         const int wave_n  = wave % WAVES_N;
 
-        const int tiles   = args.grid_m * args.grid_n;
-        const int slice   = blockIdx.x / tiles;
-        const int tile_id = blockIdx.x - slice * tiles;
-        const tile_coord t = map_tile(tile_id, args.grid_m, args.grid_n, args.group);
+        const block_work w = decode_block(args);
+        const int slice    = w.slice;
+        const tile_coord t = map_tile(w.tile_id, args.grid_m, args.grid_n, args.group);
         const int row0 = t.m * BM;
         const int col0 = t.n * BN;
 
         const int k_steps_total = args.K / BK;
-        const int steps_per     = (k_steps_total + args.k_slices - 1) / args.k_slices;
+        const int steps_per     = (k_steps_total + w.slices - 1) / w.slices;
         const int step_begin    = slice * steps_per;
         int       step_end      = step_begin + steps_per;
         if(step_end > k_steps_total)
@@ -597,16 +603,17 @@ struct direct_gemm
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
         }
 
-        if(args.k_slices == 1)
+        if(w.slices == 1)
         {
             OutT* C = static_cast<OutT*>(args.C) + batch * args.batch_stride_c;
-            write_out<MI, GUARD_C>(acc, C, args.M, args.N, row0 + wave_m * WTM, col0 + wave_n * WTN, lane);
+            write_out<MI, GUARD_C>(acc, C, args.M, args.N, args.N, row0 + wave_m * WTM, col0 + wave_n * WTN, lane);
         }
         else
         {
-            float* P = args.partials
-                       + ((long long)batch * args.k_slices + slice) * (long long)args.M * args.N;
-            write_out<MI, GUARD_C>(acc, P, args.M, args.N, row0 + wave_m * WTM, col0 + wave_n * WTN, lane);
+            long long pitch;
+            float*    P = partial_base<BM, BN>(args, w, batch, row0, col0, pitch);
+            write_out<MI, GUARD_C>(
+                acc, P, args.M, args.N, pitch, row0 + wave_m * WTM, col0 + wave_n * WTN, lane);
         }
     }
 };

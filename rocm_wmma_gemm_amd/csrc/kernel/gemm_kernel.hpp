@@ -62,9 +62,51 @@ struct gemm_args
     long long   batch_stride_a, batch_stride_b, batch_stride_c; // elements
     int         grid_m, grid_n; // tiles along M and N
     int         group; // tile-row band height of the tile map
-    int         k_slices; // split-K factor (1 = off)
-    float*      partials; // split-K workspace: [slice][M][N] fp32, or nullptr
+    int         k_slices; // split-K factor of the split tiles (1 = off)
+    int         tail_begin; // tiles [0, tail_begin) of the walk order run whole K, the rest are
+                            // split k_slices ways; 0 = every tile is split (plain split-K)
+    float*      partials; // split-K workspace, fp32, or nullptr.  tail_begin == 0:
+                          // [batch][slice][M][N] planes; else [batch][split tile][slice][BM][BN]
 };
+
+// What one workgroup works on.  blockIdx.x enumerates the whole tiles first, then
+// (slice, split tile) pairs, slices outermost.
+struct block_work
+{
+    int tile_id; // position in the tile walk (see map_tile)
+    int slice, slices; // K slice of this workgroup and how many the tile has (1 = whole K)
+};
+
+__device__ __forceinline__ block_work decode_block(const gemm_args& args)
+{
+    const int b = blockIdx.x;
+    if(b < args.tail_begin || args.k_slices == 1)
+    {
+        return {b, 0, 1};
+    }
+    const int split_tiles = args.grid_m * args.grid_n - args.tail_begin;
+    const int r           = b - args.tail_begin;
+    const int slice       = r / split_tiles;
+    return {args.tail_begin + (r - slice * split_tiles), slice, args.k_slices};
+}
+
+// Where a split workgroup's fp32 partial tile goes: a pointer P and a row pitch such
+// that element (row, col) of C (global coordinates) is P[row * pitch + col].
+template<int BM, int BN>
+__device__ __forceinline__ float* partial_base(
+    const gemm_args& args, const block_work& w, long long batch, int row0, int col0, long long& pitch)
+{
+    if(args.tail_begin == 0)
+    {
+        pitch = args.N;
+        return args.partials + (batch * args.k_slices + w.slice) * (long long)args.M * args.N;
+    }
+    const long long split_tiles = args.grid_m * args.grid_n - args.tail_begin;
+    const long long t           = w.tile_id - args.tail_begin;
+    pitch                       = BN;
+    return args.partials + ((batch * split_tiles + t) * args.k_slices + w.slice) * (long long)(BM * BN)
+           - ((long long)row0 * BN + col0);
+}
 
 template<in_kind IN>
 __device__ __forceinline__ f32x16 mfma_32x32x16(u32x4 a, u32x4 b, f32x16 c)
@@ -413,17 +455,16 @@ struct staged_gemm
         const int lane_lo = lane & 31;
         const int lane_hi = lane >> 5;
 
-        // blockIdx.x enumerates (k slice, tile); blockIdx.y the batch entry.
-        const int tiles   = args.grid_m * args.grid_n;
-        const int slice   = blockIdx.x / tiles;
-        const int tile_id = blockIdx.x - slice * tiles;
-        const tile_coord t = map_tile(tile_id, args.grid_m, args.grid_n, args.group);
+        // blockIdx.x enumerates tiles and K slices; blockIdx.y the batch entry.
+        const block_work w = decode_block(args);
+        const int slice    = w.slice;
+        const tile_coord t = map_tile(w.tile_id, args.grid_m, args.grid_n, args.group);
         const int row0 = t.m * BM;
         const int col0 = t.n * BN;
 
         // K range of this slice, in whole BK steps.
         const int k_steps_total = (args.K + BK - 1) / BK;
-        const int steps_per     = (k_steps_total + args.k_slices - 1) / args.k_slices;
+        const int steps_per     = (k_steps_total + w.slices - 1) / w.slices;
         const int step_begin    = slice * steps_per;
         int       step_end      = step_begin + steps_per;
         if(step_end > k_steps_total)
@@ -502,7 +543,7 @@ struct staged_gemm
         // Epilogue.  Accumulator register v of a 32x32 tile holds row
         // 8*(v/4) + 4*(lane/32) + v%4 and column lane%32.
         const bool guarded = MODE != load_mode::vec_unguarded;
-        if(args.k_slices == 1)
+        if(w.slices == 1)
         {
             OutT* C = static_cast<OutT*>(args.C) + batch * args.batch_stride_c;
 #pragma unroll
@@ -528,8 +569,8 @@ struct staged_gemm
         else
         {
             // split-K: fp32 partial sums, reduced by a second kernel.
-            float* P = args.partials
-                       + ((long long)batch * args.k_slices + slice) * (long long)args.M * args.N;
+            long long pitch;
+            float*    P = partial_base<BM, BN>(args, w, batch, row0, col0, pitch);
 #pragma unroll
             for(int i = 0; i < TM; ++i)
             {
@@ -544,7 +585,7 @@ struct staged_gemm
                             = row0 + wave_m * WTM + i * 32 + 8 * (v / 4) + 4 * lane_hi + (v % 4);
                         if(!guarded || (row < args.M && col < args.N))
                         {
-                            P[(long long)row * args.N + col] = acc[i][j][v];
+                            P[(long long)row * pitch + col] = acc[i][j][v];
                         }
                     }
                 }
@@ -580,6 +621,68 @@ __global__ void __launch_bounds__(256) reduce_partials(OutT* __restrict__ C,
             s += P[k * plane + i];
         }
         out[i] = to_out<OutT>(s);
+    }
+}
+
+// The same for the compact layout of a split tail (gemm_args::tail_begin > 0): a
+// workgroup sums k_slices partial values for 4096 consecutive elements of one split
+// tile (blockIdx.x = tile * chunks + chunk) and writes those that lie inside C.  Few
+// tiles are split, so the work is cut fine enough to spread over the CUs and each
+// thread keeps 4 independent 16-byte loads per slice in flight.
+constexpr int reduce_chunk_elems = 4096;
+
+template<class OutT>
+__global__ void __launch_bounds__(256) reduce_split_tiles(OutT* __restrict__ C,
+                                                          const float* __restrict__ partials,
+                                                          int       M,
+                                                          int       N,
+                                                          int       block_m,
+                                                          int       block_n,
+                                                          int       grid_m,
+                                                          int       grid_n,
+                                                          int       group,
+                                                          int       tail_begin,
+                                                          int       k_slices,
+                                                          long long batch_stride_c)
+{
+    const long long  batch       = blockIdx.y;
+    const long long  split_tiles = grid_m * grid_n - tail_begin;
+    const int        elems       = block_m * block_n;
+    const int        chunks      = elems / reduce_chunk_elems;
+    const int        tile        = blockIdx.x / chunks;
+    const int        chunk       = blockIdx.x - tile * chunks;
+    const tile_coord t           = map_tile(tail_begin + tile, grid_m, grid_n, group);
+    const int        row0 = t.m * block_m, col0 = t.n * block_n;
+    const float*     P   = partials + (batch * split_tiles + tile) * k_slices * (long long)elems;
+    OutT*            out = C + batch * batch_stride_c;
+    f32x4            s[4];
+#pragma unroll
+    for(int u = 0; u < 4; ++u)
+    {
+        s[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    const int e0 = chunk * reduce_chunk_elems + threadIdx.x * 4;
+    for(int k = 0; k < k_slices; ++k)
+    {
+#pragma unroll
+        for(int u = 0; u < 4; ++u)
+        {
+            s[u] += *reinterpret_cast<const f32x4*>(P + (long long)k * elems + e0 + u * 1024);
+        }
+    }
+#pragma unroll
+    for(int u = 0; u < 4; ++u)
+    {
+        const int e   = e0 + u * 1024;
+        const int row = row0 + e / block_n, col = col0 + e % block_n; // block_n % 4 == 0
+#pragma unroll
+        for(int v = 0; v < 4; ++v)
+        {
+            if(row < M && col + v < N)
+            {
+                out[(long long)row * N + col + v] = to_out<OutT>(s[u][v]);
+            }
+        }
     }
 }
 

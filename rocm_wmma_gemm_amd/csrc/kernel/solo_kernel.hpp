@@ -305,15 +305,14 @@ struct solo_gemm
         const int wave_m = wave / WAVES_N;
         const int wave_n = wave % WAVES_N;
 
-        const int tiles   = args.grid_m * args.grid_n;
-        const int slice   = blockIdx.x / tiles;
-        const int tile_id = blockIdx.x - slice * tiles;
-        const tile_coord t = map_tile(tile_id, args.grid_m, args.grid_n, args.group);
+        const block_work w = decode_block(args);
+        const int slice    = w.slice;
+        const tile_coord t = map_tile(w.tile_id, args.grid_m, args.grid_n, args.group);
         const int row0 = t.m * BM;
         const int col0 = t.n * BN;
 
         const int k_steps_total = args.K / BK;
-        const int steps_per     = (k_steps_total + args.k_slices - 1) / args.k_slices;
+        const int steps_per     = (k_steps_total + w.slices - 1) / w.slices;
         const int step_begin    = slice * steps_per;
         int       step_end      = step_begin + steps_per;
         if(step_end > k_steps_total)
@@ -419,7 +418,7 @@ struct solo_gemm
             asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
         }
 
-        if(args.k_slices == 1)
+        if(w.slices == 1)
         {
             OutT* C = static_cast<OutT*>(args.C) + batch * args.batch_stride_c;
             if constexpr(sizeof(OutT) == 2 && !GUARD_C)
@@ -433,15 +432,15 @@ struct solo_gemm
             else
             {
                 write_out<MI, GUARD_C>(
-                    acc, C, args.M, args.N, row0 + wave_m * WTM, col0 + wave_n * WTN, lane);
+                    acc, C, args.M, args.N, args.N, row0 + wave_m * WTM, col0 + wave_n * WTN, lane);
             }
         }
         else
         {
-            float* P = args.partials
-                       + ((long long)batch * args.k_slices + slice) * (long long)args.M * args.N;
+            long long pitch;
+            float*    P = partial_base<BM, BN>(args, w, batch, row0, col0, pitch);
             write_out<MI, GUARD_C>(
-                acc, P, args.M, args.N, row0 + wave_m * WTM, col0 + wave_n * WTN, lane);
+                acc, P, args.M, args.N, pitch, row0 + wave_m * WTM, col0 + wave_n * WTN, lane);
         }
     }
 };

@@ -287,22 +287,36 @@ int main(int argc, char** argv)
                         lay.c_str(), sel_var, sel_sk, med, mn, tf, 100.0 * tf / peak_tf);
             std::fflush(stdout);
 #ifdef WITH_ROCBLAS
-            if(with_rocblas && blas && batch == 1 && lc == 1)
+            if(with_rocblas && blas && batch == 1)
             {
                 // rocBLAS is column-major: C(col) = op(A) op(B); a row-major operand is
-                // the transpose of a column-major one.
+                // the transpose of a column-major one.  A row-major C (M x N) is the
+                // column-major N x M matrix C^T = B^T A^T: same buffers, operands swapped.
                 rocblas_set_stream(blas, stream);
                 const rocblas_datatype in_t = bf16 ? rocblas_datatype_bf16_r : rocblas_datatype_f16_r;
                 const rocblas_datatype out_t
                     = c_is_32 ? rocblas_datatype_f32_r : in_t;
                 const float alpha = 1.0f, beta = 0.0f;
-                const rocblas_operation ta = la ? rocblas_operation_none : rocblas_operation_transpose;
-                const rocblas_operation tb = lb ? rocblas_operation_none : rocblas_operation_transpose;
+                // as a column-major matrix: A is M x K (ld M) if col-major, else K x M (ld K)
                 const rocblas_int lda = la ? sh.m : sh.k, ldb = lb ? sh.k : sh.n;
                 auto blas_call = [&]() {
-                    rocblas_gemm_ex(blas, ta, tb, sh.m, sh.n, sh.k, &alpha, A, in_t, lda, B, in_t,
-                                    ldb, &beta, C, out_t, sh.m, C, out_t, sh.m,
-                                    rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+                    if(lc == 1)
+                    {
+                        const rocblas_operation ta = la ? rocblas_operation_none : rocblas_operation_transpose;
+                        const rocblas_operation tb = lb ? rocblas_operation_none : rocblas_operation_transpose;
+                        rocblas_gemm_ex(blas, ta, tb, sh.m, sh.n, sh.k, &alpha, A, in_t, lda, B, in_t,
+                                        ldb, &beta, C, out_t, sh.m, C, out_t, sh.m,
+                                        rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+                    }
+                    else
+                    {
+                        // C^T (N x M, ld N) = op(B) op(A) with op(B) = B^T (N x K), op(A) = A^T (K x M)
+                        const rocblas_operation tb = lb ? rocblas_operation_transpose : rocblas_operation_none;
+                        const rocblas_operation ta = la ? rocblas_operation_transpose : rocblas_operation_none;
+                        rocblas_gemm_ex(blas, tb, ta, sh.n, sh.m, sh.k, &alpha, B, in_t, ldb, A, in_t,
+                                        lda, &beta, C, out_t, sh.n, C, out_t, sh.n,
+                                        rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+                    }
                 };
                 for(int w = 0; w < warmup; ++w)
                     blas_call();

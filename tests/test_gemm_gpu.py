@@ -187,6 +187,34 @@ def test_every_variant_and_split_k_agree_with_oracle(loader):
                                 f"C{lc} A{la} B{lb} {tname}: {e}") from None
 
 
+def test_split_tail_wave_agrees_with_oracle(loader):
+    """Negative split field: only the tiles of the last, partial wave over the 256 CUs are
+    cut along K (compact partial tiles + their own reduce kernel).  Shapes with more
+    tiles than CUs for both tile sizes, whole and ragged, every pipeline."""
+    by_tile = {}
+    for v in loader.variants():
+        by_tile.setdefault((v.block_m, v.block_n, v.pipeline), v)
+    cases = []
+    for (bm, bn, pipe), v in sorted(by_tile.items()):
+        if (bm, bn) == (256, 256):
+            cases += [(v, 4352, 4352, 256), (v, 4300, 4400, 264)]   # 17 x 17 and 17 x 18 tiles
+        elif (bm, bn) == (128, 128):
+            cases += [(v, 2304, 2304, 256), (v, 2200, 2310, 200)]   # 18 x 18 and 18 x 19 tiles
+    assert cases
+    for v, M, N, K in cases:
+        for split in (-2, -3):
+            for (lc, la, lb) in [(0, 0, 1), (1, 1, 0)]:
+                din, dout = TYPE_PAIRS["f16_f16" if split == -2 else "f32_bf16"]
+                A, B = make_inputs(M, N, K, la, lb, din, seed_a=3, seed_b=4)
+                gpu = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout,
+                              variant=(v.index, 4, split))
+                try:
+                    check_against_oracle(gpu, A, B, M, N, K, lc, la, lb, din, dout)
+                except AssertionError as e:
+                    raise AssertionError(f"variant {v.index} split {split} {M}x{N}x{K} layouts "
+                                         f"C{lc} A{la} B{lb}: {e}") from None
+
+
 def test_degenerate_arguments(loader):
     import torch
 

@@ -166,7 +166,7 @@ def _mfma_loops(asm_text):
         if m:
             label_at[m.group(1)] = n
             continue
-        m = re.match(r"^\s+s_cbranch_\w+\s+(\.LBB\w+)", line)
+        m = re.match(r"^\s+s_c?branch\w*\s+(\.LBB\w+)", line)
         if m and m.group(1) in label_at:
             body = lines[label_at[m.group(1)]:n]
             if any("v_mfma" in b for b in body):
