@@ -18,8 +18,7 @@
 // K-contiguous rows are 128 bytes, so every load fetches whole cache lines).  The
 // fragments of the next K step are always read one step ahead, so the stage of the
 // tile being multiplied is free for the next loads as soon as all waves have passed
-// the barrier in the middle of the tile.  Loads of tiles past the end of K are skipped
-// (a uniform branch per load).  Measured with the shader clock on 8192^3:
+// the barrier in the middle of the tile.  Measured with the shader clock on 8192^3:
 // 1117 + 1186 cycles for the two steps of a tile (1024 each would be MFMA-bound) plus
 // about 70 in the wait and the barrier, where issuing a tile's loads back to back
 // had cost 1700-1900 cycles for the second step.
@@ -157,7 +156,6 @@ struct solo_gemm
         int          wave;
         const InT*   a_src;
         const InT*   b_src;
-        bool         loads_on; // false once the tile the loads would fetch is past the end of K
     };
 
     // Which loads of a tile a step issues: loads BEGIN .. BEGIN+COUNT-1 (A's loads come
@@ -200,11 +198,8 @@ struct solo_gemm
         if constexpr(PLAN::count > 0 && M >= PLAN::first && (M - PLAN::first) % PLAN::gap == 0
                      && (M - PLAN::first) / PLAN::gap < PLAN::count)
         {
-            if(c.loads_on)
-            {
-                issue_one(c.oa, c.ob, PLAN::begin + (M - PLAN::first) / PLAN::gap, c.a_src, c.b_src,
-                          c.fill, c.wave);
-            }
+            issue_one(c.oa, c.ob, PLAN::begin + (M - PLAN::first) / PLAN::gap, c.a_src, c.b_src,
+                      c.fill, c.wave);
         }
     }
 
@@ -354,9 +349,25 @@ struct solo_gemm
         {
             u32x4 fa[2][TM], fb[2][TN];
             const unsigned int lds_addr = (unsigned int)(size_t)lds;
+            // Past the end of K the source pointers wrap to the first tile, so the last two
+            // tiles' worth of loads fetch K tiles 0 and 1 again into stages nobody reads.
+            // That keeps the loop uniform, and it is kept on purpose: switching those loads
+            // off (tried with a branch per load and with a zero-sized buffer descriptor)
+            // made back-to-back calls on the same operands 5 % slower at 4096^3, because
+            // the 32 workgroups of an XCD leave exactly the first two K tiles of their
+            // operand panels in its 4 MiB L2 for the next call; a call on fresh operands
+            // pays 2 of K/64 tiles of extra L2 -> LDS traffic for nothing.
+            const InT* const a_first = a_src;
+            const InT* const b_first = b_src;
+            const InT* const a_end   = a_src + (long long)nk * a_step;
             auto advance = [&]() {
                 a_src += a_step;
                 b_src += b_step;
+                if(a_src == a_end)
+                {
+                    a_src = a_first;
+                    b_src = b_first;
+                }
             };
             // Ring of 2 tiles, two K steps per tile.  Tile t: first step on K step 0 with
             // the reads of K step 1; then wait for the own loads of tile t+1 and the own
@@ -374,34 +385,24 @@ struct solo_gemm
                 issue_one(oa, ob, v, a_src, b_src, lds, wave);
             }
             advance();
-            if(nk > 1)
-            {
 #pragma unroll
-                for(int v = 0; v < LOADS_B; ++v)
-                {
-                    issue_one(oa, ob, v, a_src, b_src, lds + STAGE, wave);
-                }
+            for(int v = 0; v < LOADS_B; ++v)
+            {
+                issue_one(oa, ob, v, a_src, b_src, lds + STAGE, wave);
             }
             const InT* a_prev = a_src;
             const InT* b_prev = b_src;
             advance();
-            if(nk > 1)
-            {
-                __builtin_amdgcn_s_waitcnt(waitcnt_imm(LOADS_B));
-            }
-            else
-            {
-                __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
-            }
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(LOADS_B));
             __builtin_amdgcn_s_barrier();
             read_first(std::make_integer_sequence<int, TM>{}, std::make_integer_sequence<int, TN>{},
                        oa, ob, lds_addr, fa[0], fb[0]);
             for(int it = 0; it < nk; ++it)
             {
                 const step_ctx c0{oa, ob, lds_addr + (it & 1) * STAGE, lds + ((it + 1) & 1) * STAGE,
-                                  wave, a_prev, b_prev, it + 1 < nk};
+                                  wave, a_prev, b_prev};
                 const step_ctx c1{oa, ob, lds_addr + ((it + 1) & 1) * STAGE, lds + (it & 1) * STAGE,
-                                  wave, a_src, b_src, it + 2 < nk};
+                                  wave, a_src, b_src};
                 __builtin_amdgcn_s_waitcnt(waitcnt_imm(63)); // last step's fragment reads
                 step<1, plan_a>(c0, fa[0], fb[0], fa[1], fb[1], acc);
                 __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
@@ -411,9 +412,9 @@ struct solo_gemm
                 b_prev = b_src;
                 advance();
             }
-            // the last fragment reads (of a tile that does not exist) may still be in
-            // flight; the MFMAs are invisible to the compiler, so cover their result
-            // latency by hand
+            // the wrapped tail loads and the last fragment reads may still be in flight;
+            // the MFMAs are invisible to the compiler, so cover their result latency by
+            // hand
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
             asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
         }
