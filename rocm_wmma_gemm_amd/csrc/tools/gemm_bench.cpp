@@ -6,6 +6,10 @@
 //              [--variant V --swizzle S --split_k K]   force one compiled variant
 //              [--rocblas]                             also time rocblas_gemm_ex
 //              [--data cyclic|random]
+//              [--names]   also print each result under the reference's benchmark name,
+//                          "{A:m_layout::...,B:...,C:...,m:M,n:N,k:K}/manual_time ...", in
+//                          the column order its report generator parses
+//                          (reference docs/generate_report.py:36-58)
 //
 // Measures what the reference's benchmarks measure (reference
 // benchmark/gemm/bench_half_half.cpp:78-114): hipEvent time around each enqueue,
@@ -148,6 +152,7 @@ int main(int argc, char** argv)
     int    reps = 20, warmup = 3, variant = -1, swizzle = 4, split_k = 1;
     size_t batch = 1;
     bool   with_rocblas = false;
+    bool   names        = false;
     for(int i = 1; i < argc; ++i)
     {
         auto next = [&](const char* flag) -> const char* {
@@ -181,6 +186,8 @@ int main(int argc, char** argv)
             data = next("--data");
         else if(a == "--rocblas")
             with_rocblas = true;
+        else if(a == "--names")
+            names = true;
         else
         {
             std::fprintf(stderr, "unknown argument %s\n", a.c_str());
@@ -285,6 +292,16 @@ int main(int argc, char** argv)
             std::snprintf(dims, sizeof dims, "%zu,%zu,%zu", sh.m, sh.n, sh.k);
             std::printf("%-10s %-22s %-4s %8d %6d %10.4f %10.4f %8.1f %7.1f%%\n", type.c_str(), dims,
                         lay.c_str(), sel_var, sel_sk, med, mn, tf, 100.0 * tf / peak_tf);
+            if(names)
+            {
+                // name/manual_time  time  cpu  iterations  avg_tflops  bytes_per_second
+                const double gib_s = ((double)(sh.m * sh.k + sh.k * sh.n) * 2 + (double)sh.m * sh.n * (c_is_32 ? 4 : 2))
+                                     * batch / (med * 1e-3) / (1024.0 * 1024.0 * 1024.0);
+                std::printf("{A:m_layout::%s,B:m_layout::%s,C:m_layout::%s,m:%zu,n:%zu,k:%zu}/manual_time"
+                            " %10.3f ms %10.3f ms %8d %10.4f %12.4fGi/s\n",
+                            la ? "col_major" : "row_major", lb ? "col_major" : "row_major",
+                            lc ? "col_major" : "row_major", sh.m, sh.n, sh.k, med, med, reps, tf, gib_s);
+            }
             std::fflush(stdout);
 #ifdef WITH_ROCBLAS
             if(with_rocblas && blas && batch == 1)
