@@ -99,63 +99,124 @@ struct solo_gemm
         return (vmcnt & 15) | (7 << 4) | (0 << 8) | ((vmcnt >> 4) << 14);
     }
 
-    // Wave-level load v of the tile (A's loads first, then B's), as a buffer load: the
-    // tile origin goes into a buffer descriptor in scalar registers and the lane's byte
-    // offset inside the tile is loop-invariant, so a load costs no vector ALU work
-    // (with a 64-bit address per lane it cost an add per load and twice the address
-    // traffic; measured 1-2 % in throughput at the power limit).
-    __device__ __forceinline__ static void issue_one(const op_a&  oa,
-                                                     const op_b&  ob,
-                                                     int          v,
-                                                     const InT*   a_src,
-                                                     const InT*   b_src,
-                                                     lds_char_ptr stage,
-                                                     int          wave)
+    // Addressing of one operand's global -> LDS loads.  Load i of a tile (i = 0 ..
+    // PER_WAVE-1; it fills the 1 KiB LDS block wave + i*WAVES) is a buffer load whose
+    // address is split three ways so that nothing is computed per load: the tile origin
+    // sits in the buffer descriptor (scalar registers, advanced once per tile), the
+    // part that depends on i is a scalar offset i * stride, and the lane's own part is
+    // a vector offset that is the same for every i (K-contiguous: the swizzle of row
+    // 8*(wave + 4i) + lane/8 does not depend on i) or alternates between two values
+    // with the parity of i (M/N-contiguous: the swizzle term 2*((kg/2)%2) does).
+    template<bool KMAJOR, int ROWS>
+    struct load_addr
     {
-        // dword 3 of the descriptor: 32-bit raw buffer; every tile span fits 32 bits
-        // (the host checks), so the range check never fires
-        constexpr int RSRC_FLAGS = 0x00020000;
-        if(v < op_a::PER_WAVE)
+        static_assert(WAVES == 4 && BK == 64 && (KMAJOR || ROWS == 256), "derived for this tile and wave count");
+        unsigned int voff[KMAJOR ? 1 : 2]; // bytes
+        unsigned int stride; // bytes between load i and load i+1
+
+        __device__ __forceinline__ void init(int wave, int lane, long long ld)
         {
-            const int t    = wave + v * WAVES;
-            auto      rsrc = __builtin_amdgcn_make_buffer_rsrc(
-                const_cast<InT*>(a_src), 0, 0xffffffff, RSRC_FLAGS);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                rsrc,
-                (__attribute__((address_space(3))) void*)(stage + t * 1024),
-                16,
-                (int)(oa.lane_off[v] * 2u),
-                0,
-                0,
-                RWG_LOAD_AUX);
+            if constexpr(KMAJOR)
+            {
+                constexpr int CH   = BK / 8;
+                const int     r    = 8 * wave + lane / CH; // row of load 0; load i adds 32 rows
+                const int     c    = (lane % CH) ^ swizzle_of_row<CH, MI>(r);
+                voff[0]            = (unsigned int)((r * ld + c * 8) * 2);
+                stride             = (unsigned int)(32 * ld * 2);
+            }
+            else
+            {
+                // block t = wave + 4i: k group kg = t/2 = wave/2 + 2i, 128-row half mh = wave%2
+                const int j = lane / 16, cphys = lane % 16;
+#pragma unroll
+                for(int p = 0; p < 2; ++p) // p = (kg/2) % 2 = i % 2
+                {
+                    const int c = cphys ^ (4 * j) ^ (2 * p);
+                    voff[p]     = (unsigned int)((((wave >> 1) * 4 + j) * ld + (wave & 1) * 128 + c * 8) * 2);
+                }
+                stride = (unsigned int)(8 * ld * 2);
+            }
+        }
+
+        template<int I>
+        __device__ __forceinline__ unsigned int vector_offset() const
+        {
+            return voff[KMAJOR ? 0 : (I & 1)];
+        }
+    };
+
+    using addr_a = load_addr<A_KMAJOR, BM>;
+    using addr_b = load_addr<B_KMAJOR, BN>;
+
+    // 128-bit buffer descriptor of a tile: base = its origin, no stride, no range check
+    // that could fire (every tile span fits 32 bits: the host checks), raw 32-bit format.
+    __device__ __forceinline__ static u32x4 descriptor(const InT* origin)
+    {
+        const unsigned long long p = (unsigned long long)origin;
+        return u32x4{(unsigned int)p, (unsigned int)(p >> 32) & 0xffffu, 0xffffffffu, 0x00020000u};
+    }
+
+    // One MFMA and, in its shadow, one global -> LDS load: M0 (the load's LDS
+    // destination) is written before the MFMA, which fills the wait state M0 needs
+    // before the load may use it.  lds_block = LDS byte address of this wave's block 0
+    // of the operand's stage; LDS_IMM = i * WAVES * 1024.
+    template<int LDS_IMM>
+    __device__ __forceinline__ static void mfma_and_load(f32x4&       acc,
+                                                         const u32x4& fa,
+                                                         const u32x4& fb,
+                                                         unsigned int lds_block,
+                                                         unsigned int voff,
+                                                         const u32x4& rsrc,
+                                                         unsigned int soff)
+    {
+        if constexpr(IN == in_kind::f16)
+        {
+            asm volatile("s_add_u32 m0, %[ldsb], %[imm]\n\t"
+                         "v_mfma_f32_16x16x32_f16 %[acc], %[b], %[a], %[acc]\n\t"
+                         "buffer_load_dwordx4 %[voff], %[rsrc], %[soff] offen lds"
+                         : [acc] "+a"(acc)
+                         : [b] "v"(fb), [a] "v"(fa), [ldsb] "s"(lds_block), [imm] "n"(LDS_IMM),
+                           [voff] "v"(voff), [rsrc] "s"(rsrc), [soff] "s"(soff)
+                         : "memory", "scc");
         }
         else
         {
-            const int w    = v - op_a::PER_WAVE;
-            const int t    = wave + w * WAVES;
-            auto      rsrc = __builtin_amdgcn_make_buffer_rsrc(
-                const_cast<InT*>(b_src), 0, 0xffffffff, RSRC_FLAGS);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                rsrc,
-                (__attribute__((address_space(3))) void*)(stage + A_BYTES + t * 1024),
-                16,
-                (int)(ob.lane_off[w] * 2u),
-                0,
-                0,
-                RWG_LOAD_AUX);
+            asm volatile("s_add_u32 m0, %[ldsb], %[imm]\n\t"
+                         "v_mfma_f32_16x16x32_bf16 %[acc], %[b], %[a], %[acc]\n\t"
+                         "buffer_load_dwordx4 %[voff], %[rsrc], %[soff] offen lds"
+                         : [acc] "+a"(acc)
+                         : [b] "v"(fb), [a] "v"(fa), [ldsb] "s"(lds_block), [imm] "n"(LDS_IMM),
+                           [voff] "v"(voff), [rsrc] "s"(rsrc), [soff] "s"(soff)
+                         : "memory", "scc");
         }
+    }
+
+    // A load on its own (prologue).
+    template<int LDS_IMM>
+    __device__ __forceinline__ static void load_only(unsigned int lds_block,
+                                                     unsigned int voff,
+                                                     const u32x4& rsrc,
+                                                     unsigned int soff)
+    {
+        asm volatile("s_add_u32 m0, %[ldsb], %[imm]\n\t"
+                     "s_nop 0\n\t"
+                     "buffer_load_dwordx4 %[voff], %[rsrc], %[soff] offen lds"
+                     :
+                     : [ldsb] "s"(lds_block), [imm] "n"(LDS_IMM), [voff] "v"(voff), [rsrc] "s"(rsrc),
+                       [soff] "s"(soff)
+                     : "memory", "scc");
     }
 
     // Everything a step works on.
     struct step_ctx
     {
-        const op_a&  oa;
-        const op_b&  ob;
-        unsigned int rd; // LDS byte address of the stage the fragments are read from
-        lds_char_ptr fill; // stage the loads go to
-        int          wave;
-        const InT*   a_src;
-        const InT*   b_src;
+        const op_a&   oa;
+        const op_b&   ob;
+        const addr_a& la;
+        const addr_b& lb;
+        unsigned int  rd; // LDS byte address of the stage the fragments are read from
+        unsigned int  fill; // LDS byte address of this wave's block 0 in the stage the loads go to
+        u32x4         rsrc_a, rsrc_b; // descriptors of the tile the loads fetch
     };
 
     // Which loads of a tile a step issues: loads BEGIN .. BEGIN+COUNT-1 (A's loads come
@@ -182,7 +243,30 @@ struct solo_gemm
                                                 u32x4 (&nb)[TN],
                                                 f32x4 (&acc)[TM][TN])
     {
-        mfma_16x16x32_pinned<IN>(acc[M / TN][M % TN], fa[M / TN], fb[M % TN]);
+        constexpr bool HAS_LOAD = PLAN::count > 0 && M >= PLAN::first
+                                  && (M - PLAN::first) % PLAN::gap == 0
+                                  && (M - PLAN::first) / PLAN::gap < PLAN::count;
+        if constexpr(HAS_LOAD)
+        {
+            constexpr int V = PLAN::begin + (M - PLAN::first) / PLAN::gap; // load of the tile
+            if constexpr(V < op_a::PER_WAVE)
+            {
+                mfma_and_load<V * WAVES * 1024>(acc[M / TN][M % TN], fa[M / TN], fb[M % TN], c.fill,
+                                                c.la.template vector_offset<V>(), c.rsrc_a,
+                                                V * c.la.stride);
+            }
+            else
+            {
+                constexpr int W = V - op_a::PER_WAVE;
+                mfma_and_load<A_BYTES + W * WAVES * 1024>(acc[M / TN][M % TN], fa[M / TN], fb[M % TN],
+                                                          c.fill, c.lb.template vector_offset<W>(),
+                                                          c.rsrc_b, W * c.lb.stride);
+            }
+        }
+        else
+        {
+            mfma_16x16x32_pinned<IN>(acc[M / TN][M % TN], fa[M / TN], fb[M % TN]);
+        }
         if constexpr(M % FRAG_GAP == 0 && M / FRAG_GAP < FRAGS)
         {
             constexpr int U = M / FRAG_GAP;
@@ -194,12 +278,6 @@ struct solo_gemm
             {
                 nb[U - TM] = c.ob.template fragment_pinned<U - TM, READ_KK>(c.rd + A_BYTES);
             }
-        }
-        if constexpr(PLAN::count > 0 && M >= PLAN::first && (M - PLAN::first) % PLAN::gap == 0
-                     && (M - PLAN::first) / PLAN::gap < PLAN::count)
-        {
-            issue_one(c.oa, c.ob, PLAN::begin + (M - PLAN::first) / PLAN::gap, c.a_src, c.b_src,
-                      c.fill, c.wave);
         }
     }
 
@@ -228,6 +306,31 @@ struct solo_gemm
         slots<READ_KK, PLAN>(
             std::make_integer_sequence<int, MFMAS>{}, c, fa, fb, na, nb, acc);
         __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // Loads V... of a tile without MFMAs around them (prologue).
+    template<int... V>
+    __device__ __forceinline__ static void issue_loads(std::integer_sequence<int, V...>,
+                                                       const addr_a& la,
+                                                       const addr_b& lb,
+                                                       unsigned int  fill,
+                                                       const u32x4&  rsrc_a,
+                                                       const u32x4&  rsrc_b)
+    {
+        (
+            [&] {
+                if constexpr(V < op_a::PER_WAVE)
+                {
+                    load_only<V * WAVES * 1024>(fill, la.template vector_offset<V>(), rsrc_a, V * la.stride);
+                }
+                else
+                {
+                    constexpr int W = V - op_a::PER_WAVE;
+                    load_only<A_BYTES + W * WAVES * 1024>(fill, lb.template vector_offset<W>(), rsrc_b,
+                                                          W * lb.stride);
+                }
+            }(),
+            ...);
     }
 
     // All fragments of K step 0 of the tile at LDS byte address rd.
@@ -378,18 +481,17 @@ struct solo_gemm
             constexpr int LOADS_A = VM_LOADS / 4, LOADS_B = VM_LOADS - LOADS_A;
             using plan_b = load_plan<2, (MFMAS - 2) / LOADS_B, 0, LOADS_B>;
             using plan_a = load_plan<1, 4, LOADS_B, LOADS_A>;
+            addr_a la;
+            addr_b lb;
+            la.init(wave, lane, a_ld);
+            lb.init(wave, lane, b_ld);
+            const unsigned int wave_block = lds_addr + wave * 1024; // this wave's block 0, stage 0
             // prologue: tile 0 and the first part of tile 1 on their way, tile 0 landed
-#pragma unroll
-            for(int v = 0; v < VM_LOADS; ++v)
-            {
-                issue_one(oa, ob, v, a_src, b_src, lds, wave);
-            }
+            issue_loads(std::make_integer_sequence<int, VM_LOADS>{}, la, lb, wave_block,
+                        descriptor(a_src), descriptor(b_src));
             advance();
-#pragma unroll
-            for(int v = 0; v < LOADS_B; ++v)
-            {
-                issue_one(oa, ob, v, a_src, b_src, lds + STAGE, wave);
-            }
+            issue_loads(std::make_integer_sequence<int, LOADS_B>{}, la, lb, wave_block + STAGE,
+                        descriptor(a_src), descriptor(b_src));
             const InT* a_prev = a_src;
             const InT* b_prev = b_src;
             advance();
@@ -399,10 +501,11 @@ struct solo_gemm
                        oa, ob, lds_addr, fa[0], fb[0]);
             for(int it = 0; it < nk; ++it)
             {
-                const step_ctx c0{oa, ob, lds_addr + (it & 1) * STAGE, lds + ((it + 1) & 1) * STAGE,
-                                  wave, a_prev, b_prev};
-                const step_ctx c1{oa, ob, lds_addr + ((it + 1) & 1) * STAGE, lds + (it & 1) * STAGE,
-                                  wave, a_src, b_src};
+                const step_ctx c0{oa, ob, la, lb, lds_addr + (it & 1) * STAGE,
+                                  wave_block + ((it + 1) & 1) * STAGE, descriptor(a_prev),
+                                  descriptor(b_prev)};
+                const step_ctx c1{oa, ob, la, lb, lds_addr + ((it + 1) & 1) * STAGE,
+                                  wave_block + (it & 1) * STAGE, descriptor(a_src), descriptor(b_src)};
                 __builtin_amdgcn_s_waitcnt(waitcnt_imm(63)); // last step's fragment reads
                 step<1, plan_a>(c0, fa[0], fb[0], fa[1], fb[1], acc);
                 __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
