@@ -351,10 +351,21 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
             split_k    = -plan.split_k;
         }
     }
-    if(split_k > k_steps)
-    {
-        split_k = k_steps;
-    }
+    // Slices hold ceil(k_steps / split_k) K steps each; keep only as many as are not
+    // empty (5 steps 4 ways is 2, 2, 1 and nothing for a fourth slice).
+    auto without_empty_slices = [k_steps](int slices) {
+        if(slices > k_steps)
+        {
+            slices = k_steps;
+        }
+        if(slices > 1)
+        {
+            const int per = (k_steps + slices - 1) / slices;
+            slices        = (k_steps + per - 1) / per;
+        }
+        return slices;
+    };
+    split_k = without_empty_slices(split_k);
     const size_t split_tiles = tiles - tail_begin;
     if(tail_begin + split_tiles * static_cast<size_t>(split_k) > 0x7fffffffull)
     {
@@ -370,7 +381,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
     size_t batches_per_launch = std::min<size_t>(p.batch, 65535);
     while(split_k > 1 && plane_bytes * split_k > (size_t{1} << 30))
     {
-        --split_k;
+        split_k = without_empty_slices(split_k - 1);
     }
     if(split_k == 1)
     {
@@ -380,6 +391,13 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
     {
         batches_per_launch
             = std::min(batches_per_launch, std::max<size_t>((size_t{1} << 30) / (plane_bytes * split_k), 1));
+    }
+    // A persistent kernel numbers its work items over the whole launch with an int.
+    const size_t blocks_per_batch = tail_begin + split_tiles * static_cast<size_t>(split_k);
+    const bool   persistent       = v.pipeline == 5;
+    if(persistent)
+    {
+        batches_per_launch = std::min(batches_per_launch, std::max<size_t>(0x7fffffffull / blocks_per_batch, 1));
     }
     const size_t partial_bytes = split_k > 1 ? plane_bytes * split_k * batches_per_launch : 0;
 
@@ -465,9 +483,17 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         args.k_slices       = split_k;
         args.tail_begin     = static_cast<int>(tail_begin);
         args.partials       = partials;
+        args.blocks_per_batch = static_cast<int>(blocks_per_batch);
+        args.batches          = static_cast<int>(nb);
 
-        const dim3 grid(static_cast<unsigned>(tail_begin + (tiles - tail_begin) * split_k),
-                        static_cast<unsigned>(nb));
+        dim3 grid(static_cast<unsigned>(blocks_per_batch), static_cast<unsigned>(nb));
+        if(persistent)
+        {
+            // one workgroup per CU (each takes a whole CU), striding over the work items
+            const size_t cus   = compute_units_of_current_device();
+            const size_t items = blocks_per_batch * nb;
+            grid               = dim3(static_cast<unsigned>(cus > 0 ? std::min(items, cus) : items), 1);
+        }
         fn<<<grid, dim3(v.threads), 0, stream>>>(args);
         if(split_k > 1 && tail_begin == 0)
         {

@@ -67,6 +67,8 @@ struct gemm_args
                             // split k_slices ways; 0 = every tile is split (plain split-K)
     float*      partials; // split-K workspace, fp32, or nullptr.  tail_begin == 0:
                           // [batch][slice][M][N] planes; else [batch][split tile][slice][BM][BN]
+    int         blocks_per_batch; // workgroups' worth of work per batch entry (whole tiles + slices)
+    int         batches; // batch entries of this launch; blocks_per_batch * batches fits an int
 };
 
 // What one workgroup works on.  blockIdx.x enumerates the whole tiles first, then
@@ -77,9 +79,8 @@ struct block_work
     int slice, slices; // K slice of this workgroup and how many the tile has (1 = whole K)
 };
 
-__device__ __forceinline__ block_work decode_block(const gemm_args& args)
+__device__ __forceinline__ block_work decode_block(const gemm_args& args, int b)
 {
-    const int b = blockIdx.x;
     if(b < args.tail_begin || args.k_slices == 1)
     {
         return {b, 0, 1};
@@ -88,6 +89,11 @@ __device__ __forceinline__ block_work decode_block(const gemm_args& args)
     const int r           = b - args.tail_begin;
     const int slice       = r / split_tiles;
     return {args.tail_begin + (r - slice * split_tiles), slice, args.k_slices};
+}
+
+__device__ __forceinline__ block_work decode_block(const gemm_args& args)
+{
+    return decode_block(args, (int)blockIdx.x);
 }
 
 // Where a split workgroup's fp32 partial tile goes: a pointer P and a row pitch such

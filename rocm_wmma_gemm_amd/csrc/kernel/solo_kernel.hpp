@@ -79,7 +79,7 @@ struct solo_gemm
     static constexpr int STAGE     = A_BYTES + B_BYTES;
     static constexpr int LDS_BYTES = STAGES * STAGE;
     static_assert(BK == 64 && STAGES == 2, "ring of 2 tiles of BLOCK_K 64");
-    static_assert(LDS_BYTES <= 160 * 1024, "tile ring does not fit the 160 KB LDS");
+    
 
     using op_a = direct_operand<A_KMAJOR, BM, BK, WTM, WAVES, MI>;
     using op_b = direct_operand<B_KMAJOR, BN, BK, WTN, WAVES, MI>;
@@ -347,54 +347,184 @@ struct solo_gemm
         ((fb[J] = ob.template fragment_pinned<J, 0>(rd + A_BYTES)), ...);
     }
 
-    // 16-bit C, whole tiles: the wave's rows go through a private LDS strip so that a
-    // store instruction writes 4 rows x 256 contiguous bytes (16 bytes per lane) instead
-    // of 16 rows x 32 bytes.  At 4096^3 the C stores are 11 % of the call.  Strip: 16 rows
+    // Whole tiles: the wave's rows go through a private LDS strip so that a store
+    // instruction writes 4 rows x 256 contiguous bytes (16 bytes per lane) instead of
+    // 16 rows x 32 bytes (16-bit C) or 16 rows x 64 bytes (fp32 C and partial sums; the
+    // strip is worth 6..9 % at 8192^3 and 13..16 % with shorter K there).  At 4096^3 the
+    // C stores are 11 % of the call.  STREAM marks the stores as streaming: C is not read
+    // again here, and without the hint the 4 MiB of C that the workgroups of an XCD write
+    // at the same time push the operand panels out of its L2 (+3..5 % with several tiles
+    // per workgroup, nothing lost with one).  Strip: 16 rows
     // at a pitch of 272 bytes (the 8-byte writes of a half-wave then fall on 32 distinct
     // 8-byte bank columns; the 16-byte reads take two cycles instead of one, which does
     // not show).  LDS operations of one wave are served in order, so the reads see the
     // writes without a barrier; the waits keep the compiler from reordering them.
     static constexpr int STRIP_PITCH = 272;
     static constexpr int STRIP_BYTES = 16 * STRIP_PITCH + 256; // rounded to 4608
-    static_assert(WAVES * STRIP_BYTES <= LDS_BYTES, "store strips must fit the tile ring");
+    static_assert(LDS_BYTES + WAVES * STRIP_BYTES <= 160 * 1024, "tile ring and store strips must fit the 160 KB LDS");
 
-    __device__ __forceinline__ static void write_out_staged(
-        const f32x4 (&acc)[TM][TN], OutT* C, int N, int row_w, int col_w, int lane, lds_char_ptr strip)
+    // Ties a row of accumulators to its registers at this point of the program: what
+    // follows reads the row from there.  Without it the compiler copies all 256
+    // accumulator registers into ordinary ones right behind the K loop, where there is
+    // no room for them, and spills.
+    __device__ __forceinline__ static void pin_row(f32x4 (&row)[TN])
     {
-        static_assert(sizeof(OutT) == 2 && TN == 8, "strip layout: 128 16-bit columns per wave");
-        typedef OutT out4 __attribute__((ext_vector_type(4)));
+        static_assert(TN == 8, "eight accumulators of a row per statement");
+        asm volatile(""
+                     : "+a"(row[0]), "+a"(row[1]), "+a"(row[2]), "+a"(row[3]), "+a"(row[4]), "+a"(row[5]),
+                       "+a"(row[6]), "+a"(row[7]));
+    }
+
+    template<bool STREAM, class DstT>
+    __device__ __forceinline__ static void write_out_staged(
+        f32x4 (&acc)[TM][TN], DstT* D, long long pitch, int row_w, int col_w, int lane, lds_char_ptr strip)
+    {
+        static_assert(TN == 8, "strip layout: 128 columns per wave");
+        // a strip row holds 256 bytes: all 128 columns of a 16-bit destination, 64 of fp32
+        constexpr int PASSES = sizeof(DstT) / 2;
+        constexpr int TILES  = TN / PASSES; // 16-column tiles per pass
+        typedef DstT out4 __attribute__((ext_vector_type(4)));
         using lds_out4 = __attribute__((address_space(3))) out4;
         using lds_u32x4 = __attribute__((address_space(3))) u32x4;
         const int r16 = lane & 15, g = lane >> 4;
 #pragma unroll
         for(int i = 0; i < TM; ++i)
         {
+            pin_row(acc[i]);
 #pragma unroll
-            for(int j = 0; j < TN; ++j)
+            for(int p = 0; p < PASSES; ++p)
             {
-                out4 o;
 #pragma unroll
-                for(int v = 0; v < 4; ++v)
+                for(int j = 0; j < TILES; ++j)
                 {
-                    o[v] = to_out<OutT>(acc[i][j][v]);
-                }
-                *reinterpret_cast<lds_out4*>(strip + r16 * STRIP_PITCH + (16 * j + 4 * g) * 2) = o;
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    out4 o;
 #pragma unroll
-            for(int q = 0; q < 4; ++q)
-            {
-                const int   row = 4 * q + g;
-                const u32x4 v   = *reinterpret_cast<lds_u32x4*>(strip + row * STRIP_PITCH + r16 * 16);
-                *reinterpret_cast<u32x4*>(C + (long long)(row_w + 16 * i + row) * N + col_w + r16 * 8) = v;
+                    for(int v = 0; v < 4; ++v)
+                    {
+                        o[v] = to_out<DstT>(acc[i][p * TILES + j][v]);
+                    }
+                    *reinterpret_cast<lds_out4*>(strip + r16 * STRIP_PITCH + (16 * j + 4 * g) * sizeof(DstT)) = o;
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+                for(int q = 0; q < 4; ++q)
+                {
+                    const int   row = 4 * q + g;
+                    const u32x4 v   = *reinterpret_cast<lds_u32x4*>(strip + row * STRIP_PITCH + r16 * 16);
+                    u32x4* const to = reinterpret_cast<u32x4*>(D + (long long)(row_w + 16 * i + row) * pitch + col_w
+                                                               + p * TILES * 16 + r16 * (16 / sizeof(DstT)));
+                    if constexpr(STREAM)
+                    {
+                        __builtin_nontemporal_store(v, to);
+                    }
+                    else
+                    {
+                        *to = v;
+                    }
+                }
+                asm volatile("" ::: "memory");
             }
-            asm volatile("" ::: "memory");
         }
     }
 
+    // One unit of work of a workgroup: a C tile (or one K slice of a split tile) of one
+    // batch entry.
+    struct work_item
+    {
+        block_work w;
+        int        batch;
+        int        row0, col0;
+        int        nk; // K tiles; the host never creates an empty slice
+        const InT* a; // first K tile of the operands
+        const InT* b;
+    };
+
+    __device__ __forceinline__ static work_item decode(const gemm_args& args, int v)
+    {
+        work_item x;
+        x.batch            = v / args.blocks_per_batch;
+        x.w                = decode_block(args, v - x.batch * args.blocks_per_batch);
+        const tile_coord t = map_tile(x.w.tile_id, args.grid_m, args.grid_n, args.group);
+        x.row0             = t.m * BM;
+        x.col0             = t.n * BN;
+
+        const int k_steps_total = args.K / BK;
+        const int steps_per     = (k_steps_total + x.w.slices - 1) / x.w.slices;
+        const int step_begin    = x.w.slice * steps_per;
+        int       step_end      = step_begin + steps_per;
+        if(step_end > k_steps_total)
+        {
+            step_end = k_steps_total;
+        }
+        x.nk = step_end - step_begin;
+
+        const long long a_sr = A_KMAJOR ? args.lda : 1, a_sk = A_KMAJOR ? 1 : args.lda;
+        const long long b_sr = B_KMAJOR ? args.ldb : 1, b_sk = B_KMAJOR ? 1 : args.ldb;
+        x.a = static_cast<const InT*>(args.A) + x.batch * args.batch_stride_a + x.row0 * a_sr
+              + (long long)step_begin * BK * a_sk;
+        x.b = static_cast<const InT*>(args.B) + x.batch * args.batch_stride_b + x.col0 * b_sr
+              + (long long)step_begin * BK * b_sk;
+        return x;
+    }
+
+    // The accumulators of a finished work item, to C or to the fp32 partial tiles.
+    __device__ __forceinline__ static void write_item(const gemm_args&   args,
+                                                      const work_item&   x,
+                                                      f32x4 (&acc)[TM][TN],
+                                                      int                row_w,
+                                                      int                col_w,
+                                                      int                lane,
+                                                      lds_char_ptr       strip)
+    {
+        if(x.w.slices == 1)
+        {
+            OutT* C = static_cast<OutT*>(args.C) + x.batch * args.batch_stride_c;
+            if constexpr(!GUARD_C)
+            {
+                write_out_staged<true>(acc, C, args.N, x.row0 + row_w, x.col0 + col_w, lane, strip);
+            }
+            else
+            {
+                write_out<MI, GUARD_C>(acc, C, args.M, args.N, args.N, x.row0 + row_w, x.col0 + col_w, lane);
+            }
+        }
+        else
+        {
+            long long pitch;
+            float*    P = partial_base<BM, BN>(args, x.w, x.batch, x.row0, x.col0, pitch);
+            if constexpr(!GUARD_C)
+            {
+                // the reduce kernel reads these next: no streaming hint
+                write_out_staged<false>(acc, P, pitch, x.row0 + row_w, x.col0 + col_w, lane, strip);
+            }
+            else
+            {
+                write_out<MI, GUARD_C>(acc, P, args.M, args.N, pitch, x.row0 + row_w, x.col0 + col_w, lane);
+            }
+        }
+    }
+
+    // Makes the zeroed accumulators safe to feed to the hand-written MFMAs: the compiler
+    // does not see that those read them, so it would not keep the wait states between
+    // the writes and the first read.
+    __device__ __forceinline__ static void settle_row(f32x4 (&row)[TN])
+    {
+        static_assert(TN == 8, "eight accumulators of a row per statement");
+        asm volatile("s_nop 4"
+                     : "+a"(row[0]), "+a"(row[1]), "+a"(row[2]), "+a"(row[3]), "+a"(row[4]), "+a"(row[5]),
+                       "+a"(row[6]), "+a"(row[7]));
+    }
+
+    // The workgroups are persistent: workgroup g works on items g, g + gridDim.x, ... of
+    // the launch, and the K tiles of all its items form ONE stream through the ring, so
+    // the loads of an item's first two K tiles go out under the last two steps of the
+    // item before it and the only thing between two items' MFMAs is the store of the
+    // accumulators.  (A workgroup per item pays, per item, the dispatch of the next
+    // workgroup, the latency of the first loads and the drain of the stores: about
+    // 13 us, nine K tiles' worth, at 256 x 256 x 64.)
     __device__ static void run(const gemm_args& args)
     {
-        __shared__ __attribute__((aligned(1024))) char lds_raw[LDS_BYTES];
+        __shared__ __attribute__((aligned(1024))) char lds_raw[LDS_BYTES + WAVES * STRIP_BYTES];
         lds_char_ptr lds = (lds_char_ptr)lds_raw;
 
         const int tid    = threadIdx.x;
@@ -403,109 +533,110 @@ struct solo_gemm
         const int wave_m = wave / WAVES_N;
         const int wave_n = wave % WAVES_N;
 
-        const block_work w = decode_block(args);
-        const int slice    = w.slice;
-        const tile_coord t = map_tile(w.tile_id, args.grid_m, args.grid_n, args.group);
-        const int row0 = t.m * BM;
-        const int col0 = t.n * BN;
+        const int items = args.blocks_per_batch * args.batches;
+        const int first = blockIdx.x;
+        const int hop   = gridDim.x;
 
-        const int k_steps_total = args.K / BK;
-        const int steps_per     = (k_steps_total + w.slices - 1) / w.slices;
-        const int step_begin    = slice * steps_per;
-        int       step_end      = step_begin + steps_per;
-        if(step_end > k_steps_total)
-        {
-            step_end = k_steps_total;
-        }
-        const int nk = step_end - step_begin;
-
-        const long long batch = blockIdx.y;
-        const InT* A = static_cast<const InT*>(args.A) + batch * args.batch_stride_a;
-        const InT* B = static_cast<const InT*>(args.B) + batch * args.batch_stride_b;
-
-        const long long a_ld = args.lda;
-        const long long b_ld = args.ldb;
-        const long long a_sr = A_KMAJOR ? a_ld : 1, a_sk = A_KMAJOR ? 1 : a_ld;
-        const long long b_sr = B_KMAJOR ? b_ld : 1, b_sk = B_KMAJOR ? 1 : b_ld;
+        const long long a_ld   = args.lda;
+        const long long b_ld   = args.ldb;
+        const long long a_step = BK * (A_KMAJOR ? 1 : a_ld), b_step = BK * (B_KMAJOR ? 1 : b_ld);
 
         op_a oa;
         op_b ob;
         oa.init(wave, lane, a_ld, wave_m * WTM);
         ob.init(wave, lane, b_ld, wave_n * WTN);
+        addr_a la;
+        addr_b lb;
+        la.init(wave, lane, a_ld);
+        lb.init(wave, lane, b_ld);
 
-        const InT* a_src = A + row0 * a_sr + (long long)step_begin * BK * a_sk;
-        const InT* b_src = B + col0 * b_sr + (long long)step_begin * BK * b_sk;
-        const long long a_step = BK * a_sk, b_step = BK * b_sk;
+        work_item cur = decode(args, first);
 
-        f32x4 acc[TM][TN];
-#pragma unroll
-        for(int i = 0; i < TM; ++i)
-        {
-#pragma unroll
-            for(int j = 0; j < TN; ++j)
+        // The stream of K tiles the loads follow; it runs two tiles ahead of the MFMAs.
+        // Past the last item it wraps to the workgroup's first item, so the last two
+        // tiles' worth of loads fetch that item's K tiles 0 and 1 again into stages nobody
+        // reads.  That keeps the loop uniform, and it is kept on purpose: switching those
+        // loads off (tried with a branch per load and with a zero-sized buffer descriptor)
+        // made back-to-back calls on the same operands 5 % slower at 4096^3, because the
+        // 32 workgroups of an XCD leave exactly the first two K tiles of their operand
+        // panels in its 4 MiB L2 for the next call; a call on fresh operands pays two
+        // tiles of extra L2 -> LDS traffic for nothing.
+        const InT* a_src       = cur.a;
+        const InT* b_src       = cur.b;
+        int        stream_left = cur.nk;
+        int        stream_item = first;
+        auto advance = [&]() {
+            a_src += a_step;
+            b_src += b_step;
+            if(--stream_left == 0)
             {
-                acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-            }
-        }
-
-        if(nk > 0)
-        {
-            u32x4 fa[2][TM], fb[2][TN];
-            const unsigned int lds_addr = (unsigned int)(size_t)lds;
-            // Past the end of K the source pointers wrap to the first tile, so the last two
-            // tiles' worth of loads fetch K tiles 0 and 1 again into stages nobody reads.
-            // That keeps the loop uniform, and it is kept on purpose: switching those loads
-            // off (tried with a branch per load and with a zero-sized buffer descriptor)
-            // made back-to-back calls on the same operands 5 % slower at 4096^3, because
-            // the 32 workgroups of an XCD leave exactly the first two K tiles of their
-            // operand panels in its 4 MiB L2 for the next call; a call on fresh operands
-            // pays 2 of K/64 tiles of extra L2 -> LDS traffic for nothing.
-            const InT* const a_first = a_src;
-            const InT* const b_first = b_src;
-            const InT* const a_end   = a_src + (long long)nk * a_step;
-            auto advance = [&]() {
-                a_src += a_step;
-                b_src += b_step;
-                if(a_src == a_end)
+                stream_item += hop;
+                if(stream_item >= items)
                 {
-                    a_src = a_first;
-                    b_src = b_first;
+                    stream_item = first;
                 }
-            };
-            // Ring of 2 tiles, two K steps per tile.  Tile t: first step on K step 0 with
-            // the reads of K step 1; then wait for the own loads of tile t+1 and the own
-            // reads of tile t, barrier; second step on K step 1 with the reads of tile
-            // t+1's K step 0.  Tile t's stage is free from that barrier on: the loads of
-            // tile t+2 go out under the second step (three quarters of them) and the
-            // first quarter of tile t+1's first step.
-            constexpr int LOADS_A = VM_LOADS / 4, LOADS_B = VM_LOADS - LOADS_A;
-            using plan_b = load_plan<2, (MFMAS - 2) / LOADS_B, 0, LOADS_B>;
-            using plan_a = load_plan<1, 4, LOADS_B, LOADS_A>;
-            addr_a la;
-            addr_b lb;
-            la.init(wave, lane, a_ld);
-            lb.init(wave, lane, b_ld);
-            const unsigned int wave_block = lds_addr + wave * 1024; // this wave's block 0, stage 0
-            // prologue: tile 0 and the first part of tile 1 on their way, tile 0 landed
-            issue_loads(std::make_integer_sequence<int, VM_LOADS>{}, la, lb, wave_block,
-                        descriptor(a_src), descriptor(b_src));
-            advance();
-            issue_loads(std::make_integer_sequence<int, LOADS_B>{}, la, lb, wave_block + STAGE,
-                        descriptor(a_src), descriptor(b_src));
-            const InT* a_prev = a_src;
-            const InT* b_prev = b_src;
-            advance();
-            __builtin_amdgcn_s_waitcnt(waitcnt_imm(LOADS_B));
-            __builtin_amdgcn_s_barrier();
-            read_first(std::make_integer_sequence<int, TM>{}, std::make_integer_sequence<int, TN>{},
-                       oa, ob, lds_addr, fa[0], fb[0]);
-            for(int it = 0; it < nk; ++it)
+                const work_item nx = decode(args, stream_item);
+                a_src              = nx.a;
+                b_src              = nx.b;
+                stream_left        = nx.nk;
+            }
+        };
+
+        // Ring of 2 tiles, two K steps per tile.  Tile t: first step on K step 0 with
+        // the reads of K step 1; then wait for the own loads of tile t+1 and the own
+        // reads of tile t, barrier; second step on K step 1 with the reads of tile
+        // t+1's K step 0.  Tile t's stage is free from that barrier on: the loads of
+        // tile t+2 go out under the second step (three quarters of them) and the
+        // first quarter of tile t+1's first step.
+        constexpr int LOADS_A = VM_LOADS / 4, LOADS_B = VM_LOADS - LOADS_A;
+        using plan_b = load_plan<2, (MFMAS - 2) / LOADS_B, 0, LOADS_B>;
+        using plan_a = load_plan<1, 4, LOADS_B, LOADS_A>;
+        const unsigned int lds_addr   = (unsigned int)(size_t)lds;
+        const unsigned int wave_block = lds_addr + wave * 1024; // this wave's block 0, stage 0
+        lds_char_ptr       strip      = lds + LDS_BYTES + wave * STRIP_BYTES;
+
+        u32x4 fa[2][TM], fb[2][TN];
+        // prologue: tile 0 and the first part of tile 1 on their way, tile 0 landed
+        issue_loads(std::make_integer_sequence<int, VM_LOADS>{}, la, lb, wave_block,
+                    descriptor(a_src), descriptor(b_src));
+        advance();
+        issue_loads(std::make_integer_sequence<int, LOADS_B>{}, la, lb, wave_block + STAGE,
+                    descriptor(a_src), descriptor(b_src));
+        const InT* a_prev = a_src;
+        const InT* b_prev = b_src;
+        advance();
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(LOADS_B));
+        __builtin_amdgcn_s_barrier();
+        read_first(std::make_integer_sequence<int, TM>{}, std::make_integer_sequence<int, TN>{},
+                   oa, ob, lds_addr, fa[0], fb[0]);
+
+        unsigned int here = 0; // stage (byte offset) of the tile the MFMAs are on
+        int          item = first;
+        for(;;)
+        {
+            f32x4 acc[TM][TN];
+#pragma unroll
+            for(int i = 0; i < TM; ++i)
             {
-                const step_ctx c0{oa, ob, la, lb, lds_addr + (it & 1) * STAGE,
-                                  wave_block + ((it + 1) & 1) * STAGE, descriptor(a_prev),
-                                  descriptor(b_prev)};
-                const step_ctx c1{oa, ob, la, lb, lds_addr + ((it + 1) & 1) * STAGE,
-                                  wave_block + (it & 1) * STAGE, descriptor(a_src), descriptor(b_src)};
+#pragma unroll
+                for(int j = 0; j < TN; ++j)
+                {
+                    acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                }
+            }
+#pragma unroll
+            for(int i = 0; i < TM; ++i)
+            {
+                settle_row(acc[i]);
+            }
+
+            for(int it = 0; it < cur.nk; ++it)
+            {
+                const unsigned int there = STAGE - here;
+                const step_ctx c0{oa, ob, la, lb, lds_addr + here, wave_block + there,
+                                  descriptor(a_prev), descriptor(b_prev)};
+                const step_ctx c1{oa, ob, la, lb, lds_addr + there, wave_block + here,
+                                  descriptor(a_src), descriptor(b_src)};
                 __builtin_amdgcn_s_waitcnt(waitcnt_imm(63)); // last step's fragment reads
                 step<1, plan_a>(c0, fa[0], fb[0], fa[1], fb[1], acc);
                 __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
@@ -514,38 +645,27 @@ struct solo_gemm
                 a_prev = a_src;
                 b_prev = b_src;
                 advance();
+                here = there;
             }
-            // the wrapped tail loads and the last fragment reads may still be in flight;
             // the MFMAs are invisible to the compiler, so cover their result latency by
-            // hand
-            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+            // hand; the next item's first fragments and loads stay in flight
             asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-        }
+            write_item(args, cur, acc, wave_m * WTM, wave_n * WTN, lane, strip);
 
-        if(w.slices == 1)
-        {
-            OutT* C = static_cast<OutT*>(args.C) + batch * args.batch_stride_c;
-            if constexpr(sizeof(OutT) == 2 && !GUARD_C)
+            item += hop;
+            if(item >= items)
             {
-                // every wave has waited for its own loads; after the barrier no load of
-                // the tile ring is in flight and the ring can hold the store strips
-                __builtin_amdgcn_s_barrier();
-                write_out_staged(acc, C, args.N, row0 + wave_m * WTM, col0 + wave_n * WTN, lane,
-                                 lds + wave * STRIP_BYTES);
+                break;
             }
-            else
-            {
-                write_out<MI, GUARD_C>(
-                    acc, C, args.M, args.N, args.N, row0 + wave_m * WTM, col0 + wave_n * WTN, lane);
-            }
+            cur = decode(args, item);
+            // The last step read these fragments already; reading them again here instead
+            // of keeping them across the stores leaves the stores the registers (with 64
+            // more live the compiler spilled accumulators to scratch memory).
+            read_first(std::make_integer_sequence<int, TM>{}, std::make_integer_sequence<int, TN>{},
+                       oa, ob, lds_addr + here, fa[0], fb[0]);
         }
-        else
-        {
-            long long pitch;
-            float*    P = partial_base<BM, BN>(args, w, batch, row0, col0, pitch);
-            write_out<MI, GUARD_C>(
-                acc, P, args.M, args.N, pitch, row0 + wave_m * WTM, col0 + wave_n * WTN, lane);
-        }
+        // the wrapped tail loads are still in flight
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
     }
 };
 

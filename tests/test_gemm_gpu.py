@@ -215,6 +215,40 @@ def test_split_tail_wave_agrees_with_oracle(loader):
                                          f"C{lc} A{la} B{lb}: {e}") from None
 
 
+def test_workgroups_that_take_several_tiles_agree_with_oracle(loader):
+    """The one-wave-per-SIMD kernel launches one workgroup per CU, and each walks over
+    work items CU count apart with ONE load stream running through them.  Cases: more
+    tiles than the 256 CUs with 1, 2 and 3 K tiles per item (with one K tile the load
+    stream is two items ahead of the MFMAs; with three the ring parity flips from item
+    to item), items that straddle batch entries, a K split on top, a ragged edge, fp32
+    and 16-bit C."""
+    solo = [v for v in loader.variants() if v.pipeline == 5]
+    assert solo, "no one-wave-per-SIMD variant compiled"
+    v = solo[0]
+    cases = [  # M, N, K, batch, split field
+        (4352, 4352, 64, 1, 1),     # 289 items of one K tile
+        (4352, 4608, 192, 1, 1),    # 306 items of three K tiles
+        (1024, 768, 128, 30, 1),    # 12 tiles x 30 batch entries = 360 items
+        (2048, 2304, 320, 2, 2),    # 72 tiles x 2 slices x 2 batch entries = 288 items
+        (4344, 4360, 128, 1, 1),    # ragged edges (guarded stores)
+    ]
+    for n, (M, N, K, batch, split) in enumerate(cases):
+        tname = "f16_f16" if n % 2 == 0 else "f32_bf16"
+        din, dout = TYPE_PAIRS[tname]
+        for (lc, la, lb) in [(0, 0, 1), (1, 1, 0)]:
+            A = np.concatenate([O.init_matrix(M, K, la, din, seed=30 + b) for b in range(batch)])
+            B = np.concatenate([O.init_matrix(K, N, lb, din, seed=60 + b) for b in range(batch)])
+            gpu = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout, batch=batch,
+                          variant=(v.index, 4, split))
+            for b in range(batch):
+                try:
+                    check_against_oracle(gpu[b * M * N:(b + 1) * M * N], A[b * M * K:(b + 1) * M * K],
+                                         B[b * K * N:(b + 1) * K * N], M, N, K, lc, la, lb, din, dout)
+                except AssertionError as e:
+                    raise AssertionError(f"{M}x{N}x{K} batch {b}/{batch} split {split} layouts "
+                                         f"C{lc} A{la} B{lb} {tname}: {e}") from None
+
+
 def test_degenerate_arguments(loader):
     import torch
 

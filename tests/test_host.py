@@ -203,10 +203,32 @@ def test_hand_scheduled_kernel_keeps_accumulators_in_place(tmp_path):
             f"{func}: MFMAs outside the main loop (peeled or duplicated code)"
         bad = [b for b in body if re.search(r"v_accvgpr_|scratch_", b)]
         assert not bad, f"{func}: accumulator traffic or spills inside the MFMA loop: {bad[:3]}"
-    # after the last MFMA of each kernel: two s_nop 15 before anything names an AGPR
-    for func in loops:
-        body = text[text.index(func + ":"):]
-        body = body[:body.index(".Lfunc_end")]
-        tail = body[body.rindex("v_mfma"):].split("\n")
-        first_use = next(i for i, b in enumerate(tail) if i > 0 and re.search(r"[ ,]a\[?\d", b))
-        assert sum("s_nop 15" in b for b in tail[:first_use]) >= 2, func
+    # on every path that leaves the MFMA loop: two s_nop 15 before anything names an AGPR
+    for func, body in loops.items():
+        whole = text[text.index(func + ":"):]
+        lines = whole[:whole.index(".Lfunc_end")].split("\n")
+        label_at = {m.group(1): n for n, line in enumerate(lines)
+                    if (m := re.match(r"^(\.LBB\w+):", line))}
+        last = max(n for n, line in enumerate(lines) if "v_mfma" in line)
+        seen, todo, checked = set(), [(last + 1, 0)], 0
+        while todo:
+            n, nops = todo.pop()
+            while n < len(lines) and (n, nops) not in seen:
+                seen.add((n, nops))
+                line = lines[n]
+                if "v_mfma" in line:
+                    break  # back in the loop
+                nops += "s_nop 15" in line
+                if nops >= 2:
+                    checked += 1
+                    break
+                assert not re.search(r"[ ,]a\[?\d", line), f"{func}: {line.strip()} too early after the MFMAs"
+                m = re.match(r"^\s+s_(c?)branch\w*\s+(\.LBB\w+)", line)
+                if "s_endpgm" in line:
+                    break
+                if m:
+                    todo.append((label_at[m.group(2)], nops))
+                    if not m.group(1):
+                        break
+                n += 1
+        assert checked >= 1, func
