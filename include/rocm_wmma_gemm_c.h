@@ -76,8 +76,11 @@ int rocm_wmma_gemm_variant_info_get(int variant, rocm_wmma_gemm_variant_info* in
  * gemm_config_gfx950_*.json, then shape heuristics).  type_idx as above.
  * Also reports the swizzle (tile-row group height) and the split field: s > 1 = every
  * tile's K range is cut into s slices; -s < -1 = only the tiles of the last, partial
- * wave over the compute units are cut into s slices; 1 = no split.  Returns the variant
- * index, or -1 for invalid arguments. */
+ * wave over the compute units are cut into s slices; -1 = the persistent kernel's
+ * workgroups each take the same number of K tiles of the sequence of all K tiles of the
+ * launch, wherever the tile borders fall, and the cut tiles are added up afterwards (other
+ * kernels read -1 as 1); 1 = no split.  Returns the variant index, or -1 for invalid
+ * arguments. */
 int rocm_wmma_gemm_select(size_t M, size_t N, size_t K, int type_idx, int layout_c, int layout_a,
                           int layout_b, int* swizzle, int* split_k);
 

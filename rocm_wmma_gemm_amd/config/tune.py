@@ -59,12 +59,15 @@ def key_of(entry: dict):
 
 
 def config_json(v, swizzle: int, split_k: int) -> dict:
-    """split_k as the library's hook takes it: s > 1 every tile split, -s only the tail wave."""
+    """split_k as the library's hook takes it: s > 1 every tile split, -s (s > 1) only the
+    tail wave, -1 the persistent kernel's walk by K tile."""
     cfg = {"warps_m": v.warps_m, "warps_n": v.warps_n, "warp_tile_m": v.warp_tile_m,
            "warp_tile_n": v.warp_tile_n, "swizzle": swizzle, "bits": 128,
            "block_k": v.block_k, "pipeline": v.pipeline, "split_k": max(split_k, 1)}
     if split_k < -1:
         cfg["tail_split"] = -split_k
+    if split_k == -1:
+        cfg["stream_k"] = 1
     return cfg
 
 
@@ -90,6 +93,9 @@ def candidates(variants, M, N, K, lc):
             for s in (2, 3, 4, 6, 8):
                 if tail * s <= CUS * 5 // 4 and k_steps // s >= 4:
                     splits.append(-s)
+        # the persistent kernel can also give every workgroup the same number of K tiles
+        if v.pipeline == 5 and tiles % CUS != 0 and tiles * k_steps >= 4 * CUS:
+            splits.append(-1)
         for sw in swizzles:
             for sk in splits:
                 out.append((v, sw, sk))

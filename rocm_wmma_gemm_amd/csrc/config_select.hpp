@@ -24,7 +24,8 @@ struct launch_plan
 {
     int variant; // index into the compiled variant table
     int swizzle; // tile-row band height of the tile map
-    int split_k; // K slices (1 = off); -s = split only the last, partial wave of tiles s ways
+    int split_k; // K slices (1 = off); -s (s > 1) = split only the last, partial wave of tiles s
+                 // ways; -1 = persistent kernel walks by K tile (equal K tiles per workgroup)
 };
 
 struct tuned_entry

@@ -393,13 +393,33 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
             = std::min(batches_per_launch, std::max<size_t>((size_t{1} << 30) / (plane_bytes * split_k), 1));
     }
     // A persistent kernel numbers its work items over the whole launch with an int.
-    const size_t blocks_per_batch = tail_begin + split_tiles * static_cast<size_t>(split_k);
-    const bool   persistent       = v.pipeline == 5;
+    size_t     blocks_per_batch = tail_begin + split_tiles * static_cast<size_t>(split_k);
+    const bool persistent       = v.pipeline == 5;
     if(persistent)
     {
         batches_per_launch = std::min(batches_per_launch, std::max<size_t>(0x7fffffffull / blocks_per_batch, 1));
     }
-    const size_t partial_bytes = split_k > 1 ? plane_bytes * split_k * batches_per_launch : 0;
+    // plan.split_k == -1, persistent kernel: the workgroups walk by K tile instead of by
+    // tile, each over the same number of K tiles of the sequence of all K tiles of the
+    // launch; tiles cut by the borders of those ranges are added up from two fp32 slots
+    // per workgroup.  For tile counts that fill the CUs badly (144 or 320 tiles on 256).
+    size_t stream_groups = 0, stream_units = 0;
+    if(persistent && plan.split_k == -1)
+    {
+        const size_t cus         = compute_units_of_current_device();
+        const size_t total_units = tiles * p.batch * static_cast<size_t>(k_steps);
+        const size_t chunks      = v.block_m * v.block_n / device::reduce_chunk_elems;
+        if(cus > 0 && total_units > 0 && total_units <= 0x7fffffffull && tiles * p.batch * chunks <= 0x7fffffffull)
+        {
+            stream_groups      = std::min(cus, total_units);
+            stream_units       = (total_units + stream_groups - 1) / stream_groups;
+            stream_groups      = (total_units + stream_units - 1) / stream_units;
+            batches_per_launch = p.batch;
+        }
+    }
+    const size_t partial_bytes = stream_groups > 0
+                                     ? 2 * stream_groups * v.block_m * v.block_n * sizeof(float)
+                                     : (split_k > 1 ? plane_bytes * split_k * batches_per_launch : 0);
 
     char* workspace = nullptr;
     if(pack_bytes + partial_bytes > 0)
@@ -419,11 +439,18 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
                 }
                 return launch<OutT>(type_idx, retry, p, stream);
             }
-            split_k    = 1;
-            tail_begin = 0;
+            split_k          = 1;
+            tail_begin       = 0;
+            blocks_per_batch = tiles;
+            stream_groups    = 0;
+            stream_units     = 0;
+            if(persistent)
+            {
+                batches_per_launch = std::min<size_t>(p.batch, std::max<size_t>(0x7fffffffull / tiles, 1));
+            }
         }
     }
-    float* partials = split_k > 1 ? reinterpret_cast<float*>(workspace + pack_bytes) : nullptr;
+    float* partials = split_k > 1 || stream_groups > 0 ? reinterpret_cast<float*>(workspace + pack_bytes) : nullptr;
 
     if(packed)
     {
@@ -485,6 +512,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         args.partials       = partials;
         args.blocks_per_batch = static_cast<int>(blocks_per_batch);
         args.batches          = static_cast<int>(nb);
+        args.stream_units     = static_cast<int>(stream_units);
 
         dim3 grid(static_cast<unsigned>(blocks_per_batch), static_cast<unsigned>(nb));
         if(persistent)
@@ -493,8 +521,25 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
             const size_t cus   = compute_units_of_current_device();
             const size_t items = blocks_per_batch * nb;
             grid               = dim3(static_cast<unsigned>(cus > 0 ? std::min(items, cus) : items), 1);
+            if(stream_groups > 0)
+            {
+                grid = dim3(static_cast<unsigned>(stream_groups), 1);
+            }
         }
         fn<<<grid, dim3(v.threads), 0, stream>>>(args);
+        if(stream_groups > 0)
+        {
+            if(stream_units % static_cast<size_t>(k_steps) != 0)
+            {
+                // (ranges of whole tiles cut nothing)
+                device::reduce_stream_tiles<OutT>
+                    <<<dim3(static_cast<unsigned>(tiles * nb * (v.block_m * v.block_n / device::reduce_chunk_elems))),
+                       dim3(256), 0, stream>>>(static_cast<OutT*>(args.C), partials, args.M, args.N, v.block_m,
+                                               v.block_n, args.grid_m, args.grid_n, args.group, k_steps,
+                                               args.stream_units, args.batch_stride_c);
+            }
+            continue;
+        }
         if(split_k > 1 && tail_begin == 0)
         {
             const long long plane  = static_cast<long long>(p.M) * static_cast<long long>(p.N);

@@ -505,7 +505,7 @@ struct direct_gemm
         __builtin_amdgcn_sched_barrier(0);
     }
 
-    __device__ static void run(const gemm_args& args)
+    __device__ __forceinline__ static void run(const gemm_args& args)
     {
         __shared__ __attribute__((aligned(1024))) char lds_raw[LDS_BYTES];
         lds_char_ptr lds = (lds_char_ptr)lds_raw;

@@ -69,6 +69,10 @@ struct gemm_args
                           // [batch][slice][M][N] planes; else [batch][split tile][slice][BM][BN]
     int         blocks_per_batch; // workgroups' worth of work per batch entry (whole tiles + slices)
     int         batches; // batch entries of this launch; blocks_per_batch * batches fits an int
+    int         stream_units; // persistent kernel only.  0: workgroups take whole items.  U > 0:
+                              // workgroup g takes K tiles [g * U, (g + 1) * U) of the sequence of all
+                              // K tiles of all tiles of all batch entries; partials then holds two
+                              // [BM][BN] slots per workgroup
 };
 
 // What one workgroup works on.  blockIdx.x enumerates the whole tiles first, then
@@ -449,7 +453,7 @@ struct staged_gemm
         }
     }
 
-    __device__ static void run(const gemm_args& args)
+    __device__ __forceinline__ static void run(const gemm_args& args)
     {
         __shared__ u32x4 lds[2 * STAGE];
 
@@ -687,6 +691,92 @@ __global__ void __launch_bounds__(256) reduce_split_tiles(OutT* __restrict__ C,
             if(row < M && col + v < N)
             {
                 out[(long long)row * N + col + v] = to_out<OutT>(s[u][v]);
+            }
+        }
+    }
+}
+
+// Adds up the parts of the tiles that a persistent kernel walking by K tile
+// (gemm_args::stream_units > 0) left in the workgroups' fp32 slots.  Workgroup w worked
+// on K tiles [w * units, (w + 1) * units) of the sequence in which tile number t (walk
+// order, batch entries one after the other) holds K tiles [t * k_tiles, (t + 1) * k_tiles).
+// A tile inside one range went to C whole and is skipped here; of any other tile,
+// workgroup w's part is in slot 2w if the part holds the first K tile of w's range,
+// else in slot 2w + 1.  Parts are added in ascending order of w.  blockIdx.x = tile *
+// chunks + chunk, 4096 elements per chunk as in reduce_split_tiles.
+template<class OutT>
+__global__ void __launch_bounds__(256) reduce_stream_tiles(OutT* __restrict__ C,
+                                                           const float* __restrict__ partials,
+                                                           int       M,
+                                                           int       N,
+                                                           int       block_m,
+                                                           int       block_n,
+                                                           int       grid_m,
+                                                           int       grid_n,
+                                                           int       group,
+                                                           int       k_tiles,
+                                                           int       units,
+                                                           long long batch_stride_c)
+{
+    const int elems    = block_m * block_n;
+    const int chunks   = elems / reduce_chunk_elems;
+    const int tile_lin = blockIdx.x / chunks;
+    const int chunk    = blockIdx.x - tile_lin * chunks;
+    const int k_first  = tile_lin * k_tiles;
+    const int first    = k_first / units;
+    const int last     = (k_first + k_tiles - 1) / units;
+    if(first == last)
+    {
+        return;
+    }
+    const int        tiles = grid_m * grid_n;
+    const int        batch = tile_lin / tiles;
+    const tile_coord t     = map_tile(tile_lin - batch * tiles, grid_m, grid_n, group);
+    const int        row0 = t.m * block_m, col0 = t.n * block_n;
+    OutT*            out = C + batch * batch_stride_c;
+    f32x4            s[4];
+#pragma unroll
+    for(int u = 0; u < 4; ++u)
+    {
+        s[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    const int e0 = chunk * reduce_chunk_elems + threadIdx.x * 4;
+    for(int w = first; w <= last; ++w)
+    {
+        const long long slot = 2 * (long long)w + (w * units >= k_first ? 0 : 1);
+        const float*    P    = partials + slot * elems;
+#pragma unroll
+        for(int u = 0; u < 4; ++u)
+        {
+            s[u] += *reinterpret_cast<const f32x4*>(P + e0 + u * 1024);
+        }
+    }
+    typedef OutT out4 __attribute__((ext_vector_type(4)));
+    const bool vector_ok = (N & 3) == 0 && ((unsigned long long)out & (sizeof(out4) - 1)) == 0;
+#pragma unroll
+    for(int u = 0; u < 4; ++u)
+    {
+        const int e   = e0 + u * 1024;
+        const int row = row0 + e / block_n, col = col0 + e % block_n; // block_n % 4 == 0
+        if(vector_ok && row < M && col + 3 < N)
+        {
+            out4 o;
+#pragma unroll
+            for(int v = 0; v < 4; ++v)
+            {
+                o[v] = to_out<OutT>(s[u][v]);
+            }
+            *reinterpret_cast<out4*>(out + (long long)row * N + col) = o;
+        }
+        else
+        {
+#pragma unroll
+            for(int v = 0; v < 4; ++v)
+            {
+                if(row < M && col + v < N)
+                {
+                    out[(long long)row * N + col + v] = to_out<OutT>(s[u][v]);
+                }
             }
         }
     }

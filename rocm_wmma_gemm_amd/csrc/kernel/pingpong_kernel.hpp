@@ -101,7 +101,7 @@ struct pingpong_gemm
         ((fb[Y / TN][Y % TN] = ob.template fragment_pinned<Y % TN, Y / TN>(stage + A_BYTES)), ...);
     }
 
-    __device__ static void run(const gemm_args& args)
+    __device__ __forceinline__ static void run(const gemm_args& args)
     {
         __shared__ __attribute__((aligned(1024))) char lds_raw[LDS_BYTES];
         lds_char_ptr       lds      = (lds_char_ptr)lds_raw;

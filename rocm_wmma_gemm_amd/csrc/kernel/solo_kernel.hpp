@@ -148,6 +148,15 @@ struct solo_gemm
     using addr_a = load_addr<A_KMAJOR, BM>;
     using addr_b = load_addr<B_KMAJOR, BN>;
 
+    // The same pointer, held in scalar registers (it must be the same in every lane).
+    __device__ __forceinline__ static const InT* scalar_pointer(const InT* p)
+    {
+        const unsigned long long v  = (unsigned long long)p;
+        const unsigned int       lo = __builtin_amdgcn_readfirstlane((unsigned int)v);
+        const unsigned int       hi = __builtin_amdgcn_readfirstlane((unsigned int)(v >> 32));
+        return (const InT*)(((unsigned long long)hi << 32) | lo);
+    }
+
     // 128-bit buffer descriptor of a tile: base = its origin, no stride, no range check
     // that could fire (every tile span fits 32 bits: the host checks), raw 32-bit format.
     __device__ __forceinline__ static u32x4 descriptor(const InT* origin)
@@ -427,43 +436,112 @@ struct solo_gemm
         }
     }
 
-    // One unit of work of a workgroup: a C tile (or one K slice of a split tile) of one
-    // batch entry.
+    // One unit of work of a workgroup: a C tile, or a run of K tiles of one, of one batch
+    // entry.
     struct work_item
     {
-        block_work w;
         int        batch;
         int        row0, col0;
-        int        nk; // K tiles; the host never creates an empty slice
+        int        nk; // K tiles, at least one
         const InT* a; // first K tile of the operands
         const InT* b;
+        float*     partial; // nullptr: the item is a whole tile and goes to C; else where
+                            // element (row, col) of C, global coordinates, goes:
+                            // partial[row * pitch + col]
+        long long  pitch;
+        int        next; // position of the workgroup's next item
     };
 
-    __device__ __forceinline__ static work_item decode(const gemm_args& args, int v)
+    // The items of a workgroup, in one of two orders.
+    //  - by item (args.stream_units == 0): the launch holds blocks_per_batch * batches
+    //    items (whole tiles first, then K slices of the split tiles, per batch entry);
+    //    a position is an item number and workgroup g takes g, g + gridDim.x, ...
+    //  - by K tile (args.stream_units = U > 0): all K tiles of all tiles of all batch
+    //    entries form one sequence, tile after tile in walk order, and workgroup g takes
+    //    K tiles [g * U, (g + 1) * U) of it: every workgroup does the same number of
+    //    MFMAs whatever the tile count.  A position is a K tile number; an item is the
+    //    part of the workgroup's range that lies in one tile.  A tile that lies in one
+    //    range goes to C; of a tile cut by range borders every part goes to the
+    //    workgroup's first or second fp32 slot ("first": the part holds the range's first
+    //    K tile) and reduce_stream_tiles adds the parts up.
+    struct walk
+    {
+        int begin, end, hop; // positions of this workgroup: begin, then item.next, while < end
+
+        __device__ __forceinline__ static walk of(const gemm_args& args)
+        {
+            if(args.stream_units == 0)
+            {
+                return {(int)blockIdx.x, args.blocks_per_batch * args.batches, (int)gridDim.x};
+            }
+            const int total = args.grid_m * args.grid_n * args.batches * (args.K / BK);
+            const int begin = blockIdx.x * args.stream_units;
+            const int end   = begin + args.stream_units;
+            return {begin, end < total ? end : total, 0};
+        }
+    };
+
+    __device__ __forceinline__ static work_item decode(const gemm_args& args, const walk& wk, int pos)
     {
         work_item x;
-        x.batch            = v / args.blocks_per_batch;
-        x.w                = decode_block(args, v - x.batch * args.blocks_per_batch);
-        const tile_coord t = map_tile(x.w.tile_id, args.grid_m, args.grid_n, args.group);
-        x.row0             = t.m * BM;
-        x.col0             = t.n * BN;
-
         const int k_steps_total = args.K / BK;
-        const int steps_per     = (k_steps_total + x.w.slices - 1) / x.w.slices;
-        const int step_begin    = x.w.slice * steps_per;
-        int       step_end      = step_begin + steps_per;
-        if(step_end > k_steps_total)
+        int       step_begin;
+        if(wk.hop != 0)
         {
-            step_end = k_steps_total;
+            x.batch            = pos / args.blocks_per_batch;
+            const block_work w = decode_block(args, pos - x.batch * args.blocks_per_batch);
+            const tile_coord t = map_tile(w.tile_id, args.grid_m, args.grid_n, args.group);
+            x.row0             = t.m * BM;
+            x.col0             = t.n * BN;
+            const int steps_per = (k_steps_total + w.slices - 1) / w.slices;
+            step_begin          = w.slice * steps_per;
+            int step_end        = step_begin + steps_per;
+            if(step_end > k_steps_total)
+            {
+                step_end = k_steps_total;
+            }
+            x.nk      = step_end - step_begin;
+            x.next    = pos + wk.hop;
+            x.partial = nullptr;
+            x.pitch   = args.N;
+            if(w.slices > 1)
+            {
+                x.partial = partial_base<BM, BN>(args, w, x.batch, x.row0, x.col0, x.pitch);
+            }
         }
-        x.nk = step_end - step_begin;
-
+        else
+        {
+            const int tiles    = args.grid_m * args.grid_n;
+            const int tile_lin = pos / k_steps_total;
+            step_begin         = pos - tile_lin * k_steps_total;
+            x.batch            = tile_lin / tiles;
+            const tile_coord t = map_tile(tile_lin - x.batch * tiles, args.grid_m, args.grid_n, args.group);
+            x.row0             = t.m * BM;
+            x.col0             = t.n * BN;
+            x.nk               = k_steps_total - step_begin;
+            if(x.nk > wk.end - pos)
+            {
+                x.nk = wk.end - pos;
+            }
+            x.next    = pos + x.nk;
+            x.partial = nullptr;
+            x.pitch   = args.N;
+            if(x.nk != k_steps_total)
+            {
+                const long long slot = 2 * (long long)blockIdx.x + (pos == wk.begin ? 0 : 1);
+                x.partial = args.partials + slot * (long long)(BM * BN) - ((long long)x.row0 * BN + x.col0);
+                x.pitch   = BN;
+            }
+        }
         const long long a_sr = A_KMAJOR ? args.lda : 1, a_sk = A_KMAJOR ? 1 : args.lda;
         const long long b_sr = B_KMAJOR ? args.ldb : 1, b_sk = B_KMAJOR ? 1 : args.ldb;
-        x.a = static_cast<const InT*>(args.A) + x.batch * args.batch_stride_a + x.row0 * a_sr
-              + (long long)step_begin * BK * a_sk;
-        x.b = static_cast<const InT*>(args.B) + x.batch * args.batch_stride_b + x.col0 * b_sr
-              + (long long)step_begin * BK * b_sk;
+        // The integer divisions above run on the vector ALU (there is no scalar divide),
+        // and the compiler then tends to keep what depends on them in vector registers;
+        // the buffer descriptors built from these pointers must be scalar.
+        x.a = scalar_pointer(static_cast<const InT*>(args.A) + x.batch * args.batch_stride_a
+                             + x.row0 * a_sr + (long long)step_begin * BK * a_sk);
+        x.b = scalar_pointer(static_cast<const InT*>(args.B) + x.batch * args.batch_stride_b
+                             + x.col0 * b_sr + (long long)step_begin * BK * b_sk);
         return x;
     }
 
@@ -476,7 +554,7 @@ struct solo_gemm
                                                       int                lane,
                                                       lds_char_ptr       strip)
     {
-        if(x.w.slices == 1)
+        if(x.partial == nullptr)
         {
             OutT* C = static_cast<OutT*>(args.C) + x.batch * args.batch_stride_c;
             if constexpr(!GUARD_C)
@@ -488,19 +566,15 @@ struct solo_gemm
                 write_out<MI, GUARD_C>(acc, C, args.M, args.N, args.N, x.row0 + row_w, x.col0 + col_w, lane);
             }
         }
+        else if constexpr(!GUARD_C)
+        {
+            // the reduce kernel reads these next: no streaming hint
+            write_out_staged<false>(acc, x.partial, x.pitch, x.row0 + row_w, x.col0 + col_w, lane, strip);
+        }
         else
         {
-            long long pitch;
-            float*    P = partial_base<BM, BN>(args, x.w, x.batch, x.row0, x.col0, pitch);
-            if constexpr(!GUARD_C)
-            {
-                // the reduce kernel reads these next: no streaming hint
-                write_out_staged<false>(acc, P, pitch, x.row0 + row_w, x.col0 + col_w, lane, strip);
-            }
-            else
-            {
-                write_out<MI, GUARD_C>(acc, P, args.M, args.N, pitch, x.row0 + row_w, x.col0 + col_w, lane);
-            }
+            write_out<MI, GUARD_C>(
+                acc, x.partial, args.M, args.N, x.pitch, x.row0 + row_w, x.col0 + col_w, lane);
         }
     }
 
@@ -515,14 +589,14 @@ struct solo_gemm
                        "+a"(row[6]), "+a"(row[7]));
     }
 
-    // The workgroups are persistent: workgroup g works on items g, g + gridDim.x, ... of
-    // the launch, and the K tiles of all its items form ONE stream through the ring, so
+    // The workgroups are persistent: a workgroup works on its items (see walk) one after
+    // the other, and the K tiles of all its items form ONE stream through the ring, so
     // the loads of an item's first two K tiles go out under the last two steps of the
     // item before it and the only thing between two items' MFMAs is the store of the
     // accumulators.  (A workgroup per item pays, per item, the dispatch of the next
     // workgroup, the latency of the first loads and the drain of the stores: about
     // 13 us, nine K tiles' worth, at 256 x 256 x 64.)
-    __device__ static void run(const gemm_args& args)
+    __device__ __forceinline__ static void run(const gemm_args& args)
     {
         __shared__ __attribute__((aligned(1024))) char lds_raw[LDS_BYTES + WAVES * STRIP_BYTES];
         lds_char_ptr lds = (lds_char_ptr)lds_raw;
@@ -533,9 +607,7 @@ struct solo_gemm
         const int wave_m = wave / WAVES_N;
         const int wave_n = wave % WAVES_N;
 
-        const int items = args.blocks_per_batch * args.batches;
-        const int first = blockIdx.x;
-        const int hop   = gridDim.x;
+        const walk wk = walk::of(args);
 
         const long long a_ld   = args.lda;
         const long long b_ld   = args.ldb;
@@ -550,7 +622,7 @@ struct solo_gemm
         la.init(wave, lane, a_ld);
         lb.init(wave, lane, b_ld);
 
-        work_item cur = decode(args, first);
+        work_item cur = decode(args, wk, wk.begin);
 
         // The stream of K tiles the loads follow; it runs two tiles ahead of the MFMAs.
         // Past the last item it wraps to the workgroup's first item, so the last two
@@ -564,21 +636,17 @@ struct solo_gemm
         const InT* a_src       = cur.a;
         const InT* b_src       = cur.b;
         int        stream_left = cur.nk;
-        int        stream_item = first;
+        int        stream_next = cur.next;
         auto advance = [&]() {
             a_src += a_step;
             b_src += b_step;
             if(--stream_left == 0)
             {
-                stream_item += hop;
-                if(stream_item >= items)
-                {
-                    stream_item = first;
-                }
-                const work_item nx = decode(args, stream_item);
+                const work_item nx = decode(args, wk, stream_next < wk.end ? stream_next : wk.begin);
                 a_src              = nx.a;
                 b_src              = nx.b;
                 stream_left        = nx.nk;
+                stream_next        = nx.next;
             }
         };
 
@@ -611,7 +679,6 @@ struct solo_gemm
                    oa, ob, lds_addr, fa[0], fb[0]);
 
         unsigned int here = 0; // stage (byte offset) of the tile the MFMAs are on
-        int          item = first;
         for(;;)
         {
             f32x4 acc[TM][TN];
@@ -652,12 +719,11 @@ struct solo_gemm
             asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
             write_item(args, cur, acc, wave_m * WTM, wave_n * WTN, lane, strip);
 
-            item += hop;
-            if(item >= items)
+            if(cur.next >= wk.end)
             {
                 break;
             }
-            cur = decode(args, item);
+            cur = decode(args, wk, cur.next);
             // The last step read these fragments already; reading them again here instead
             // of keeping them across the stores leaves the stores the registers (with 64
             // more live the compiler spilled accumulators to scratch memory).

@@ -221,7 +221,8 @@ def test_workgroups_that_take_several_tiles_agree_with_oracle(loader):
     tiles than the 256 CUs with 1, 2 and 3 K tiles per item (with one K tile the load
     stream is two items ahead of the MFMAs; with three the ring parity flips from item
     to item), items that straddle batch entries, a K split on top, a ragged edge, fp32
-    and 16-bit C."""
+    and 16-bit C; and the walk by K tile, where a workgroup's range of K tiles starts
+    and ends anywhere inside a tile and the parts are added up by a second kernel."""
     solo = [v for v in loader.variants() if v.pipeline == 5]
     assert solo, "no one-wave-per-SIMD variant compiled"
     v = solo[0]
@@ -231,6 +232,14 @@ def test_workgroups_that_take_several_tiles_agree_with_oracle(loader):
         (1024, 768, 128, 30, 1),    # 12 tiles x 30 batch entries = 360 items
         (2048, 2304, 320, 2, 2),    # 72 tiles x 2 slices x 2 batch entries = 288 items
         (4344, 4360, 128, 1, 1),    # ragged edges (guarded stores)
+        # split field -1: the workgroups walk by K tile, each over ceil(all K tiles / 256)
+        (3072, 3072, 512, 1, -1),   # 1152 K tiles, 5 per workgroup: tiles cut at odd places
+        (1536, 1280, 1024, 1, -1),  # 480 K tiles, 2 per workgroup: every tile in 8 parts
+        (768, 512, 640, 7, -1),     # ranges that run from one batch entry into the next
+        (1000, 1300, 320, 1, -1),   # ragged edges
+        (4096, 4096, 128, 1, -1),   # ranges of whole tiles: nothing to add up
+        (512, 512, 64, 1, -1),      # one K tile per workgroup
+        (2560, 2304, 4096, 1, -1),  # 90 tiles of 64 K tiles on 256 CUs: 23 per workgroup
     ]
     for n, (M, N, K, batch, split) in enumerate(cases):
         tname = "f16_f16" if n % 2 == 0 else "f32_bf16"
