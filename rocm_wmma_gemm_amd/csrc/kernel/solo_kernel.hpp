@@ -357,7 +357,7 @@ struct solo_gemm
     }
 
     // Whole tiles: the wave's rows go through a private LDS strip so that a store
-    // instruction writes 4 rows x 256 contiguous bytes (16 bytes per lane) instead of
+    // instruction writes 4 rows x 256 contiguous bytes (16 bytes per lane; 128-column wave tile) instead of
     // 16 rows x 32 bytes (16-bit C) or 16 rows x 64 bytes (fp32 C and partial sums; the
     // strip is worth 6..9 % at 8192^3 and 13..16 % with shorter K there).  At 4096^3 the
     // C stores are 11 % of the call.  STREAM marks the stores as streaming: C is not read
@@ -368,8 +368,9 @@ struct solo_gemm
     // 8-byte bank columns; the 16-byte reads take two cycles instead of one, which does
     // not show).  LDS operations of one wave are served in order, so the reads see the
     // writes without a barrier; the waits keep the compiler from reordering them.
-    static constexpr int STRIP_PITCH = 272;
-    static constexpr int STRIP_BYTES = 16 * STRIP_PITCH + 256; // rounded to 4608
+    static constexpr int ROW_BYTES   = TN * 32; // 256 for the 128-column wave tile
+    static constexpr int STRIP_PITCH = ROW_BYTES + 16;
+    static constexpr int STRIP_BYTES = (16 * STRIP_PITCH + 1023) / 1024 * 1024;
     static_assert(LDS_BYTES + WAVES * STRIP_BYTES <= 160 * 1024, "tile ring and store strips must fit the 160 KB LDS");
 
     // Ties a row of accumulators to its registers at this point of the program: what
@@ -378,24 +379,39 @@ struct solo_gemm
     // no room for them, and spills.
     __device__ __forceinline__ static void pin_row(f32x4 (&row)[TN])
     {
-        static_assert(TN == 8, "eight accumulators of a row per statement");
-        asm volatile(""
-                     : "+a"(row[0]), "+a"(row[1]), "+a"(row[2]), "+a"(row[3]), "+a"(row[4]), "+a"(row[5]),
-                       "+a"(row[6]), "+a"(row[7]));
+        static_assert(TN % 2 == 0, "two accumulators per statement");
+#pragma unroll
+        for(int j = 0; j < TN; j += 2)
+        {
+            asm volatile("" : "+a"(row[j]), "+a"(row[j + 1]));
+        }
     }
 
     template<bool STREAM, class DstT>
     __device__ __forceinline__ static void write_out_staged(
         f32x4 (&acc)[TM][TN], DstT* D, long long pitch, int row_w, int col_w, int lane, lds_char_ptr strip)
     {
-        static_assert(TN == 8, "strip layout: 128 columns per wave");
-        // a strip row holds 256 bytes: all 128 columns of a 16-bit destination, 64 of fp32
+        // a strip row holds ROW_BYTES: all columns of the wave tile for a 16-bit
+        // destination, half of them for fp32
         constexpr int PASSES = sizeof(DstT) / 2;
-        constexpr int TILES  = TN / PASSES; // 16-column tiles per pass
+        static_assert(TN % PASSES == 0, "whole tiles per pass");
+        constexpr int TILES   = TN / PASSES; // 16-column tiles per pass
+        constexpr int CHUNKS  = ROW_BYTES / 16; // 16-byte pieces of a strip row
+        constexpr int READS   = 16 * CHUNKS / 64; // store instructions per pass
+        static_assert(16 * CHUNKS % 64 == 0, "the strip divides over the lanes");
         typedef DstT out4 __attribute__((ext_vector_type(4)));
         using lds_out4 = __attribute__((address_space(3))) out4;
         using lds_u32x4 = __attribute__((address_space(3))) u32x4;
         const int r16 = lane & 15, g = lane >> 4;
+        int       strip_at[READS]; // this lane's piece of read q: byte offset in the strip,
+        long long dest_at[READS]; // and element offset in D from the row block's origin
+#pragma unroll
+        for(int q = 0; q < READS; ++q)
+        {
+            const int piece = q * 64 + lane, row = piece / CHUNKS, c = piece % CHUNKS;
+            strip_at[q]     = row * STRIP_PITCH + c * 16;
+            dest_at[q]      = row * pitch + c * (16 / (int)sizeof(DstT));
+        }
 #pragma unroll
         for(int i = 0; i < TM; ++i)
         {
@@ -415,13 +431,12 @@ struct solo_gemm
                     *reinterpret_cast<lds_out4*>(strip + r16 * STRIP_PITCH + (16 * j + 4 * g) * sizeof(DstT)) = o;
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                DstT* const block = D + (long long)(row_w + 16 * i) * pitch + col_w + p * TILES * 16;
 #pragma unroll
-                for(int q = 0; q < 4; ++q)
+                for(int q = 0; q < READS; ++q)
                 {
-                    const int   row = 4 * q + g;
-                    const u32x4 v   = *reinterpret_cast<lds_u32x4*>(strip + row * STRIP_PITCH + r16 * 16);
-                    u32x4* const to = reinterpret_cast<u32x4*>(D + (long long)(row_w + 16 * i + row) * pitch + col_w
-                                                               + p * TILES * 16 + r16 * (16 / sizeof(DstT)));
+                    const u32x4  v  = *reinterpret_cast<lds_u32x4*>(strip + strip_at[q]);
+                    u32x4* const to = reinterpret_cast<u32x4*>(block + dest_at[q]);
                     if constexpr(STREAM)
                     {
                         __builtin_nontemporal_store(v, to);
@@ -583,10 +598,12 @@ struct solo_gemm
     // the writes and the first read.
     __device__ __forceinline__ static void settle_row(f32x4 (&row)[TN])
     {
-        static_assert(TN == 8, "eight accumulators of a row per statement");
-        asm volatile("s_nop 4"
-                     : "+a"(row[0]), "+a"(row[1]), "+a"(row[2]), "+a"(row[3]), "+a"(row[4]), "+a"(row[5]),
-                       "+a"(row[6]), "+a"(row[7]));
+        static_assert(TN % 2 == 0, "two accumulators per statement");
+#pragma unroll
+        for(int j = 0; j < TN; j += 2)
+        {
+            asm volatile("s_nop 4" : "+a"(row[j]), "+a"(row[j + 1]));
+        }
     }
 
     // The workgroups are persistent: a workgroup works on its items (see walk) one after

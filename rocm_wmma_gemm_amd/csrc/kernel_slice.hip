@@ -55,8 +55,10 @@ constexpr kernel_fn entry()
             device::pingpong_gemm<kIn, out_t, RWG_AK != 0, RWG_BK != 0, BM, BN, BK, WM, WN,
                                   (BK == 64 ? 2 : 4), MODE == device::load_mode::vec_guarded, 16>>;
     }
-    else if constexpr(MODE != device::load_mode::scalar && PIPE == 5)
+    else if constexpr(MODE != device::load_mode::scalar && PIPE == 5
+                      && (BM % 128 == 0 || RWG_AK != 0) && (BN % 128 == 0 || RWG_BK != 0))
     {
+        // (the LDS layout of an M/N-contiguous operand works in 128-row halves)
         return &device::gemm_entry<
             device::solo_gemm<kIn, out_t, RWG_AK != 0, RWG_BK != 0, BM, BN, BK, WM, WN,
                               (BK == 64 ? 2 : 4), MODE == device::load_mode::vec_guarded>>;

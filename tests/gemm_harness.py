@@ -51,6 +51,19 @@ def make_inputs(M, N, K, la, lb, din, seed_a=1, seed_b=1, dist="uniform", lo=-1.
     return A, B
 
 
+def built_for(v, lc, la, lb):
+    """Whether tile variant v is compiled for this layout triple: in the direct-to-LDS
+    pipelines a tile extent that is no multiple of 128 needs its operand K-contiguous in
+    kernel space (C row-major: A row-major, B column-major; a column-major C swaps the
+    operands)."""
+    if v.pipeline == 0:
+        return True
+    a_k, b_k = la == 0, lb == 1
+    if lc == 1:
+        a_k, b_k = b_k, a_k
+    return (v.block_m % 128 == 0 or a_k) and (v.block_n % 128 == 0 or b_k)
+
+
 def run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout, batch=1, poison=True, variant=None):
     import torch
 

@@ -11,8 +11,8 @@ import numpy as np
 import pytest
 
 import oracle as O
-from gemm_harness import (LAYOUTS8, TYPE_PAIRS, check_against_oracle, checksum_check, layout_id,
-                          make_inputs, run_gpu, to_device, to_host, torch_dtype)
+from gemm_harness import (LAYOUTS8, TYPE_PAIRS, built_for, check_against_oracle, checksum_check,
+                          layout_id, make_inputs, run_gpu, to_device, to_host, torch_dtype)
 
 pytestmark = pytest.mark.gpu
 
@@ -173,10 +173,16 @@ def test_every_variant_and_split_k_agree_with_oracle(loader):
     for v in loader.variants():
         for split_k in (1, 3):
             for (M, N, K) in ((512, 512, 512), (300, 520, 264), (77, 91, 1003)):
-                for (lc, la, lb) in [(0, 0, 1), (0, 1, 0), (1, 0, 0), (1, 1, 1)]:
+                for (lc, la, lb) in [(0, 0, 1), (0, 1, 0), (1, 0, 0), (1, 1, 1), (1, 0, 1)]:
                     for tname in ("f16_f16", "f32_bf16"):
                         din, dout = TYPE_PAIRS[tname]
                         A, B = make_inputs(M, N, K, la, lb, din, seed_a=7, seed_b=8)
+                        if not built_for(v, lc, la, lb):
+                            dA, dB = to_device(A, din), to_device(B, din)
+                            dC = to_device(np.zeros(M * N, dtype=A.dtype if dout != O.F32 else np.float32), dout)
+                            assert loader.run_variant(v.index, 4, split_k, dC, dA, dB, M, N, K,
+                                                      lc, la, lb) == -1, (v.index, lc, la, lb)
+                            continue
                         gpu = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout,
                                       variant=(v.index, 4, split_k))
                         try:
@@ -225,7 +231,6 @@ def test_workgroups_that_take_several_tiles_agree_with_oracle(loader):
     and ends anywhere inside a tile and the parts are added up by a second kernel."""
     solo = [v for v in loader.variants() if v.pipeline == 5]
     assert solo, "no one-wave-per-SIMD variant compiled"
-    v = solo[0]
     cases = [  # M, N, K, batch, split field
         (4352, 4352, 64, 1, 1),     # 289 items of one K tile
         (4352, 4608, 192, 1, 1),    # 306 items of three K tiles
@@ -241,10 +246,15 @@ def test_workgroups_that_take_several_tiles_agree_with_oracle(loader):
         (512, 512, 64, 1, -1),      # one K tile per workgroup
         (2560, 2304, 4096, 1, -1),  # 90 tiles of 64 K tiles on 256 CUs: 23 per workgroup
     ]
-    for n, (M, N, K, batch, split) in enumerate(cases):
+    # every case on the 256 x 256 tile; the other tiles (for them the same shapes are
+    # ragged, or hold other tile counts) take every third case, staggered
+    runs = [(v, n) for i, v in enumerate(solo) for n in range(len(cases))
+            if (v.block_m, v.block_n) == (256, 256) or n % 3 == i % 3]
+    for v, n in runs:
+        M, N, K, batch, split = cases[n]
         tname = "f16_f16" if n % 2 == 0 else "f32_bf16"
         din, dout = TYPE_PAIRS[tname]
-        for (lc, la, lb) in [(0, 0, 1), (1, 1, 0)]:
+        for (lc, la, lb) in [l for l in [(0, 0, 1), (1, 1, 0), (1, 0, 1)] if built_for(v, *l)][:2]:
             A = np.concatenate([O.init_matrix(M, K, la, din, seed=30 + b) for b in range(batch)])
             B = np.concatenate([O.init_matrix(K, N, lb, din, seed=60 + b) for b in range(batch)])
             gpu = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout, batch=batch,
@@ -254,8 +264,8 @@ def test_workgroups_that_take_several_tiles_agree_with_oracle(loader):
                     check_against_oracle(gpu[b * M * N:(b + 1) * M * N], A[b * M * K:(b + 1) * M * K],
                                          B[b * K * N:(b + 1) * K * N], M, N, K, lc, la, lb, din, dout)
                 except AssertionError as e:
-                    raise AssertionError(f"{M}x{N}x{K} batch {b}/{batch} split {split} layouts "
-                                         f"C{lc} A{la} B{lb} {tname}: {e}") from None
+                    raise AssertionError(f"variant {v.index} {M}x{N}x{K} batch {b}/{batch} split {split} "
+                                         f"layouts C{lc} A{la} B{lb} {tname}: {e}") from None
 
 
 def test_degenerate_arguments(loader):
