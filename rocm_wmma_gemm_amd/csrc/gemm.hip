@@ -227,6 +227,24 @@ int staged_fallback(const variant_desc& v)
     return 0;
 }
 
+// A direct-to-LDS variant other than the persistent kernel with the same workgroup tile
+// (the 16x16x32 ping-pong kernel first), else what staged_fallback gives.
+int elementwise_store_variant(const variant_desc& v)
+{
+    for(int pipeline : {4, 2, 3, 1})
+    {
+        for(int i = 0; i < num_variants; ++i)
+        {
+            const variant_desc& w = variant_table[i];
+            if(w.pipeline == pipeline && w.block_m == v.block_m && w.block_n == v.block_n)
+            {
+                return i;
+            }
+        }
+    }
+    return staged_fallback(v);
+}
+
 size_t round_up(size_t x, size_t to)
 {
     return (x + to - 1) / to * to;
@@ -269,6 +287,23 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
     size_t      ldb      = p.b_kmajor ? p.K : p.N;
     size_t      k_kernel = p.K;
     size_t      stride_a = p.stride_a, stride_b = p.stride_b;
+    if(variant_table[plan.variant].pipeline == 5)
+    {
+        // The persistent kernel stores C in 16-byte pieces through a buffer descriptor per
+        // tile: every row of C must start on 16 bytes and hold whole pieces, and a tile's
+        // rows must span less than 2 GiB.  Anything else goes to a kernel with the same
+        // tile that stores element by element.
+        const bool c_pieces = aligned16(p.C) && p.N % 8 == 0 && (p.batch == 1 || p.stride_c % 8 == 0)
+                              && p.N < (size_t{1} << 21);
+        if(!c_pieces)
+        {
+            plan.variant = elementwise_store_variant(variant_table[plan.variant]);
+            if(plan.split_k == -1)
+            {
+                plan.split_k = 1;
+            }
+        }
+    }
     int         mode     = pick_mode(p, variant_table[plan.variant], plan.split_k);
     size_t      pack_bytes = 0;
     bool        packed     = false;
@@ -286,6 +321,14 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
             {
                 mode = static_cast<int>(device::load_mode::vec_guarded);
             }
+        }
+        else if(dv.pipeline == 5 && mode == static_cast<int>(device::load_mode::vec_guarded)
+                && p.K % dv.block_k == 0 && spans_fit(dv, p.a_kmajor, p.b_kmajor, lda, ldb))
+        {
+            // Ragged M or N only, rows aligned: the persistent kernel takes the operands as
+            // they are.  Its buffer descriptors end at the operands' ends, tiles that hang
+            // over an edge read zeros or neighbouring data there, and the guarded stores
+            // leave those rows and columns out.
         }
         else
         {

@@ -157,12 +157,25 @@ struct solo_gemm
         return (const InT*)(((unsigned long long)hi << 32) | lo);
     }
 
-    // 128-bit buffer descriptor of a tile: base = its origin, no stride, no range check
-    // that could fire (every tile span fits 32 bits: the host checks), raw 32-bit format.
-    __device__ __forceinline__ static u32x4 descriptor(const InT* origin)
+    // 128-bit buffer descriptor of a tile: base = its origin, no stride, raw 32-bit format,
+    // and a range that ends where the operand's allocation ends (`end`), so that a tile
+    // that hangs over the edge of a ragged matrix cannot read past it: a load beyond the
+    // range, whether through the vector or the scalar offset, writes zeros to LDS
+    // (mfma_probe --range).  Rows or columns past the edge but inside the allocation
+    // read whatever is there (the next k row, the next batch entry); they only reach
+    // accumulators of rows and columns of C that the guarded stores leave out.  Every
+    // tile span fits 32 bits (the host checks).
+    __device__ __forceinline__ static u32x4 descriptor(const InT* origin, const InT* end)
     {
         const unsigned long long p = (unsigned long long)origin;
-        return u32x4{(unsigned int)p, (unsigned int)(p >> 32) & 0xffffu, 0xffffffffu, 0x00020000u};
+        unsigned int             records = 0xffffffffu;
+        if constexpr(GUARD_C)
+        {
+            // (whole tiles of a matrix of whole tiles end inside it anyway)
+            const unsigned long long left = (unsigned long long)end - p;
+            records                       = left > 0xffffffffull ? 0xffffffffu : (unsigned int)left;
+        }
+        return u32x4{(unsigned int)p, (unsigned int)(p >> 32) & 0xffffu, records, 0x00020000u};
     }
 
     // One MFMA and, in its shadow, one global -> LDS load: M0 (the load's LDS
@@ -207,8 +220,10 @@ struct solo_gemm
                                                      const u32x4& rsrc,
                                                      unsigned int soff)
     {
+        // (the compiler does not look for hazards around inline assembly: four wait
+        // states cover a descriptor or offset that a v_readfirstlane has just written)
         asm volatile("s_add_u32 m0, %[ldsb], %[imm]\n\t"
-                     "s_nop 0\n\t"
+                     "s_nop 4\n\t"
                      "buffer_load_dwordx4 %[voff], %[rsrc], %[soff] offen lds"
                      :
                      : [ldsb] "s"(lds_block), [imm] "n"(LDS_IMM), [voff] "v"(voff), [rsrc] "s"(rsrc),
@@ -387,9 +402,37 @@ struct solo_gemm
         }
     }
 
-    template<bool STREAM, class DstT>
-    __device__ __forceinline__ static void write_out_staged(
-        f32x4 (&acc)[TM][TN], DstT* D, long long pitch, int row_w, int col_w, int lane, lds_char_ptr strip)
+    // The stores are buffer stores relative to the tile's origin: the part of the address
+    // that is the same for the whole wave goes into the scalar offset, the lane's part is
+    // computed once per call, and a lane whose piece lies in a row >= rows or a column >=
+    // cols of the tile (GUARDED: a tile on a ragged edge) gets an offset beyond the
+    // descriptor's 2 GiB range, so the hardware drops its store: no branch, the same code
+    // for every tile.  cols is a multiple of a piece's width (the host sends a C whose
+    // rows are not 16-byte aligned, or whose width is no multiple of 8, to another
+    // kernel), so a piece lies inside or outside as a whole; a tile's rows span less than
+    // 2 GiB (the host checks), so scalar + vector offset neither wraps nor, for a dropped
+    // lane, comes back into range.
+    static constexpr unsigned int STORE_RANGE = 0x80000000u;
+
+    // (the compiler's own buffer store: it knows how long the store reads its data
+    // registers and keeps the next write to them away)
+    template<bool STREAM>
+    __device__ __forceinline__ static void store_piece(const u32x4& v, unsigned int lane_offset,
+                                                       __amdgpu_buffer_rsrc_t rsrc, unsigned int wave_offset)
+    {
+        __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, lane_offset, wave_offset, STREAM ? 2 : 0); // 2 = nt
+    }
+
+    template<bool STREAM, bool GUARDED, class DstT>
+    __device__ __forceinline__ static void write_out_staged(f32x4 (&acc)[TM][TN],
+                                                            DstT*        tile, // element (0, 0) of the workgroup's tile
+                                                            long long    pitch,
+                                                            int          rows, // of the tile that exist
+                                                            int          cols,
+                                                            int          row_w, // the wave's corner in the tile
+                                                            int          col_w,
+                                                            int          lane,
+                                                            lds_char_ptr strip)
     {
         // a strip row holds ROW_BYTES: all columns of the wave tile for a 16-bit
         // destination, half of them for fp32
@@ -398,19 +441,32 @@ struct solo_gemm
         constexpr int TILES   = TN / PASSES; // 16-column tiles per pass
         constexpr int CHUNKS  = ROW_BYTES / 16; // 16-byte pieces of a strip row
         constexpr int READS   = 16 * CHUNKS / 64; // store instructions per pass
+        constexpr int PIECE   = 16 / (int)sizeof(DstT); // elements of a piece
         static_assert(16 * CHUNKS % 64 == 0, "the strip divides over the lanes");
         typedef DstT out4 __attribute__((ext_vector_type(4)));
-        using lds_out4 = __attribute__((address_space(3))) out4;
+        using lds_out4  = __attribute__((address_space(3))) out4;
         using lds_u32x4 = __attribute__((address_space(3))) u32x4;
-        const int r16 = lane & 15, g = lane >> 4;
-        int       strip_at[READS]; // this lane's piece of read q: byte offset in the strip,
-        long long dest_at[READS]; // and element offset in D from the row block's origin
+        // (the tile's origin is the same in every lane; see scalar_pointer)
+        const unsigned long long base = (unsigned long long)tile;
+        // (readfirstlane returns a signed int: through unsigned int, or the low half's
+        // sign bit smears over the high half)
+        const unsigned int lo = (unsigned int)__builtin_amdgcn_readfirstlane((unsigned int)base);
+        const unsigned int hi = (unsigned int)__builtin_amdgcn_readfirstlane((unsigned int)(base >> 32));
+        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            (void*)(((unsigned long long)hi << 32) | (unsigned long long)lo), 0, (int)STORE_RANGE, 0x00020000);
+        const int                r16 = lane & 15, g = lane >> 4;
+        // this lane's piece of read q: row and column in the 16-row block, strip address,
+        // offset in the destination
+        int          piece_row[READS], piece_col[READS], strip_at[READS];
+        unsigned int piece_off[READS];
 #pragma unroll
         for(int q = 0; q < READS; ++q)
         {
-            const int piece = q * 64 + lane, row = piece / CHUNKS, c = piece % CHUNKS;
-            strip_at[q]     = row * STRIP_PITCH + c * 16;
-            dest_at[q]      = row * pitch + c * (16 / (int)sizeof(DstT));
+            const int piece = q * 64 + lane;
+            piece_row[q]    = piece / CHUNKS;
+            piece_col[q]    = piece % CHUNKS * PIECE;
+            strip_at[q]     = piece_row[q] * STRIP_PITCH + piece % CHUNKS * 16;
+            piece_off[q]    = (unsigned int)((piece_row[q] * pitch + piece_col[q]) * (long long)sizeof(DstT));
         }
 #pragma unroll
         for(int i = 0; i < TM; ++i)
@@ -431,20 +487,19 @@ struct solo_gemm
                     *reinterpret_cast<lds_out4*>(strip + r16 * STRIP_PITCH + (16 * j + 4 * g) * sizeof(DstT)) = o;
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                DstT* const block = D + (long long)(row_w + 16 * i) * pitch + col_w + p * TILES * 16;
+                const int          row0 = row_w + 16 * i, col0 = col_w + p * TILES * 16; // of the block
+                const unsigned int wave_offset = __builtin_amdgcn_readfirstlane(
+                    (unsigned int)((row0 * pitch + col0) * (long long)sizeof(DstT)));
 #pragma unroll
                 for(int q = 0; q < READS; ++q)
                 {
-                    const u32x4  v  = *reinterpret_cast<lds_u32x4*>(strip + strip_at[q]);
-                    u32x4* const to = reinterpret_cast<u32x4*>(block + dest_at[q]);
-                    if constexpr(STREAM)
+                    const u32x4  v      = *reinterpret_cast<lds_u32x4*>(strip + strip_at[q]);
+                    unsigned int offset = piece_off[q];
+                    if constexpr(GUARDED)
                     {
-                        __builtin_nontemporal_store(v, to);
+                        offset = row0 + piece_row[q] < rows && col0 + piece_col[q] < cols ? offset : STORE_RANGE;
                     }
-                    else
-                    {
-                        *to = v;
-                    }
+                    store_piece<STREAM>(v, offset, rsrc, wave_offset);
                 }
                 asm volatile("" ::: "memory");
             }
@@ -571,25 +626,18 @@ struct solo_gemm
     {
         if(x.partial == nullptr)
         {
-            OutT* C = static_cast<OutT*>(args.C) + x.batch * args.batch_stride_c;
-            if constexpr(!GUARD_C)
-            {
-                write_out_staged<true>(acc, C, args.N, x.row0 + row_w, x.col0 + col_w, lane, strip);
-            }
-            else
-            {
-                write_out<MI, GUARD_C>(acc, C, args.M, args.N, args.N, x.row0 + row_w, x.col0 + col_w, lane);
-            }
-        }
-        else if constexpr(!GUARD_C)
-        {
-            // the reduce kernel reads these next: no streaming hint
-            write_out_staged<false>(acc, x.partial, x.pitch, x.row0 + row_w, x.col0 + col_w, lane, strip);
+            OutT* C = static_cast<OutT*>(args.C) + x.batch * args.batch_stride_c + (long long)x.row0 * args.N + x.col0;
+            write_out_staged<true, GUARD_C>(acc, C, args.N, args.M - x.row0, args.N - x.col0, row_w, col_w, lane,
+                                            strip);
         }
         else
         {
-            write_out<MI, GUARD_C>(
-                acc, x.partial, args.M, args.N, x.pitch, x.row0 + row_w, x.col0 + col_w, lane);
+            // The reduce kernel reads these next: no streaming hint.  A tile of its own
+            // has nothing to leave out; whole planes of a ragged C do.
+            const bool own_tile = args.tail_begin != 0 || args.stream_units != 0;
+            write_out_staged<false, GUARD_C>(acc, x.partial + (long long)x.row0 * x.pitch + x.col0, x.pitch,
+                                             own_tile ? BM : args.M - x.row0, own_tile ? BN : args.N - x.col0,
+                                             row_w, col_w, lane, strip);
         }
     }
 
@@ -639,6 +687,12 @@ struct solo_gemm
         la.init(wave, lane, a_ld);
         lb.init(wave, lane, b_ld);
 
+        // one past the last element of each operand (all batch entries)
+        const InT* const a_end = static_cast<const InT*>(args.A) + (args.batches - 1) * args.batch_stride_a
+                                 + (long long)(A_KMAJOR ? args.M : args.K) * a_ld;
+        const InT* const b_end = static_cast<const InT*>(args.B) + (args.batches - 1) * args.batch_stride_b
+                                 + (long long)(B_KMAJOR ? args.N : args.K) * b_ld;
+
         work_item cur = decode(args, wk, wk.begin);
 
         // The stream of K tiles the loads follow; it runs two tiles ahead of the MFMAs.
@@ -683,10 +737,10 @@ struct solo_gemm
         u32x4 fa[2][TM], fb[2][TN];
         // prologue: tile 0 and the first part of tile 1 on their way, tile 0 landed
         issue_loads(std::make_integer_sequence<int, VM_LOADS>{}, la, lb, wave_block,
-                    descriptor(a_src), descriptor(b_src));
+                    descriptor(a_src, a_end), descriptor(b_src, b_end));
         advance();
         issue_loads(std::make_integer_sequence<int, LOADS_B>{}, la, lb, wave_block + STAGE,
-                    descriptor(a_src), descriptor(b_src));
+                    descriptor(a_src, a_end), descriptor(b_src, b_end));
         const InT* a_prev = a_src;
         const InT* b_prev = b_src;
         advance();
@@ -718,9 +772,9 @@ struct solo_gemm
             {
                 const unsigned int there = STAGE - here;
                 const step_ctx c0{oa, ob, la, lb, lds_addr + here, wave_block + there,
-                                  descriptor(a_prev), descriptor(b_prev)};
+                                  descriptor(a_prev, a_end), descriptor(b_prev, b_end)};
                 const step_ctx c1{oa, ob, la, lb, lds_addr + there, wave_block + here,
-                                  descriptor(a_src), descriptor(b_src)};
+                                  descriptor(a_src, a_end), descriptor(b_src, b_end)};
                 __builtin_amdgcn_s_waitcnt(waitcnt_imm(63)); // last step's fragment reads
                 step<1, plan_a>(c0, fa[0], fb[0], fa[1], fb[1], acc);
                 __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));

@@ -4,6 +4,8 @@
 //
 //   mfma_probe            run every check, print PASS/FAIL lines and the ceilings
 //   mfma_probe --dump     additionally print raw lane dumps of the LDS paths
+//   mfma_probe --range    what buffer_load ... lds does past the descriptor's num_records
+//   mfma_probe --read N   time a read-only stream over N MiB (grid size x loads in flight)
 //   mfma_probe --copy N   run only the copy kernel over N MiB (reference point for
 //                         scaling FETCH_SIZE / WRITE_SIZE counters)
 //   mfma_probe --ceiling  run only the sustained MFMA-rate measurement on pseudo-random
@@ -131,6 +133,41 @@ __global__ void lds_dma_dump(const _Float16* src, const int* goff, float* out, i
     }
 }
 
+// ---- 3b. range check of buffer_load_dwordx4 ... offen lds -----------------------
+// Four loads of one wave through a raw buffer descriptor (stride 0) whose num_records
+// is `records` bytes, into four 1 KiB LDS blocks that start out as -1:
+//   block 0: voffset = 16*lane,                   soffset = 0
+//   block 1: voffset = 16*lane + voff_shift,      soffset = 0
+//   block 2: voffset = 16*lane,                   soffset = soff_shift
+//   block 3: voffset = 16*lane + voff_shift / 2,  soffset = 0
+// The source holds element value = element index, and every address used lies inside
+// it whatever the descriptor says.
+__global__ void range_check_dump(const _Float16* src, float* out, unsigned records, unsigned voff_shift,
+                                 unsigned soff_shift)
+{
+    __shared__ __attribute__((aligned(1024))) _Float16 lds[2048];
+    for(int i = threadIdx.x; i < 2048; i += 64)
+    {
+        lds[i] = (_Float16)-1.0f;
+    }
+    __syncthreads();
+    const unsigned long long p    = (unsigned long long)src;
+    const u32x4              rsrc = {(unsigned)p, (unsigned)(p >> 32) & 0xffffu, records, 0x00020000u};
+    const unsigned           base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
+    const unsigned           v0 = 16 * threadIdx.x, v1 = v0 + voff_shift, v3 = v0 + voff_shift / 2;
+    const unsigned           zero = 0;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(base), "v"(v0), "s"(rsrc), "s"(zero) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(base + 1024), "v"(v1), "s"(rsrc), "s"(zero) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(base + 2048), "v"(v0), "s"(rsrc), "s"(soff_shift) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(base + 3072), "v"(v3), "s"(rsrc), "s"(zero) : "memory");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    for(int i = threadIdx.x; i < 2048; i += 64)
+    {
+        out[i] = (float)lds[i];
+    }
+}
+
 // ---- 4. MFMA issue ceiling ------------------------------------------------------
 template<int CHAINS>
 __global__ void __launch_bounds__(256) mfma_peak(float* out, int iters)
@@ -180,6 +217,36 @@ __global__ void __launch_bounds__(256) copy_kernel(u32x4* __restrict__ dst, cons
     }
 }
 
+
+// ---- 5b. read-only stream (what a skinny, operand-streaming GEMM can reach) -----
+// Each thread keeps UNROLL independent 16-byte loads in flight and folds them into one
+// value, so nothing is written but one word per thread.
+template<int UNROLL>
+__global__ void __launch_bounds__(256) read_kernel(unsigned* __restrict__ out, const u32x4* __restrict__ src, size_t n)
+{
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    u32x4        acc  = {0u, 0u, 0u, 0u};
+    size_t       i    = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for(; i + (UNROLL - 1) * step < n; i += UNROLL * step)
+    {
+        u32x4 v[UNROLL];
+#pragma unroll
+        for(int u = 0; u < UNROLL; ++u)
+        {
+            v[u] = src[i + u * step];
+        }
+#pragma unroll
+        for(int u = 0; u < UNROLL; ++u)
+        {
+            acc ^= v[u];
+        }
+    }
+    for(; i < n; i += step)
+    {
+        acc ^= src[i];
+    }
+    out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = acc.x ^ acc.y ^ acc.z ^ acc.w;
+}
 
 // ---- 6. LDS read throughput under a given per-lane address pattern ------------
 // Every lane issues `iters` x 8 reads at its own fixed byte address (plus a per-read
@@ -589,7 +656,8 @@ int main(int argc, char** argv)
     bool   dump     = false;
     bool   ceiling  = false;
     bool   lds_groups = false;
-    size_t copy_mib = 0;
+    size_t copy_mib = 0, read_mib = 0;
+    bool   range_check = false;
     for(int i = 1; i < argc; ++i)
     {
         if(!std::strcmp(argv[i], "--dump"))
@@ -600,6 +668,10 @@ int main(int argc, char** argv)
             lds_groups = true;
         if(!std::strcmp(argv[i], "--copy") && i + 1 < argc)
             copy_mib = std::strtoull(argv[++i], nullptr, 10);
+        if(!std::strcmp(argv[i], "--range"))
+            range_check = true;
+        if(!std::strcmp(argv[i], "--read") && i + 1 < argc)
+            read_mib = std::strtoull(argv[++i], nullptr, 10);
     }
     hipDeviceProp_t prop;
     CHECK(hipGetDeviceProperties(&prop, 0));
@@ -771,6 +843,92 @@ int main(int argc, char** argv)
             std::printf("\n");
         }
         std::printf("\n");
+        return 0;
+    }
+
+    if(range_check)
+    {
+        // 8 KiB of source, descriptor says 1 KiB; shifts of 1 KiB
+        std::vector<_Float16> src(4096);
+        for(int i = 0; i < 4096; ++i)
+            src[i] = (_Float16)(float)(i % 2048);
+        _Float16* dSrc;
+        float*    dOut;
+        CHECK(hipMalloc(&dSrc, 8192));
+        CHECK(hipMalloc(&dOut, 2048 * 4));
+        CHECK(hipMemcpy(dSrc, src.data(), 8192, hipMemcpyHostToDevice));
+        range_check_dump<<<1, 64>>>(dSrc, dOut, 1024u, 1024u, 1024u);
+        CHECK(hipDeviceSynchronize());
+        std::vector<float> out(2048);
+        CHECK(hipMemcpy(out.data(), dOut, 2048 * 4, hipMemcpyDeviceToHost));
+        const char* what[4] = {"voffset inside num_records", "voffset past num_records", "soffset past num_records",
+                               "voffset: lanes 0-31 inside, 32-63 past"};
+        for(int b = 0; b < 4; ++b)
+        {
+            int data = 0, zero = 0, untouched = 0, other = 0;
+            for(int l = 0; l < 64; ++l)
+            {
+                const int   src_elem = b == 0 ? 8 * l : b == 3 ? 8 * l + 256 : 8 * l + 512;
+                int         d = 0, z = 0, u = 0;
+                for(int j = 0; j < 8; ++j)
+                {
+                    const float v = out[b * 512 + l * 8 + j];
+                    d += v == (float)((src_elem + j) % 2048);
+                    z += v == 0.0f;
+                    u += v == -1.0f;
+                }
+                // element 0 of the source is 0.0 too: count a lane as data first
+                if(d == 8)
+                    ++data;
+                else if(z == 8)
+                    ++zero;
+                else if(u == 8)
+                    ++untouched;
+                else
+                    ++other;
+            }
+            std::printf("range check, %-40s lanes with data %2d, zeros %2d, LDS untouched %2d, other %2d\n", what[b],
+                        data, zero, untouched, other);
+        }
+        return 0;
+    }
+
+    if(read_mib)
+    {
+        const size_t bytes = read_mib << 20, n = bytes / 16;
+        u32x4*       src;
+        unsigned*    out;
+        CHECK(hipMalloc(&src, bytes));
+        CHECK(hipMalloc(&out, 8192 * 256 * sizeof(unsigned)));
+        CHECK(hipMemset(src, 1, bytes));
+        hipEvent_t e0, e1;
+        CHECK(hipEventCreate(&e0));
+        CHECK(hipEventCreate(&e1));
+        const int grids[] = {512, 1024, 2048, 4096, 8192};
+        for(int g : grids)
+        {
+            for(int unroll = 0; unroll < 3; ++unroll)
+            {
+                float best = 1e30f;
+                for(int rep = 0; rep < 6; ++rep)
+                {
+                    CHECK(hipEventRecord(e0));
+                    if(unroll == 0)
+                        read_kernel<2><<<g, 256>>>(out, src, n);
+                    else if(unroll == 1)
+                        read_kernel<4><<<g, 256>>>(out, src, n);
+                    else
+                        read_kernel<8><<<g, 256>>>(out, src, n);
+                    CHECK(hipEventRecord(e1));
+                    CHECK(hipEventSynchronize(e1));
+                    float ms;
+                    CHECK(hipEventElapsedTime(&ms, e0, e1));
+                    best = ms < best ? ms : best;
+                }
+                std::printf("read %zu MiB, grid %d x 256, %d loads in flight per thread: %.4f ms -> %.2f TB/s\n",
+                            read_mib, g, 2 << unroll, best, (double)bytes / best / 1e9);
+            }
+        }
         return 0;
     }
 

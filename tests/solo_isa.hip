@@ -7,3 +7,5 @@ using namespace rocm_wmma_gemm;
 template __global__ void device::gemm_entry<device::solo_gemm<device::in_kind::f16, _Float16, true, true, 256, 256, 64, 2, 2, 2, false>>(device::gemm_args);
 template __global__ void device::gemm_entry<device::solo_gemm<device::in_kind::bf16, float, false, false, 256, 256, 64, 2, 2, 2, true>>(device::gemm_args);
 template __global__ void device::gemm_entry<device::solo_gemm<device::in_kind::f16, _Float16, true, false, 256, 256, 64, 2, 2, 2, false>>(device::gemm_args);
+template __global__ void device::gemm_entry<device::solo_gemm<device::in_kind::f16, _Float16, true, true, 256, 256, 64, 2, 2, 2, true>>(device::gemm_args);
+template __global__ void device::gemm_entry<device::solo_gemm<device::in_kind::bf16, __bf16, true, true, 256, 192, 64, 2, 2, 2, false>>(device::gemm_args);

@@ -237,6 +237,8 @@ def test_workgroups_that_take_several_tiles_agree_with_oracle(loader):
         (1024, 768, 128, 30, 1),    # 12 tiles x 30 batch entries = 360 items
         (2048, 2304, 320, 2, 2),    # 72 tiles x 2 slices x 2 batch entries = 288 items
         (4344, 4360, 128, 1, 1),    # ragged edges (guarded stores)
+        (392, 648, 256, 3, 1),      # ragged, several batch entries: operands are read as they
+                                    # are, rows past an edge come from the next batch entry
         # split field -1: the workgroups walk by K tile, each over ceil(all K tiles / 256)
         (3072, 3072, 512, 1, -1),   # 1152 K tiles, 5 per workgroup: tiles cut at odd places
         (1536, 1280, 1024, 1, -1),  # 480 K tiles, 2 per workgroup: every tile in 8 parts
