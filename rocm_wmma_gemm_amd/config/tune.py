@@ -79,7 +79,7 @@ def candidates(variants, M, N, K, lc):
         tiles = -(-rows // v.block_m) * -(-cols // v.block_n)
         k_steps = -(-K // v.block_k)
         # a tile much larger than the problem only wastes work
-        if max(v.block_m, v.block_n) >= 192 and (rows < 192 or cols < 192):
+        if (v.block_m >= 192 and rows < 192) or (v.block_n >= 192 and cols < 192):
             continue
         swizzles = [1] if tiles <= 8 else [4, 8, 16]
         splits = [1]

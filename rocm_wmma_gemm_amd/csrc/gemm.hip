@@ -22,9 +22,9 @@ namespace host
 {
 
 // LDS per workgroup: the staged pipeline double-buffers one tile pair; the direct
-// pipeline keeps a ring of 2 (BLOCK_K 64) or 4 (BLOCK_K 32) tile pairs.
+// pipelines keep a ring of 2 (BLOCK_K 64) or 4 (BLOCK_K 32, and pipeline 6) tile pairs.
 #define RWG_VARIANT(IDX, BM, BN, BK, WM, WN, PIPE)                                         \
-    {BM, BN, BK, WM, WN, PIPE, ((PIPE) != 0 && (BK) == 32 ? 4 : 2) * (BM + BN) * BK * 2,   \
+    {BM, BN, BK, WM, WN, PIPE, ((PIPE) == 6 || ((PIPE) != 0 && (BK) == 32) ? 4 : 2) * (BM + BN) * BK * 2,   \
      64 * WM * WN},
 const variant_desc variant_table[num_variants] = {
 #include "variants.def"
@@ -258,15 +258,6 @@ bool spans_fit(const variant_desc& v, bool a_kmajor, bool b_kmajor, size_t lda, 
     return a_span < (1ull << 32) && b_span < (1ull << 32);
 }
 
-// Padding pays when the GEMM is large next to the copy: the copy moves every operand
-// element twice, the GEMM does 2*M*N*K/(M*K + K*N) FLOP per operand element.
-bool padding_pays(const kernel_problem& p)
-{
-    const double flop_per_elem
-        = 2.0 * p.M * p.N * p.K / (static_cast<double>(p.M) * p.K + static_cast<double>(p.K) * p.N);
-    return flop_per_elem >= 256.0 && p.M >= 128 && p.N >= 128 && p.K >= 128;
-}
-
 template<class OutT>
 int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hipStream_t stream)
 {
@@ -306,7 +297,8 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
     }
     int         mode     = pick_mode(p, variant_table[plan.variant], plan.split_k);
     size_t      pack_bytes = 0;
-    bool        packed     = false;
+    bool        packed     = false; // the kernel reads a padded copy of ...
+    bool        copy_a = false, copy_b = false; // ... this operand
 
     if(variant_table[plan.variant].pipeline != 0)
     {
@@ -317,7 +309,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         {
             // The 16x16x32 kernels store 4 elements of C at a time when unguarded.
             const bool c_vec = aligned16(p.C) && (p.batch == 1 || p.stride_c % 8 == 0);
-            if(dv.pipeline >= 3 && !c_vec)
+            if((dv.pipeline == 3 || dv.pipeline == 4) && !c_vec)
             {
                 mode = static_cast<int>(device::load_mode::vec_guarded);
             }
@@ -333,21 +325,34 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         else
         {
             // Ragged or misaligned: run the direct kernel on zero-padded copies when the
-            // problem is big enough to pay for the copy, else take the staged kernel.
+            // problem is big enough to pay for the copy, else take the staged kernel.  Only
+            // an operand that needs it is copied: one whose rows are aligned and whose
+            // extents are whole tiles stays where it is (a skinny GEMM pads its small
+            // operand and streams the big one from where it lies).
             const size_t m_pad = round_up(p.M, dv.block_m), n_pad = round_up(p.N, dv.block_n),
                          k_pad = round_up(p.K, dv.block_k);
+            const bool   strides_ok = p.batch == 1 || (p.stride_a % 8 == 0 && p.stride_b % 8 == 0);
+            copy_a = !(k_pad == p.K && m_pad == p.M && strides_ok && aligned16(p.A)
+                       && (p.a_kmajor ? p.K : p.M) % 8 == 0);
+            copy_b = !(k_pad == p.K && n_pad == p.N && strides_ok && aligned16(p.B)
+                       && (p.b_kmajor ? p.K : p.N) % 8 == 0);
             const size_t pa = m_pad * k_pad, pb = k_pad * n_pad;
-            const size_t plda = p.a_kmajor ? k_pad : m_pad, pldb = p.b_kmajor ? k_pad : n_pad;
-            pack_bytes = round_up((pa + pb) * p.batch * in_bytes, 256);
-            if(padding_pays(p) && spans_fit(dv, p.a_kmajor, p.b_kmajor, plda, pldb)
-               && pack_bytes <= workspace_limit_bytes / 2)
+            const size_t plda = !copy_a ? lda : p.a_kmajor ? k_pad : m_pad;
+            const size_t pldb = !copy_b ? ldb : p.b_kmajor ? k_pad : n_pad;
+            const size_t copied = (copy_a ? pa : 0) + (copy_b ? pb : 0);
+            pack_bytes = round_up(copied * p.batch * in_bytes, 256);
+            // padding pays when the GEMM is large next to the copy, which moves every copied
+            // element twice: at least 256 FLOP per copied element
+            const bool pays = copied > 0 && p.K >= 128
+                              && 2.0 * p.M * p.N * p.K / static_cast<double>(copied) >= 256.0;
+            if(pays && spans_fit(dv, p.a_kmajor, p.b_kmajor, plda, pldb) && pack_bytes <= workspace_limit_bytes / 2)
             {
                 packed   = true;
                 lda      = plda;
                 ldb      = pldb;
                 k_kernel = k_pad;
-                stride_a = pa;
-                stride_b = pb;
+                stride_a = copy_a ? pa : p.stride_a;
+                stride_b = copy_b ? pb : p.stride_b;
                 mode     = static_cast<int>(device::load_mode::vec_guarded); // guarded C stores
             }
             else
@@ -498,7 +503,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
     if(packed)
     {
         auto* wa = reinterpret_cast<unsigned short*>(workspace);
-        auto* wb = wa + stride_a * p.batch;
+        auto* wb = wa + (copy_a ? stride_a * p.batch : 0);
         // operand as a 2-D array: `outer` rows of `inner` contiguous elements
         const size_t a_outer = p.a_kmajor ? p.M : p.K, a_inner = p.a_kmajor ? p.K : p.M;
         const size_t b_outer = p.b_kmajor ? p.N : p.K, b_inner = p.b_kmajor ? p.K : p.N;
@@ -506,23 +511,35 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         for(size_t b0 = 0; b0 < p.batch; b0 += 65535)
         {
             const unsigned nb = static_cast<unsigned>(std::min<size_t>(65535, p.batch - b0));
-            const dim3 ga(static_cast<unsigned>(std::min<size_t>((lda / 2 + 255) / 256, 64)),
-                          static_cast<unsigned>(std::min<size_t>(a_outer_pad, 65535)), nb);
-            device::pack_padded<unsigned short><<<ga, dim3(256), 0, stream>>>(
-                static_cast<const unsigned short*>(p.A) + b0 * p.stride_a, wa + b0 * stride_a,
-                static_cast<int>(a_outer), static_cast<int>(a_inner), static_cast<int>(a_outer_pad),
-                static_cast<int>(lda), static_cast<long long>(p.stride_a),
-                static_cast<long long>(stride_a));
-            const dim3 gb(static_cast<unsigned>(std::min<size_t>((ldb / 2 + 255) / 256, 64)),
-                          static_cast<unsigned>(std::min<size_t>(b_outer_pad, 65535)), nb);
-            device::pack_padded<unsigned short><<<gb, dim3(256), 0, stream>>>(
-                static_cast<const unsigned short*>(p.B) + b0 * p.stride_b, wb + b0 * stride_b,
-                static_cast<int>(b_outer), static_cast<int>(b_inner), static_cast<int>(b_outer_pad),
-                static_cast<int>(ldb), static_cast<long long>(p.stride_b),
-                static_cast<long long>(stride_b));
+            if(copy_a)
+            {
+                const dim3 ga(static_cast<unsigned>(std::min<size_t>((lda / 2 + 255) / 256, 64)),
+                              static_cast<unsigned>(std::min<size_t>(a_outer_pad, 65535)), nb);
+                device::pack_padded<unsigned short><<<ga, dim3(256), 0, stream>>>(
+                    static_cast<const unsigned short*>(p.A) + b0 * p.stride_a, wa + b0 * stride_a,
+                    static_cast<int>(a_outer), static_cast<int>(a_inner), static_cast<int>(a_outer_pad),
+                    static_cast<int>(lda), static_cast<long long>(p.stride_a),
+                    static_cast<long long>(stride_a));
+            }
+            if(copy_b)
+            {
+                const dim3 gb(static_cast<unsigned>(std::min<size_t>((ldb / 2 + 255) / 256, 64)),
+                              static_cast<unsigned>(std::min<size_t>(b_outer_pad, 65535)), nb);
+                device::pack_padded<unsigned short><<<gb, dim3(256), 0, stream>>>(
+                    static_cast<const unsigned short*>(p.B) + b0 * p.stride_b, wb + b0 * stride_b,
+                    static_cast<int>(b_outer), static_cast<int>(b_inner), static_cast<int>(b_outer_pad),
+                    static_cast<int>(ldb), static_cast<long long>(p.stride_b),
+                    static_cast<long long>(stride_b));
+            }
         }
-        a_ptr = wa;
-        b_ptr = wb;
+        if(copy_a)
+        {
+            a_ptr = wa;
+        }
+        if(copy_b)
+        {
+            b_ptr = wb;
+        }
     }
 
     kernel_fn fn = lookup_kernel(type_idx, p.a_kmajor, p.b_kmajor, plan.variant, mode);

@@ -23,7 +23,7 @@ using out_t = std::conditional<RWG_TYPE == 0, _Float16,
 template<int BM, int BN, int BK, int WM, int WN, int PIPE, device::load_mode MODE>
 constexpr kernel_fn entry()
 {
-    static_assert(PIPE >= 0 && PIPE <= 5, "unknown pipeline");
+    static_assert(PIPE >= 0 && PIPE <= 6, "unknown pipeline");
     if constexpr(PIPE == 0)
     {
         return &device::gemm_entry<
@@ -62,6 +62,12 @@ constexpr kernel_fn entry()
         return &device::gemm_entry<
             device::solo_gemm<kIn, out_t, RWG_AK != 0, RWG_BK != 0, BM, BN, BK, WM, WN,
                               (BK == 64 ? 2 : 4), MODE == device::load_mode::vec_guarded>>;
+    }
+    else if constexpr(MODE != device::load_mode::scalar && PIPE == 6
+                      && (BM % 128 == 0 || RWG_AK != 0) && (BN % 128 == 0 || RWG_BK != 0))
+    {
+        return &device::gemm_entry<device::direct_gemm<kIn, out_t, RWG_AK != 0, RWG_BK != 0, BM, BN, BK, WM, WN, 4,
+                                                       MODE == device::load_mode::vec_guarded>>;
     }
     else
     {

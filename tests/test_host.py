@@ -136,6 +136,20 @@ def test_generator_rejects_unknown_variant_and_roundtrips(tmp_path):
     assert "{64, 64, 64, 0, 0, 1, 0, {0, 16, 1}}" in text
 
 
+def test_split_fields_of_a_config_entry():
+    """split_k: every tile cut; tail_split: only the last partial wave of tiles (negative
+    field); stream_k: the persistent kernel's walk by K tile (-1)."""
+    sys.path.insert(0, os.path.join(ROOT, "rocm_wmma_gemm_amd", "config"))
+    import generate_config as G
+
+    assert G.split_field({}) == 1
+    assert G.split_field({"split_k": 8}) == 8
+    assert G.split_field({"split_k": 1, "tail_split": 3}) == -3
+    assert G.split_field({"split_k": 1, "tail_split": 1}) == 1
+    assert G.split_field({"split_k": 1, "stream_k": 1}) == -1
+    assert G.split_field({"split_k": 4, "stream_k": 0}) == 4
+
+
 def test_shipped_json_matches_reference_schema():
     import json
 
