@@ -35,6 +35,8 @@
 #ifndef ROCM_WMMA_GEMM_DIRECT_KERNEL_HPP
 #define ROCM_WMMA_GEMM_DIRECT_KERNEL_HPP
 
+#include <utility>
+
 #include "gemm_kernel.hpp"
 
 // Cache-policy bits of the global -> LDS loads (0 = default: cached in L1 and L2).
@@ -360,6 +362,29 @@ struct direct_gemm
         return (vmcnt & 15) | (7 << 4) | (0 << 8) | ((vmcnt >> 4) << 14);
     }
 
+    // With an operand that is contiguous along M or N the fragment reads are volatile
+    // inline assembly: behind a global -> LDS load the compiler puts s_waitcnt vmcnt(0) in
+    // front of every ds_read_b64_tr_b16 it knows of, which waits for the loads of the
+    // tiles further down the ring too and leaves the ring one tile deep in effect (at
+    // 2048^3 the M/N-contiguous layouts ran 20-30 % behind the K-contiguous one, more
+    // with a ring of 4).  The compiler does not track these reads, so each call first
+    // waits for the reads of the call before it, whose fragments the MFMAs that follow
+    // this call consume, and the caller waits once more behind the K loop.
+    static constexpr bool PINNED_READS = !A_KMAJOR || !B_KMAJOR;
+
+    template<int KKI, int... I, int... J>
+    __device__ __forceinline__ static void read_pinned(std::integer_sequence<int, I...>,
+                                                       std::integer_sequence<int, J...>,
+                                                       const op_a&  oa,
+                                                       const op_b&  ob,
+                                                       unsigned int stage,
+                                                       u32x4 (&fa)[TM],
+                                                       u32x4 (&fb)[TN])
+    {
+        ((fa[I] = oa.template fragment_pinned<I, KKI>(stage)), ...);
+        ((fb[J] = ob.template fragment_pinned<J, KKI>(stage + A_BYTES)), ...);
+    }
+
     __device__ __forceinline__ static void load_fragments(const op_a& oa,
                                                           const op_b& ob,
                                                           lds_char_ptr stage,
@@ -367,15 +392,44 @@ struct direct_gemm
                                                           u32x4 (&fa)[TM],
                                                           u32x4 (&fb)[TN])
     {
-#pragma unroll
-        for(int i = 0; i < TM; ++i)
+        if constexpr(PINNED_READS)
         {
-            fa[i] = oa.fragment(stage, i, kk);
+            static_assert(KK <= 4, "one case per K step below");
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0); // no MFMA of this phase in front of the wait
+            const unsigned int addr = (unsigned int)(size_t)stage;
+            constexpr auto     sa = std::make_integer_sequence<int, TM>{};
+            constexpr auto     sb = std::make_integer_sequence<int, TN>{};
+            // kk is a constant after unrolling
+            if(kk == 0)
+            {
+                read_pinned<0>(sa, sb, oa, ob, addr, fa, fb);
+            }
+            else if(kk == 1)
+            {
+                read_pinned<1 % KK>(sa, sb, oa, ob, addr, fa, fb);
+            }
+            else if(kk == 2)
+            {
+                read_pinned<2 % KK>(sa, sb, oa, ob, addr, fa, fb);
+            }
+            else
+            {
+                read_pinned<3 % KK>(sa, sb, oa, ob, addr, fa, fb);
+            }
         }
-#pragma unroll
-        for(int j = 0; j < TN; ++j)
+        else
         {
-            fb[j] = ob.fragment(stage + A_BYTES, j, kk);
+#pragma unroll
+            for(int i = 0; i < TM; ++i)
+            {
+                fa[i] = oa.fragment(stage, i, kk);
+            }
+#pragma unroll
+            for(int j = 0; j < TN; ++j)
+            {
+                fb[j] = ob.fragment(stage + A_BYTES, j, kk);
+            }
         }
     }
 
@@ -599,8 +653,11 @@ struct direct_gemm
                 a_src = a_src + a_step > a_last ? a_last : a_src + a_step;
                 b_src = b_src + b_step > b_last ? b_last : b_src + b_step;
             }
-            // redundant tail loads may still be in flight
+            // redundant tail loads, and the last fragment reads (nobody uses them, but they
+            // must not land in registers that hold something else by then), may still be
+            // in flight
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+            __builtin_amdgcn_sched_barrier(0);
         }
 
         if(w.slices == 1)

@@ -1,18 +1,19 @@
-// One-wave-per-SIMD MFMA GEMM kernel for gfx950 (4 waves, 128 x 128 wave tiles).
+// One-wave-per-SIMD MFMA GEMM kernel for gfx950 (4 waves, 128 x 128 wave tiles; also
+// 96-wide ones), with persistent workgroups.
 //
-// Same data path as the direct kernel (direct_kernel.hpp: global -> LDS with
-// global_load_lds_dwordx4, swizzled LDS layouts, ds_read_b64_tr_b16 for operands that
-// are contiguous along M or N) on the 16x16x32 MFMA, but with the largest wave tile
-// the register file allows: 128 x 128 per wave = 256 accumulator registers, all of
-// the AGPRs.  A wave then reads 16 operand fragments from LDS per 64 MFMAs, against
-// 12 per 32 for the 128 x 64 wave tiles of the 8-wave kernels: one third fewer LDS
-// bytes per FLOP, which is what the power-capped clock responds to.
+// Same LDS layouts as the direct kernel (direct_kernel.hpp: swizzled K-contiguous rows,
+// ds_read_b64_tr_b16 for operands that are contiguous along M or N) on the 16x16x32
+// MFMA, but with the largest wave tile the register file allows: 128 x 128 per wave =
+// 256 accumulator registers, all of the AGPRs.  A wave then reads 16 operand fragments
+// from LDS per 64 MFMAs, against 12 per 32 for the 128 x 64 wave tiles of the 8-wave
+// kernels: one third fewer LDS bytes per FLOP, which is what the power-capped clock
+// responds to.
 //
 // With one wave per SIMD nothing hides a stall, so the schedule is fixed by hand:
 // the MFMAs are volatile inline assembly (which also pins every accumulator to its
 // AGPRs: with the builtin the register allocator moved accumulators between the two
-// register files inside the loop), and the LDS reads and global -> LDS loads of a K
-// step sit between them in source order.
+// register files inside the loop), and the LDS reads and global -> LDS loads (buffer
+// loads, also inline assembly) of a K step sit between them in source order.
 //
 // Ring of 2 tiles of BLOCK_K 64 (two MFMA K steps per tile, one barrier per tile;
 // K-contiguous rows are 128 bytes, so every load fetches whole cache lines).  The
@@ -22,6 +23,11 @@
 // 1117 + 1186 cycles for the two steps of a tile (1024 each would be MFMA-bound) plus
 // about 70 in the wait and the barrier, where issuing a tile's loads back to back
 // had cost 1700-1900 cycles for the second step.
+//
+// A launch has one workgroup per CU; each works through its tiles (or K slices, or a
+// range of K tiles: see walk) with one load stream running through all of them, and
+// stores C through per-wave LDS strips as 16-byte buffer stores.  Loads and stores go
+// through buffer descriptors whose range check handles the ragged edges of a matrix.
 //
 // Role with respect to the reference: as the other kernels, its gemm_impl (reference
 // rocm_wmma_gemm/include/rocm_wmma_gemm/kernel/kernel.hpp:108-556).
