@@ -247,3 +247,33 @@ def test_hand_scheduled_kernel_keeps_accumulators_in_place(tmp_path):
                         break
                 n += 1
         assert checked >= 1, func
+
+
+def test_tile_ring_of_the_direct_kernels_stays_deep_for_transposed_operands(tmp_path):
+    """Behind a global -> LDS load the compiler waits for ALL outstanding loads (s_waitcnt
+    vmcnt(0)) in front of every ds_read_b64_tr_b16 it knows of, which empties the ring of
+    prefetched tiles at every K step.  The kernels read those fragments through inline
+    assembly instead; their MFMA loops must hold the transposing reads and no wait for
+    vmcnt(0) other than the ring-of-2 kernel's own at its barrier."""
+    hipcc = "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not found")
+    asm = tmp_path / "direct_isa.s"
+    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature",
+           "-Xclang", "-packed-fp32-ops", "-I" + os.path.join(ROOT, "rocm_wmma_gemm_amd", "csrc"),
+           "-S", "--cuda-device-only", "-o", str(asm), os.path.join(ROOT, "tests", "direct_isa.hip")]
+    subprocess.run(cmd, check=True, capture_output=True, timeout=600)
+    loops = {}
+    for f, body in _mfma_loops(asm.read_text()):
+        if "direct_gemm" in f and (f not in loops or len(body) < len(loops[f])):
+            loops[f] = body
+    assert len(loops) == 2
+    for func, body in loops.items():
+        assert any("ds_read_b64_tr_b16" in b for b in body), func
+        # the only such wait that belongs there is the ring-of-2 kernel's own, in front
+        # of the barrier at which the next tile must have landed
+        code = [b.strip() for b in body if b.startswith("\t") and not b.strip().startswith((";", "."))]
+        waits = [n for n, b in enumerate(code) if re.search(r"s_waitcnt.*vmcnt\(0\)", b)]
+        stray = [code[n] for n in waits if not code[n + 1].startswith("s_barrier")]
+        assert not stray, f"{func}: {stray}"
+        assert len(waits) <= 1, func
