@@ -111,6 +111,168 @@ launch_plan heuristic_plan(size_t m, size_t n, size_t k, int lc)
     return plan;
 }
 
+namespace
+{
+// Compiled variants as the model sees them.
+struct model_variant
+{
+    int block_m, block_n, block_k, waves_m, waves_n, pipeline;
+};
+#define RWG_VARIANT(IDX, BM, BN, BK, WM, WN, PIPE) {BM, BN, BK, WM, WN, PIPE},
+const model_variant model_variants[] = {
+#include "variants.def"
+};
+#undef RWG_VARIANT
+
+// Microseconds per K tile of 64 with every CU of an MI355X at work, and per tile for
+// its stores, read off the tuner's measurements (persistent 16x16x32 kernel at 4096^3
+// to 8192^3 and 3072^3; ring-of-4 direct kernel at 2048^3 and the skinny shapes).
+bool step_cost(const model_variant& v, double* step_us, double* item_us)
+{
+    if(v.block_k != 64)
+    {
+        return false;
+    }
+    const int area = v.block_m * v.block_n;
+    if(v.pipeline == 5)
+    {
+        *step_us = area == 256 * 256 ? 1.30 : area == 256 * 192 ? 1.05 : area == 192 * 192 ? 0.90 : 0.0;
+        *item_us = 5.0;
+        return *step_us > 0.0;
+    }
+    if(v.pipeline == 6)
+    {
+        *step_us = area == 128 * 128 ? 0.60 : area == 64 * 256 ? 0.50 : 0.0;
+        *item_us = 2.0;
+        return *step_us > 0.0;
+    }
+    return false;
+}
+
+size_t ceil_div(size_t a, size_t b)
+{
+    return (a + b - 1) / b;
+}
+} // namespace
+
+// A plan from arithmetic instead of from the nearest tuned shape: for every compiled
+// variant of the two pipelines that serve regular shapes, and every way to split, the
+// time is estimated as launch + waves of tiles over the CUs x (K tiles x time per K
+// tile + stores) + what the split costs in partial sums, and the cheapest wins.  What
+// the nearest tuned shape cannot know is how THIS shape's tile count falls on 256 CUs:
+// 3584^3 next to the tuned 3072^3 inherited its 192 x 192 tiles (361 of them, two waves
+// with the second less than half full) and ran at 0.7 of the 196 tiles of 256 x 256.
+// On the 208 tuned entries the model can serve, its pick is on average 2.7 % slower than
+// the tuner's, 25 % at worst.
+bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_plan* out)
+{
+    const size_t rows = lc == 0 ? m : n;
+    const size_t cols = lc == 0 ? n : m;
+    // operands in kernel space: a column-major C runs as the transposed problem
+    bool a_kmajor = la == 0, b_kmajor = lb == 1;
+    if(lc != 0)
+    {
+        const bool t = a_kmajor;
+        a_kmajor     = b_kmajor;
+        b_kmajor     = t;
+    }
+    if(k < 64 || k % 64 != 0 || rows % 8 != 0 || cols % 8 != 0 || rows < 16 || cols < 16)
+    {
+        return false; // shapes the direct kernels would only take through padded copies
+    }
+    constexpr size_t cus           = 256;
+    constexpr double launch_us     = 6.0;
+    constexpr double reduce_us     = 4.0;
+    constexpr double plane_bytes_per_us = 2.2e6; // partial planes: written, then read by reduce_partials
+    constexpr double tile_bytes_per_us  = 3.7e6; // partial tiles (split tail, walk by K tile)
+    const size_t     kt            = k / 64;
+    double           best          = 0.0;
+    bool             found         = false;
+    const int        count         = static_cast<int>(sizeof(model_variants) / sizeof(model_variants[0]));
+    for(int i = 0; i < count; ++i)
+    {
+        const model_variant& v = model_variants[i];
+        double               step = 0.0, item = 0.0;
+        if(!step_cost(v, &step, &item))
+        {
+            continue;
+        }
+        const size_t bm = v.block_m, bn = v.block_n;
+        if((bm % 128 != 0 && !a_kmajor) || (bn % 128 != 0 && !b_kmajor))
+        {
+            continue; // not built for this layout
+        }
+        if((bm >= 192 && rows < 192) || (bn >= 192 && cols < 192))
+        {
+            continue; // a tile much larger than the problem
+        }
+        if(v.pipeline == 6 && (bm == 64 || bn == 64) && rows > 128 && cols > 128)
+        {
+            continue; // the 64-wide tiles are for skinny shapes
+        }
+        const size_t tm = ceil_div(rows, bm), tn = ceil_div(cols, bn), tiles = tm * tn;
+        const double tile_bytes = static_cast<double>(bm * bn) * 4.0;
+        // only the persistent kernel takes ragged M or N as they are; the others run on
+        // padded copies of the operands that need them (two more launches)
+        double copies_us = 0.0;
+        if(v.pipeline != 5 && (rows % bm != 0 || cols % bn != 0))
+        {
+            const double elems = (rows % bm != 0 ? static_cast<double>(tm * bm) * k : 0.0)
+                                 + (cols % bn != 0 ? static_cast<double>(tn * bn) * k : 0.0);
+            copies_us = launch_us + elems * 2.0 * 2.0 / 3.0e6;
+        }
+        auto consider = [&](double t, int split) {
+            t += copies_us;
+            if(!found || t < best)
+            {
+                found        = true;
+                best         = t;
+                out->variant = i;
+                out->swizzle = 4;
+                out->split_k = split;
+            }
+        };
+        // whole tiles
+        consider(launch_us + static_cast<double>(ceil_div(tiles, cus)) * (kt * step + item), 1);
+        // only the last, partial wave of tiles split
+        for(size_t s = 2; s <= 4 && v.pipeline == 5; ++s)
+        {
+            if(tiles > cus && tiles % cus != 0 && kt / s >= 4 && (tiles % cus) * s <= cus * 5 / 4)
+            {
+                consider(launch_us + static_cast<double>(tiles / cus) * (kt * step + item)
+                             + ceil_div(kt, s) * step + item + reduce_us
+                             + (tiles % cus) * s * tile_bytes * 2.0 / tile_bytes_per_us,
+                         -static_cast<int>(s));
+            }
+        }
+        // every tile split (few tiles, long K)
+        if(tiles < cus)
+        {
+            for(size_t s = 2; s <= 32; s *= 2)
+            {
+                if(kt / s < 4)
+                {
+                    break;
+                }
+                consider(launch_us + static_cast<double>(ceil_div(tiles * s, cus)) * (ceil_div(kt, s) * step + item)
+                             + reduce_us + s * tiles * tile_bytes * 2.0 / plane_bytes_per_us,
+                         static_cast<int>(s));
+            }
+        }
+        // the persistent kernel's walk by K tile: for few tiles and a long K only (with
+        // many tiles the workgroups of an XCD stop walking K in step and lose each
+        // other's operand panels in L2: 7168^3 ran at 950 TFLOP/s this way, 1250 by tile)
+        if(v.pipeline == 5 && tiles * 4 <= cus && tiles * kt >= 4 * cus)
+        {
+            const size_t groups = tiles * kt < cus ? tiles * kt : cus;
+            consider(launch_us + ceil_div(tiles * kt, groups) * step + item + reduce_us
+                         + groups * 1.25 * tile_bytes * 2.0 / tile_bytes_per_us,
+                     -1);
+        }
+    }
+    return found;
+}
+
 launch_plan select_plan_from(const tuned_entry* table, size_t count, size_t m, size_t n, size_t k,
                              int type_idx, int lc, int la, int lb)
 {
@@ -137,6 +299,19 @@ launch_plan select_plan_from(const tuned_entry* table, size_t count, size_t m, s
 
 launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int la, int lb)
 {
+    // a tuned entry for exactly this shape first (the reference's order, steps 1 and 2) ...
+    const int   group = type_group_of(type_idx);
+    launch_plan plan;
+    if(find_exact(tuned_table, tuned_count, m, n, k, group, la, lb, lc, &plan)
+       || (group != 0 && find_exact(tuned_table, tuned_count, m, n, k, 0, la, lb, lc, &plan)))
+    {
+        return plan;
+    }
+    // ... then the model for regular shapes, and the nearest tuned entry for the rest
+    if(model_plan(m, n, k, lc, la, lb, &plan))
+    {
+        return plan;
+    }
     return select_plan_from(tuned_table, tuned_count, m, n, k, type_idx, lc, la, lb);
 }
 

@@ -1,8 +1,10 @@
 // Shape -> launch plan.  The tuned table comes from gemm_config_gfx950_*.json via
-// config/generate_config.py; shapes the table does not name are served by its
-// nearest entry, and layouts it does not cover at all by a shape heuristic.
+// config/generate_config.py; shapes the table does not name are served by a time
+// estimate over the compiled variants when they are regular (select_plan: K a multiple
+// of 64, extents multiples of 8), else by the table's nearest entry, and layouts the
+// table does not cover at all by a shape heuristic.
 //
-// Selection order follows the reference's generated find_best_config /
+// select_plan_from follows the reference's generated find_best_config /
 // find_closest_config (reference rocm_wmma_gemm/config/generate_config.py:174-271):
 //   1. exact (M, N, K, type group, layouts) hit;
 //   2. for the fp32-output group, an exact hit in the 16-bit-output group;
@@ -46,6 +48,9 @@ bool find_exact(const tuned_entry* table, size_t count, size_t m, size_t n, size
 bool find_closest(const tuned_entry* table, size_t count, size_t m, size_t n, size_t k,
                   int type_group, int la, int lb, int lc, launch_plan* out);
 launch_plan heuristic_plan(size_t m, size_t n, size_t k, int lc);
+// Estimated-time choice among the compiled variants for a shape without a tuned entry;
+// false for shapes it does not cover (ragged K, odd extents).
+bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_plan* out);
 launch_plan select_plan_from(const tuned_entry* table, size_t count, size_t m, size_t n, size_t k,
                              int type_idx, int lc, int la, int lb);
 

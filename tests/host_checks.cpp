@@ -116,6 +116,41 @@ static int check_select()
     launch_plan e = select_plan_from(nullptr, 0, 4096, 4096, 4096, 0, 0, 0, 1);
     if(e.variant != 1)
         return fail("heuristic on empty table");
+    // The model for regular shapes without a tuned entry: what matters is how the tile
+    // count falls on 256 CUs.
+    struct tile { int bm, bn, pipeline; };
+#define RWG_VARIANT(IDX, BM, BN, BK, WM, WN, PIPE) {BM, BN, PIPE},
+    const tile tiles[] = {
+#include "variants.def"
+    };
+#undef RWG_VARIANT
+    launch_plan p;
+    // 3584^3: 196 tiles of 256 x 256 in one wave, not 361 of 192 x 192 in two
+    if(!model_plan(3584, 3584, 3584, 0, 0, 1, &p) || tiles[p.variant].bm != 256 || tiles[p.variant].bn != 256
+       || tiles[p.variant].pipeline != 5 || p.split_k != 1)
+        return fail("model: 3584^3");
+    // 3072^3, both operands K-contiguous: 256 tiles of 192 x 192
+    if(!model_plan(3072, 3072, 3072, 0, 0, 1, &p) || tiles[p.variant].bm != 192 || tiles[p.variant].bn != 192)
+        return fail("model: 3072^3");
+    // the same with both operands M/N-contiguous: 192-wide tiles are not built
+    if(!model_plan(3072, 3072, 3072, 0, 1, 0, &p) || tiles[p.variant].bm % 128 != 0
+       || tiles[p.variant].bn % 128 != 0)
+        return fail("model: 3072^3, transposed operands");
+    // a column-major C swaps the operands: A row-major, B row-major, C column-major has
+    // kernel-space A = B^T (M/N-contiguous), B = A^T (K-contiguous)
+    if(!model_plan(3072, 3072, 3072, 1, 0, 0, &p) || tiles[p.variant].bm % 128 != 0)
+        return fail("model: operand swap under a column-major C");
+    // few tiles, long K: some split
+    if(!model_plan(304, 4096, 4096, 0, 0, 1, &p) || p.split_k == 1)
+        return fail("model: 304 x 4096 x 4096 wants a split");
+    if(!model_plan(1024, 1024, 65536, 0, 0, 1, &p) || p.split_k == 1)
+        return fail("model: long K wants a split");
+    // 272 tiles of 256 x 256: the last wave of 16 tiles split
+    if(!model_plan(4352, 4096, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline != 5 || p.split_k >= -1)
+        return fail("model: tail split");
+    // not its business: ragged K, odd extents
+    if(model_plan(4096, 4096, 1000, 0, 0, 1, &p) || model_plan(4095, 4096, 4096, 0, 0, 1, &p))
+        return fail("model must leave irregular shapes alone");
     std::printf("select ok\n");
     return 0;
 }
