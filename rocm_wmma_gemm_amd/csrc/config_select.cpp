@@ -164,7 +164,7 @@ size_t ceil_div(size_t a, size_t b)
 // with the second less than half full) and ran at 0.7 of the 196 tiles of 256 x 256.
 // On the 208 tuned entries the model can serve, its pick is on average 2.7 % slower than
 // the tuner's, 25 % at worst.
-bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_plan* out)
+bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_plan* out, size_t batch)
 {
     const size_t rows = lc == 0 ? m : n;
     const size_t cols = lc == 0 ? n : m;
@@ -210,15 +210,18 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
         {
             continue; // the 64-wide tiles are for skinny shapes
         }
-        const size_t tm = ceil_div(rows, bm), tn = ceil_div(cols, bn), tiles = tm * tn;
+        // (batch entries are more tiles: the persistent kernel numbers its items over the
+        // whole batch, the others put the batch in grid.y)
+        const size_t tm = ceil_div(rows, bm), tn = ceil_div(cols, bn), tiles = tm * tn * batch;
         const double tile_bytes = static_cast<double>(bm * bn) * 4.0;
         // only the persistent kernel takes ragged M or N as they are; the others run on
         // padded copies of the operands that need them (two more launches)
         double copies_us = 0.0;
         if(v.pipeline != 5 && (rows % bm != 0 || cols % bn != 0))
         {
-            const double elems = (rows % bm != 0 ? static_cast<double>(tm * bm) * k : 0.0)
-                                 + (cols % bn != 0 ? static_cast<double>(tn * bn) * k : 0.0);
+            const double elems = ((rows % bm != 0 ? static_cast<double>(tm * bm) * k : 0.0)
+                                  + (cols % bn != 0 ? static_cast<double>(tn * bn) * k : 0.0))
+                                 * static_cast<double>(batch);
             copies_us = launch_us + elems * 2.0 * 2.0 / 3.0e6;
         }
         auto consider = [&](double t, int split) {
@@ -297,18 +300,24 @@ launch_plan select_plan_from(const tuned_entry* table, size_t count, size_t m, s
     return heuristic_plan(m, n, k, lc);
 }
 
-launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int la, int lb)
+launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int la, int lb, size_t batch)
 {
-    // a tuned entry for exactly this shape first (the reference's order, steps 1 and 2) ...
     const int   group = type_group_of(type_idx);
     launch_plan plan;
+    // the table was tuned on single GEMMs: a batch changes how many tiles there are to
+    // spread, which is the model's business
+    if(batch > 1 && model_plan(m, n, k, lc, la, lb, &plan, batch))
+    {
+        return plan;
+    }
+    // a tuned entry for exactly this shape first (the reference's order, steps 1 and 2) ...
     if(find_exact(tuned_table, tuned_count, m, n, k, group, la, lb, lc, &plan)
        || (group != 0 && find_exact(tuned_table, tuned_count, m, n, k, 0, la, lb, lc, &plan)))
     {
         return plan;
     }
     // ... then the model for regular shapes, and the nearest tuned entry for the rest
-    if(model_plan(m, n, k, lc, la, lb, &plan))
+    if(model_plan(m, n, k, lc, la, lb, &plan, 1))
     {
         return plan;
     }

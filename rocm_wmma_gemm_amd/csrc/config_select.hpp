@@ -50,7 +50,7 @@ bool find_closest(const tuned_entry* table, size_t count, size_t m, size_t n, si
 launch_plan heuristic_plan(size_t m, size_t n, size_t k, int lc);
 // Estimated-time choice among the compiled variants for a shape without a tuned entry;
 // false for shapes it does not cover (ragged K, odd extents).
-bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_plan* out);
+bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_plan* out, size_t batch = 1);
 launch_plan select_plan_from(const tuned_entry* table, size_t count, size_t m, size_t n, size_t k,
                              int type_idx, int lc, int la, int lb);
 
@@ -59,7 +59,7 @@ inline int type_group_of(int type_idx)
     return (type_idx == 1 || type_idx == 3) ? 1 : 0;
 }
 
-launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int la, int lb);
+launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int la, int lb, size_t batch = 1);
 
 } // namespace host
 } // namespace rocm_wmma_gemm

@@ -641,7 +641,7 @@ int run(int type_idx, const launch_plan* forced, void* C, void* A, void* B, size
     }
     const kernel_problem p = to_kernel_space(C, A, B, M, N, K, batch, layout_c, layout_a, layout_b);
     launch_plan          plan
-        = forced ? *forced : select_plan(M, N, K, type_idx, layout_c, layout_a, layout_b);
+        = forced ? *forced : select_plan(M, N, K, type_idx, layout_c, layout_a, layout_b, batch);
     if(variant_table[plan.variant].pipeline != 0
        && lookup_kernel(type_idx, p.a_kmajor, p.b_kmajor, plan.variant,
                         static_cast<int>(device::load_mode::vec_unguarded))
