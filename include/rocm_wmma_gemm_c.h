@@ -83,6 +83,12 @@ int rocm_wmma_gemm_variant_info_get(int variant, rocm_wmma_gemm_variant_info* in
  * arguments. */
 int rocm_wmma_gemm_select(size_t M, size_t N, size_t K, int type_idx, int layout_c, int layout_a,
                           int layout_b, int* swizzle, int* split_k);
+/* The same for a strided batch of batch_count problems of this shape: the dispatcher counts
+ * the tiles of the whole batch when it weighs tile sizes and splits, so the answer can differ
+ * from the single problem's. */
+int rocm_wmma_gemm_select_batched(size_t M, size_t N, size_t K, size_t batch_count, int type_idx,
+                                  int layout_c, int layout_a, int layout_b, int* swizzle,
+                                  int* split_k);
 
 /* Same computation as the four entry points above, but with the tile variant,
  * swizzle and split field (see above) forced (tuner hook).  Returns 0 on success, -1 if the

@@ -573,6 +573,10 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         args.blocks_per_batch = static_cast<int>(blocks_per_batch);
         args.batches          = static_cast<int>(nb);
         args.stream_units     = static_cast<int>(stream_units);
+        args.batch_by_xcd     = (persistent || v.pipeline == 6) && nb > 1 && split_k == 1 && stream_groups == 0
+                                        && blocks_per_batch * nb < (size_t{1} << 31)
+                                    ? 1
+                                    : 0;
 
         dim3 grid(static_cast<unsigned>(blocks_per_batch), static_cast<unsigned>(nb));
         if(persistent)
@@ -817,12 +821,22 @@ int rocm_wmma_gemm_variant_info_get(int variant, rocm_wmma_gemm_variant_info* in
 int rocm_wmma_gemm_select(size_t M, size_t N, size_t K, int type_idx, int layout_c, int layout_a,
                           int layout_b, int* swizzle, int* split_k)
 {
+    return rocm_wmma_gemm_select_batched(M, N, K, 1, type_idx, layout_c, layout_a, layout_b,
+                                         swizzle, split_k);
+}
+
+int rocm_wmma_gemm_select_batched(size_t M, size_t N, size_t K, size_t batch_count, int type_idx,
+                                  int layout_c, int layout_a, int layout_b, int* swizzle,
+                                  int* split_k)
+{
     using namespace rocm_wmma_gemm::host;
-    if(type_idx < 0 || type_idx >= num_types || ((layout_c | layout_a | layout_b) & ~1))
+    if(type_idx < 0 || type_idx >= num_types || ((layout_c | layout_a | layout_b) & ~1)
+       || batch_count == 0)
     {
         return -1;
     }
-    const launch_plan plan = select_plan(M, N, K, type_idx, layout_c, layout_a, layout_b);
+    const launch_plan plan
+        = select_plan(M, N, K, type_idx, layout_c, layout_a, layout_b, batch_count);
     if(swizzle)
     {
         *swizzle = plan.swizzle;

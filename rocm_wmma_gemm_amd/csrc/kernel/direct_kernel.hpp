@@ -570,9 +570,27 @@ struct direct_gemm
         const int wave_m  = wave / WAVES_N;
         const int wave_n  = wave % WAVES_N;
 
-        const block_work w = decode_block(args);
-        const int slice    = w.slice;
-        const tile_coord t = map_tile(w.tile_id, args.grid_m, args.grid_n, args.group);
+        // The hardware deals the workgroups of the grid, x fastest, round-robin over the
+        // XCDs.  With batch_by_xcd (whole tiles only) each XCD takes a contiguous run of
+        // (batch entry, tile) pairs instead of every eighth tile of every entry.
+        block_work w;
+        tile_coord t;
+        long long  batch;
+        if(args.batch_by_xcd)
+        {
+            const int item = xcd_remap((int)(blockIdx.x + blockIdx.y * gridDim.x), (int)(gridDim.x * gridDim.y));
+            const int entry = item / (int)gridDim.x;
+            batch           = entry;
+            w               = decode_block(args, item - entry * (int)gridDim.x);
+            t = banded_tile(w.tile_id, args.grid_m, args.grid_n, args.group < 1 ? 1 : args.group);
+        }
+        else
+        {
+            batch = blockIdx.y;
+            w     = decode_block(args);
+            t     = map_tile(w.tile_id, args.grid_m, args.grid_n, args.group);
+        }
+        const int slice = w.slice;
         const int row0 = t.m * BM;
         const int col0 = t.n * BN;
 
@@ -586,7 +604,6 @@ struct direct_gemm
         }
         const int nk = step_end - step_begin;
 
-        const long long batch = blockIdx.y;
         const InT* A = static_cast<const InT*>(args.A) + batch * args.batch_stride_a;
         const InT* B = static_cast<const InT*>(args.B) + batch * args.batch_stride_b;
 

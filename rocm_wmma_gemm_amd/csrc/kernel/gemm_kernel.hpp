@@ -73,6 +73,11 @@ struct gemm_args
                               // workgroup g takes K tiles [g * U, (g + 1) * U) of the sequence of all
                               // K tiles of all tiles of all batch entries; partials then holds two
                               // [BM][BN] slots per workgroup
+    int         batch_by_xcd; // persistent and direct kernels, needs k_slices == 1 and
+                              // blocks_per_batch * batches in an int.  1: the items (tile,
+                              // batch entry) are dealt so that each XCD works through one
+                              // contiguous run of batch entries, and the tiles of an entry, which
+                              // share its A and B, go through one L2 at about the same time
 };
 
 // What one workgroup works on.  blockIdx.x enumerates the whole tiles first, then

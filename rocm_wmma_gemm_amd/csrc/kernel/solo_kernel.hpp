@@ -564,9 +564,14 @@ struct solo_gemm
         int       step_begin;
         if(wk.hop != 0)
         {
-            x.batch            = pos / args.blocks_per_batch;
-            const block_work w = decode_block(args, pos - x.batch * args.blocks_per_batch);
-            const tile_coord t = map_tile(w.tile_id, args.grid_m, args.grid_n, args.group);
+            // (positions that are congruent mod 8 run on the same XCD: the grid is a
+            // multiple of 8 workgroups whenever a workgroup takes more than one position)
+            const int item     = args.batch_by_xcd ? xcd_remap(pos, wk.end) : pos;
+            x.batch            = item / args.blocks_per_batch;
+            const block_work w = decode_block(args, item - x.batch * args.blocks_per_batch);
+            const tile_coord t = args.batch_by_xcd
+                                     ? banded_tile(w.tile_id, args.grid_m, args.grid_n, args.group < 1 ? 1 : args.group)
+                                     : map_tile(w.tile_id, args.grid_m, args.grid_n, args.group);
             x.row0             = t.m * BM;
             x.col0             = t.n * BN;
             const int steps_per = (k_steps_total + w.slices - 1) / w.slices;

@@ -32,16 +32,19 @@ SETS = {
     # projection, decode-like, ragged and long-K shapes
     "other": "8192,4096,2048:4096,14336,4096:16,8192,8192:64,8192,8192:128,8192,8192:"
              "4095,5121,3001:1000,1000,1000:1024,1024,65536:3072,3072,3072:6144,6144,6144",
+    # many small problems in one strided-batch call (run with --batch_count, default 64)
+    "batched": "128,128,128:256,256,256:512,512,512:1024,1024,1024:256,256,4096:"
+               "384,640,512:1000,1000,1000:2048,2048,2048",
 }
 TITLES = {"f16_f16": "FP16 in, FP16 out", "f32_f16": "FP16 in, FP32 out",
           "bf16_bf16": "BF16 in, BF16 out", "f32_bf16": "BF16 in, FP32 out"}
 ROW = re.compile(r"^(\S+)\s+(\d+),(\d+),(\d+)\s+([rc]{3})\s+\S+\s+\S+\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)")
 
 
-def run_bench(type_pair: str, shapes: str, reps: int) -> dict:
+def run_bench(type_pair: str, shapes: str, reps: int, batch: int = 1) -> dict:
     """{(m, n, k): {'ours'|'rocblas': {layout 'abc': TFLOP/s}}}"""
     cmd = [BENCH, "--type", type_pair, "--shapes", shapes, "--layouts", "all", "--rocblas",
-           "--reps", str(reps)]
+           "--reps", str(reps), "--batch_count", str(batch)]
     print("running:", " ".join(cmd), file=sys.stderr)
     out = subprocess.run(cmd, capture_output=True, text=True, check=True, timeout=1800).stdout
     res: dict = {}
@@ -120,18 +123,25 @@ def main(argv=None) -> int:
     ap.add_argument("--set", choices=sorted(SETS), default=None)
     ap.add_argument("--shapes", default=None, help="M,N,K:M,N,K:... instead of --set")
     ap.add_argument("--reps", type=int, default=20)
+    ap.add_argument("--batch_count", type=int, default=None,
+                    help="problems per strided-batch call (default 1; 64 for --set batched); "
+                         "rocBLAS then runs rocblas_gemm_strided_batched_ex")
     ap.add_argument("--out", required=True, help="markdown file to write")
     ap.add_argument("--png", default=None, help="bar chart to write (needs matplotlib)")
     a = ap.parse_args(argv)
     shapes = a.shapes or SETS[a.set or "square"]
-    res = run_bench(a.type, shapes, a.reps)
+    batch = a.batch_count or (64 if a.set == "batched" else 1)
+    res = run_bench(a.type, shapes, a.reps, batch)
     title = {"square": "Square matrices", "rectangle": "Rectangular matrices",
-             "other": "Projection, skinny, ragged and long-K shapes"}.get(a.set, "Selected shapes")
+             "other": "Projection, skinny, ragged and long-K shapes",
+             "batched": f"Strided batches of {batch} small problems"}.get(a.set, "Selected shapes")
+    flops = "2·M·N·K" if batch == 1 else f"{batch}·2·M·N·K"
     lines = [f"# {title}: this library and rocBLAS on one MI355X\n",
-             f"TFLOP/s = 2·M·N·K / median of {a.reps} event-timed launches, seeded random operands; "
+             f"TFLOP/s = {flops} / median of {a.reps} event-timed launches, seeded random operands; "
              f"{device_line()}.",
              "Produced by `rocm_wmma_gemm_amd/csrc/tools/bench_report.py` "
-             f"(`--type {a.type} --shapes {shapes}`).\n"]
+             f"(`--type {a.type} --shapes {shapes}" + (f" --batch_count {batch}" if batch > 1 else "")
+             + "`).\n"]
     lines += table(res, a.type)
     if a.png and chart(res, a.type, a.png):
         lines.append(f"\n![chart]({os.path.basename(a.png)})")

@@ -211,9 +211,9 @@ int main(int argc, char** argv)
                                    size_t, int, int, int, void*);
     auto run_variant = reinterpret_cast<run_variant_fn>(
         dlsym(loader.native_handle(), "rocm_wmma_gemm_run_variant"));
-    using select_fn = int (*)(size_t, size_t, size_t, int, int, int, int, int*, int*);
-    auto select
-        = reinterpret_cast<select_fn>(dlsym(loader.native_handle(), "rocm_wmma_gemm_select"));
+    using select_fn = int (*)(size_t, size_t, size_t, size_t, int, int, int, int, int*, int*);
+    auto select = reinterpret_cast<select_fn>(
+        dlsym(loader.native_handle(), "rocm_wmma_gemm_select_batched"));
     using entry_fn = rocm_wmma_gemm::loader::entry_fn;
     const char* entry_names[4] = {"rocm_wmma_gemm_f16_f16", "rocm_wmma_gemm_f32_f16",
                                   "rocm_wmma_gemm_bf16_bf16", "rocm_wmma_gemm_f32_bf16"};
@@ -257,7 +257,7 @@ int main(int argc, char** argv)
             const int la = lay[0] == 'c', lb = lay[1] == 'c', lc = lay[2] == 'c';
             int       sel_swz = swizzle, sel_sk = split_k, sel_var = variant;
             if(variant < 0 && select)
-                sel_var = select(sh.m, sh.n, sh.k, tidx, lc, la, lb, &sel_swz, &sel_sk);
+                sel_var = select(sh.m, sh.n, sh.k, batch, tidx, lc, la, lb, &sel_swz, &sel_sk);
             auto call = [&]() {
                 if(variant >= 0)
                 {
@@ -304,7 +304,7 @@ int main(int argc, char** argv)
             }
             std::fflush(stdout);
 #ifdef WITH_ROCBLAS
-            if(with_rocblas && blas && batch == 1)
+            if(with_rocblas && blas)
             {
                 // rocBLAS is column-major: C(col) = op(A) op(B); a row-major operand is
                 // the transpose of a column-major one.  A row-major C (M x N) is the
@@ -316,23 +316,37 @@ int main(int argc, char** argv)
                 const float alpha = 1.0f, beta = 0.0f;
                 // as a column-major matrix: A is M x K (ld M) if col-major, else K x M (ld K)
                 const rocblas_int lda = la ? sh.m : sh.k, ldb = lb ? sh.k : sh.n;
+                // the matrices of a batch follow one another without gaps
+                const rocblas_stride sa = sh.m * sh.k, sb = sh.k * sh.n, sc = sh.m * sh.n;
                 auto blas_call = [&]() {
                     if(lc == 1)
                     {
                         const rocblas_operation ta = la ? rocblas_operation_none : rocblas_operation_transpose;
                         const rocblas_operation tb = lb ? rocblas_operation_none : rocblas_operation_transpose;
-                        rocblas_gemm_ex(blas, ta, tb, sh.m, sh.n, sh.k, &alpha, A, in_t, lda, B, in_t,
-                                        ldb, &beta, C, out_t, sh.m, C, out_t, sh.m,
-                                        rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+                        if(batch == 1)
+                            rocblas_gemm_ex(blas, ta, tb, sh.m, sh.n, sh.k, &alpha, A, in_t, lda, B,
+                                            in_t, ldb, &beta, C, out_t, sh.m, C, out_t, sh.m,
+                                            rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+                        else
+                            rocblas_gemm_strided_batched_ex(
+                                blas, ta, tb, sh.m, sh.n, sh.k, &alpha, A, in_t, lda, sa, B, in_t, ldb,
+                                sb, &beta, C, out_t, sh.m, sc, C, out_t, sh.m, sc, (rocblas_int)batch,
+                                rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
                     }
                     else
                     {
                         // C^T (N x M, ld N) = op(B) op(A) with op(B) = B^T (N x K), op(A) = A^T (K x M)
                         const rocblas_operation tb = lb ? rocblas_operation_transpose : rocblas_operation_none;
                         const rocblas_operation ta = la ? rocblas_operation_transpose : rocblas_operation_none;
-                        rocblas_gemm_ex(blas, tb, ta, sh.n, sh.m, sh.k, &alpha, B, in_t, ldb, A, in_t,
-                                        lda, &beta, C, out_t, sh.n, C, out_t, sh.n,
-                                        rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+                        if(batch == 1)
+                            rocblas_gemm_ex(blas, tb, ta, sh.n, sh.m, sh.k, &alpha, B, in_t, ldb, A,
+                                            in_t, lda, &beta, C, out_t, sh.n, C, out_t, sh.n,
+                                            rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+                        else
+                            rocblas_gemm_strided_batched_ex(
+                                blas, tb, ta, sh.n, sh.m, sh.k, &alpha, B, in_t, ldb, sb, A, in_t, lda,
+                                sa, &beta, C, out_t, sh.n, sc, C, out_t, sh.n, sc, (rocblas_int)batch,
+                                rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
                     }
                 };
                 for(int w = 0; w < warmup; ++w)
@@ -347,7 +361,7 @@ int main(int argc, char** argv)
                     CHECK(hipEventElapsedTime(&ms[r], e0, e1));
                 }
                 std::sort(ms.begin(), ms.end());
-                const double btf = 2.0 * sh.m * sh.n * sh.k / (ms[reps / 2] * 1e-3) / 1e12;
+                const double btf = 2.0 * sh.m * sh.n * sh.k * batch / (ms[reps / 2] * 1e-3) / 1e12;
                 std::printf("%-10s %-22s %-4s %8s %6s %10.4f %10.4f %8.1f %7.1f%%\n", "rocblas", dims,
                             lay.c_str(), "-", "-", ms[reps / 2], ms[0], btf, 100.0 * btf / peak_tf);
                 std::fflush(stdout);

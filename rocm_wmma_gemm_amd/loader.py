@@ -147,6 +147,9 @@ class Loader:
         L.rocm_wmma_gemm_select.restype = ctypes.c_int
         L.rocm_wmma_gemm_select.argtypes = [ctypes.c_size_t] * 3 + [ctypes.c_int] * 4 + [
             ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
+        L.rocm_wmma_gemm_select_batched.restype = ctypes.c_int
+        L.rocm_wmma_gemm_select_batched.argtypes = [ctypes.c_size_t] * 4 + [ctypes.c_int] * 4 + [
+            ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
         L.rocm_wmma_gemm_run_variant.restype = ctypes.c_int
         L.rocm_wmma_gemm_run_variant.argtypes = [ctypes.c_int] * 4 + self._ENTRY_ARGS
 
@@ -163,11 +166,13 @@ class Loader:
         return out
 
     def select(self, M: int, N: int, K: int, type_idx: int, layout_c: int, layout_a: int,
-               layout_b: int) -> tuple[int, int, int]:
-        """(variant, swizzle, split_k) the dispatcher picks for this problem."""
+               layout_b: int, batch_count: int = 1) -> tuple[int, int, int]:
+        """(variant, swizzle, split_k) the dispatcher picks for this problem (for a strided
+        batch of batch_count such problems)."""
         swz, sk = ctypes.c_int(0), ctypes.c_int(0)
-        v = self._lib.rocm_wmma_gemm_select(M, N, K, type_idx, int(layout_c), int(layout_a),
-                                            int(layout_b), ctypes.byref(swz), ctypes.byref(sk))
+        v = self._lib.rocm_wmma_gemm_select_batched(
+            M, N, K, batch_count, type_idx, int(layout_c), int(layout_a), int(layout_b),
+            ctypes.byref(swz), ctypes.byref(sk))
         return v, swz.value, sk.value
 
     # ------------------------------------------------------------------ gemm

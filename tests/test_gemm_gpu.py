@@ -270,6 +270,39 @@ def test_workgroups_that_take_several_tiles_agree_with_oracle(loader):
                                          f"layouts C{lc} A{la} B{lb} {tname}: {e}") from None
 
 
+def test_batch_entries_dealt_by_xcd_agree_with_oracle(loader):
+    """Strided batches of whole tiles on the kernels that deal (batch entry, tile) pairs
+    to the XCDs in contiguous runs: every entry's every tile must still be computed once.
+    Item counts that are and are not multiples of the 8 XCDs, fewer and more items than
+    the 256 CUs, one tile per entry, every layout class, 16-bit and fp32 C, and a ragged
+    shape on the kernels that take one."""
+    kernels = [v for v in loader.variants() if v.pipeline in (5, 6)]
+    assert kernels, "no persistent or direct-to-LDS variant compiled"
+    cases = [  # M, N, K, batch
+        (512, 768, 128, 11),    # 6 tiles of 256 x 256 x 11 entries = 66 items
+        (256, 256, 192, 37),    # one 256 x 256 tile per entry
+        (768, 1024, 64, 29),    # 12 x 29 = 348 items: more than the CUs, not a multiple of 8
+        (328, 456, 128, 9),     # ragged
+    ]
+    for i, v in enumerate(kernels):
+        for n, (M, N, K, batch) in enumerate(cases):
+            tname = "f16_f16" if (n + i) % 2 == 0 else "f32_bf16"
+            din, dout = TYPE_PAIRS[tname]
+            layouts = [l for l in [(0, 0, 1), (1, 1, 0), (0, 0, 0), (1, 1, 1)] if built_for(v, *l)]
+            lc, la, lb = layouts[(n + i) % len(layouts)]
+            A = np.concatenate([O.init_matrix(M, K, la, din, seed=130 + b) for b in range(batch)])
+            B = np.concatenate([O.init_matrix(K, N, lb, din, seed=170 + b) for b in range(batch)])
+            gpu = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout, batch=batch,
+                          variant=(v.index, 2, 1))
+            for b in range(batch):
+                try:
+                    check_against_oracle(gpu[b * M * N:(b + 1) * M * N], A[b * M * K:(b + 1) * M * K],
+                                         B[b * K * N:(b + 1) * K * N], M, N, K, lc, la, lb, din, dout)
+                except AssertionError as e:
+                    raise AssertionError(f"variant {v.index} {M}x{N}x{K} batch {b}/{batch} "
+                                         f"layouts C{lc} A{la} B{lb} {tname}: {e}") from None
+
+
 def test_degenerate_arguments(loader):
     import torch
 
