@@ -176,16 +176,20 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
         a_kmajor     = b_kmajor;
         b_kmajor     = t;
     }
-    if(k < 64 || k % 64 != 0 || rows % 8 != 0 || cols % 8 != 0 || rows < 16 || cols < 16)
+    // K need not be whole K tiles: the persistent kernel cuts a partial last tile off
+    // itself, as long as the rows of a K-contiguous operand stay 16-byte aligned
+    const bool k_whole = k % 64 == 0;
+    if(k < 64 || rows % 8 != 0 || cols % 8 != 0 || rows < 16 || cols < 16
+       || (!k_whole && (a_kmajor || b_kmajor) && k % 8 != 0))
     {
-        return false; // shapes the direct kernels would only take through padded copies
+        return false; // shapes every direct kernel would only take through padded copies
     }
     constexpr size_t cus           = 256;
     constexpr double launch_us     = 6.0;
     constexpr double reduce_us     = 4.0;
     constexpr double plane_bytes_per_us = 2.2e6; // partial planes: written, then read by reduce_partials
     constexpr double tile_bytes_per_us  = 3.7e6; // partial tiles (split tail, walk by K tile)
-    const size_t     kt            = k / 64;
+    const size_t     kt            = ceil_div(k, size_t{64});
     double           best          = 0.0;
     bool             found         = false;
     const int        count         = static_cast<int>(sizeof(model_variants) / sizeof(model_variants[0]));
@@ -214,13 +218,14 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
         // whole batch, the others put the batch in grid.y)
         const size_t tm = ceil_div(rows, bm), tn = ceil_div(cols, bn), tiles = tm * tn * batch;
         const double tile_bytes = static_cast<double>(bm * bn) * 4.0;
-        // only the persistent kernel takes ragged M or N as they are; the others run on
+        // only the persistent kernel takes ragged M, N or K as they are; the others run on
         // padded copies of the operands that need them (two more launches)
         double copies_us = 0.0;
-        if(v.pipeline != 5 && (rows % bm != 0 || cols % bn != 0))
+        if(v.pipeline != 5 && (rows % bm != 0 || cols % bn != 0 || !k_whole))
         {
-            const double elems = ((rows % bm != 0 ? static_cast<double>(tm * bm) * k : 0.0)
-                                  + (cols % bn != 0 ? static_cast<double>(tn * bn) * k : 0.0))
+            const double k_pad = static_cast<double>(kt * 64);
+            const double elems = ((rows % bm != 0 || !k_whole ? static_cast<double>(tm * bm) * k_pad : 0.0)
+                                  + (cols % bn != 0 || !k_whole ? static_cast<double>(tn * bn) * k_pad : 0.0))
                                  * static_cast<double>(batch);
             copies_us = launch_us + elems * 2.0 * 2.0 / 3.0e6;
         }

@@ -251,11 +251,11 @@ size_t round_up(size_t x, size_t to)
 }
 
 // The direct pipelines address a tile with 32-bit byte offsets from its origin.
-bool spans_fit(const variant_desc& v, bool a_kmajor, bool b_kmajor, size_t lda, size_t ldb)
+bool spans_fit(const variant_desc& v, bool a_kmajor, bool b_kmajor, size_t lda, size_t ldb, int bits = 32)
 {
     const unsigned long long a_span = (a_kmajor ? v.block_m : v.block_k) * lda * 2ull;
     const unsigned long long b_span = (b_kmajor ? v.block_n : v.block_k) * ldb * 2ull;
-    return a_span < (1ull << 32) && b_span < (1ull << 32);
+    return a_span < (1ull << bits) && b_span < (1ull << bits);
 }
 
 template<class OutT>
@@ -299,6 +299,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
     size_t      pack_bytes = 0;
     bool        packed     = false; // the kernel reads a padded copy of ...
     bool        copy_a = false, copy_b = false; // ... this operand
+    int         k_tail = 0; // columns of a partial last K tile that the kernel cuts off itself
 
     if(variant_table[plan.variant].pipeline != 0)
     {
@@ -315,12 +316,15 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
             }
         }
         else if(dv.pipeline == 5 && mode == static_cast<int>(device::load_mode::vec_guarded)
-                && p.K % dv.block_k == 0 && spans_fit(dv, p.a_kmajor, p.b_kmajor, lda, ldb))
+                && spans_fit(dv, p.a_kmajor, p.b_kmajor, lda, ldb, 31))
         {
-            // Ragged M or N only, rows aligned: the persistent kernel takes the operands as
+            // Ragged M, N or K, rows aligned: the persistent kernel takes the operands as
             // they are.  Its buffer descriptors end at the operands' ends, tiles that hang
-            // over an edge read zeros or neighbouring data there, and the guarded stores
-            // leave those rows and columns out.
+            // over an edge in M or N read zeros or neighbouring data there, and the guarded
+            // stores leave those rows and columns out; of a last K tile that the operands
+            // hold only in part the kernel reads the rest as zeros.
+            k_kernel = round_up(p.K, dv.block_k);
+            k_tail   = static_cast<int>(p.K % dv.block_k);
         }
         else
         {
@@ -573,6 +577,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         args.blocks_per_batch = static_cast<int>(blocks_per_batch);
         args.batches          = static_cast<int>(nb);
         args.stream_units     = static_cast<int>(stream_units);
+        args.k_tail           = k_tail;
         args.batch_by_xcd     = (persistent || v.pipeline == 6) && nb > 1 && split_k == 1 && stream_groups == 0
                                         && blocks_per_batch * nb < (size_t{1} << 31)
                                     ? 1

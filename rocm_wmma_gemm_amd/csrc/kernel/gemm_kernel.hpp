@@ -73,6 +73,9 @@ struct gemm_args
                               // workgroup g takes K tiles [g * U, (g + 1) * U) of the sequence of all
                               // K tiles of all tiles of all batch entries; partials then holds two
                               // [BM][BN] slots per workgroup
+    int         k_tail; // persistent kernel with guarded stores only.  0: the operands hold K
+                        // columns, a multiple of the K tile.  t > 0: they hold K - 64 + t
+                        // columns, and the kernel reads zeros for the rest of the last K tile
     int         batch_by_xcd; // persistent and direct kernels, needs k_slices == 1 and
                               // blocks_per_batch * batches in an int.  1: the items (tile,
                               // batch entry) are dealt so that each XCD works through one

@@ -105,6 +105,11 @@ struct solo_gemm
         return (vmcnt & 15) | (7 << 4) | (0 << 8) | ((vmcnt >> 4) << 14);
     }
 
+    // Largest range a load descriptor is given; a vector offset of this value is outside
+    // every descriptor's range, whatever the scalar offset adds (tile spans stay below it,
+    // so the sum does not wrap).
+    static constexpr unsigned int RANGE_MAX = 0x80000000u;
+
     // Addressing of one operand's global -> LDS loads.  Load i of a tile (i = 0 ..
     // PER_WAVE-1; it fills the 1 KiB LDS block wave + i*WAVES) is a buffer load whose
     // address is split three ways so that nothing is computed per load: the tile origin
@@ -149,6 +154,37 @@ struct solo_gemm
         {
             return voff[KMAJOR ? 0 : (I & 1)];
         }
+
+        // The offsets for a last K tile of which only columns [0, kt) exist, kt a multiple
+        // of 8.  K-contiguous: a lane fetches the same 8 columns of its row in every load,
+        // and a lane whose columns lie past kt gets an offset outside every descriptor's
+        // range (RANGE_MAX), so its loads write zeros to LDS.  M/N-contiguous: the rows
+        // past kt lie past the end of the operand's batch entry, where the descriptor
+        // ends; nothing to change.
+        __device__ __forceinline__ load_addr for_tail(int lane, int wave, int kt) const
+        {
+            load_addr t = *this;
+            if constexpr(KMAJOR)
+            {
+                constexpr int CH = BK / 8;
+                const int     r  = 8 * wave + lane / CH;
+                const int     c  = (lane % CH) ^ swizzle_of_row<CH, MI>(r);
+                t.voff[0]        = c * 8 < kt ? voff[0] : RANGE_MAX;
+            }
+            return t;
+        }
+
+        // this, or other when `take` (the same in every lane) is set
+        __device__ __forceinline__ load_addr or_else(bool take, const load_addr& other) const
+        {
+            load_addr t = *this;
+#pragma unroll
+            for(int p = 0; p < (KMAJOR ? 1 : 2); ++p)
+            {
+                t.voff[p] = take ? other.voff[p] : voff[p];
+            }
+            return t;
+        }
     };
 
     using addr_a = load_addr<A_KMAJOR, BM>;
@@ -170,7 +206,7 @@ struct solo_gemm
     // (mfma_probe --range).  Rows or columns past the edge but inside the allocation
     // read whatever is there (the next k row, the next batch entry); they only reach
     // accumulators of rows and columns of C that the guarded stores leave out.  Every
-    // tile span fits 32 bits (the host checks).
+    // tile span fits 31 bits (the host checks).
     __device__ __forceinline__ static u32x4 descriptor(const InT* origin, const InT* end)
     {
         const unsigned long long p = (unsigned long long)origin;
@@ -179,7 +215,7 @@ struct solo_gemm
         {
             // (whole tiles of a matrix of whole tiles end inside it anyway)
             const unsigned long long left = (unsigned long long)end - p;
-            records                       = left > 0xffffffffull ? 0xffffffffu : (unsigned int)left;
+            records                       = left > RANGE_MAX ? RANGE_MAX : (unsigned int)left;
         }
         return u32x4{(unsigned int)p, (unsigned int)(p >> 32) & 0xffffu, records, 0x00020000u};
     }
@@ -521,6 +557,9 @@ struct solo_gemm
         int        nk; // K tiles, at least one
         const InT* a; // first K tile of the operands
         const InT* b;
+        const InT* a_end; // where the loads' range ends (see limits)
+        const InT* b_end;
+        bool       ends_k; // the item's last K tile is the last of K
         float*     partial; // nullptr: the item is a whole tile and goes to C; else where
                             // element (row, col) of C, global coordinates, goes:
                             // partial[row * pitch + col]
@@ -623,7 +662,33 @@ struct solo_gemm
                              + x.row0 * a_sr + (long long)step_begin * BK * a_sk);
         x.b = scalar_pointer(static_cast<const InT*>(args.B) + x.batch * args.batch_stride_b
                              + x.col0 * b_sr + (long long)step_begin * BK * b_sk);
+        x.ends_k = step_begin + x.nk == k_steps_total;
+        limits(args, x);
         return x;
+    }
+
+    // Where the range of an item's load descriptors ends (guarded kernels only; the
+    // others do not check).  A K-contiguous operand: at the end of the allocation (the
+    // last batch entry's last row).  An M/N-contiguous operand: at the end of the item's
+    // batch entry, which is the end of its K rows, so that the rows of the last K tile
+    // past K read zeros in every batch entry.
+    __device__ __forceinline__ static void limits(const gemm_args& args, work_item& x)
+    {
+        if constexpr(GUARD_C)
+        {
+            const long long k_rows = args.K - (args.k_tail ? BK - args.k_tail : 0);
+            x.a_end = scalar_pointer(static_cast<const InT*>(args.A)
+                                     + (A_KMAJOR ? (args.batches - 1) * args.batch_stride_a + args.M * args.lda
+                                                 : x.batch * args.batch_stride_a + k_rows * args.lda));
+            x.b_end = scalar_pointer(static_cast<const InT*>(args.B)
+                                     + (B_KMAJOR ? (args.batches - 1) * args.batch_stride_b + args.N * args.ldb
+                                                 : x.batch * args.batch_stride_b + k_rows * args.ldb));
+        }
+        else
+        {
+            x.a_end = nullptr;
+            x.b_end = nullptr;
+        }
     }
 
     // The accumulators of a finished work item, to C or to the fp32 partial tiles.
@@ -698,11 +763,10 @@ struct solo_gemm
         la.init(wave, lane, a_ld);
         lb.init(wave, lane, b_ld);
 
-        // one past the last element of each operand (all batch entries)
-        const InT* const a_end = static_cast<const InT*>(args.A) + (args.batches - 1) * args.batch_stride_a
-                                 + (long long)(A_KMAJOR ? args.M : args.K) * a_ld;
-        const InT* const b_end = static_cast<const InT*>(args.B) + (args.batches - 1) * args.batch_stride_b
-                                 + (long long)(B_KMAJOR ? args.N : args.K) * b_ld;
+        // a last K tile that the operands hold only in part (guarded kernels)
+        const bool   k_ragged = GUARD_C && args.k_tail != 0;
+        const addr_a la_tail  = la.for_tail(lane, wave, args.k_tail);
+        const addr_b lb_tail  = lb.for_tail(lane, wave, args.k_tail);
 
         work_item cur = decode(args, wk, wk.begin);
 
@@ -717,8 +781,11 @@ struct solo_gemm
         // tiles of extra L2 -> LDS traffic for nothing.
         const InT* a_src       = cur.a;
         const InT* b_src       = cur.b;
+        const InT* a_end       = cur.a_end;
+        const InT* b_end       = cur.b_end;
         int        stream_left = cur.nk;
         int        stream_next = cur.next;
+        bool       stream_ends = cur.ends_k;
         auto advance = [&]() {
             a_src += a_step;
             b_src += b_step;
@@ -727,10 +794,15 @@ struct solo_gemm
                 const work_item nx = decode(args, wk, stream_next < wk.end ? stream_next : wk.begin);
                 a_src              = nx.a;
                 b_src              = nx.b;
+                a_end              = nx.a_end;
+                b_end              = nx.b_end;
                 stream_left        = nx.nk;
                 stream_next        = nx.next;
+                stream_ends        = nx.ends_k;
             }
         };
+        // whether the tile at (a_src, b_src) is a last K tile held only in part
+        auto partial_tile = [&]() { return k_ragged && stream_ends && stream_left == 1; };
 
         // Ring of 2 tiles, two K steps per tile.  Tile t: first step on K step 0 with
         // the reads of K step 1; then wait for the own loads of tile t+1 and the own
@@ -747,13 +819,20 @@ struct solo_gemm
 
         u32x4 fa[2][TM], fb[2][TN];
         // prologue: tile 0 and the first part of tile 1 on their way, tile 0 landed
-        issue_loads(std::make_integer_sequence<int, VM_LOADS>{}, la, lb, wave_block,
-                    descriptor(a_src, a_end), descriptor(b_src, b_end));
+        {
+            const bool part = partial_tile();
+            issue_loads(std::make_integer_sequence<int, VM_LOADS>{}, la.or_else(part, la_tail),
+                        lb.or_else(part, lb_tail), wave_block, descriptor(a_src, a_end), descriptor(b_src, b_end));
+        }
         advance();
-        issue_loads(std::make_integer_sequence<int, LOADS_B>{}, la, lb, wave_block + STAGE,
-                    descriptor(a_src, a_end), descriptor(b_src, b_end));
-        const InT* a_prev = a_src;
-        const InT* b_prev = b_src;
+        bool part_prev = partial_tile();
+        issue_loads(std::make_integer_sequence<int, LOADS_B>{}, la.or_else(part_prev, la_tail),
+                    lb.or_else(part_prev, lb_tail), wave_block + STAGE, descriptor(a_src, a_end),
+                    descriptor(b_src, b_end));
+        const InT* a_prev     = a_src;
+        const InT* b_prev     = b_src;
+        const InT* a_end_prev = a_end;
+        const InT* b_end_prev = b_end;
         advance();
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(LOADS_B));
         __builtin_amdgcn_s_barrier();
@@ -782,17 +861,23 @@ struct solo_gemm
             for(int it = 0; it < cur.nk; ++it)
             {
                 const unsigned int there = STAGE - here;
-                const step_ctx c0{oa, ob, la, lb, lds_addr + here, wave_block + there,
-                                  descriptor(a_prev, a_end), descriptor(b_prev, b_end)};
-                const step_ctx c1{oa, ob, la, lb, lds_addr + there, wave_block + here,
+                const bool     part = partial_tile();
+                const addr_a   la0 = la.or_else(part_prev, la_tail), la1 = la.or_else(part, la_tail);
+                const addr_b   lb0 = lb.or_else(part_prev, lb_tail), lb1 = lb.or_else(part, lb_tail);
+                const step_ctx c0{oa, ob, la0, lb0, lds_addr + here, wave_block + there,
+                                  descriptor(a_prev, a_end_prev), descriptor(b_prev, b_end_prev)};
+                const step_ctx c1{oa, ob, la1, lb1, lds_addr + there, wave_block + here,
                                   descriptor(a_src, a_end), descriptor(b_src, b_end)};
                 __builtin_amdgcn_s_waitcnt(waitcnt_imm(63)); // last step's fragment reads
                 step<1, plan_a>(c0, fa[0], fb[0], fa[1], fb[1], acc);
                 __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
                 __builtin_amdgcn_s_barrier();
                 step<0, plan_b>(c1, fa[1], fb[1], fa[0], fb[0], acc);
-                a_prev = a_src;
-                b_prev = b_src;
+                a_prev     = a_src;
+                b_prev     = b_src;
+                a_end_prev = a_end;
+                b_end_prev = b_end;
+                part_prev  = part;
                 advance();
                 here = there;
             }

@@ -148,9 +148,16 @@ static int check_select()
     // 272 tiles of 256 x 256: the last wave of 16 tiles split
     if(!model_plan(4352, 4096, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline != 5 || p.split_k >= -1)
         return fail("model: tail split");
-    // not its business: ragged K, odd extents
-    if(model_plan(4096, 4096, 1000, 0, 0, 1, &p) || model_plan(4095, 4096, 4096, 0, 0, 1, &p))
+    // a partial last K tile with aligned rows: the persistent kernel takes it as it is,
+    // every other kernel would pay padded copies of both operands
+    if(!model_plan(4096, 4096, 1000, 0, 0, 1, &p) || tiles[p.variant].pipeline != 5)
+        return fail("model: ragged K with aligned rows belongs to the persistent kernel");
+    // K-contiguous rows that are not 16-byte aligned, odd extents: not its business ...
+    if(model_plan(4096, 4096, 1001, 0, 0, 1, &p) || model_plan(4095, 4096, 4096, 0, 0, 1, &p))
         return fail("model must leave irregular shapes alone");
+    // ... but an odd K is fine when no operand is K-contiguous (A column-major, B row-major)
+    if(!model_plan(4096, 4096, 1001, 0, 1, 0, &p) || tiles[p.variant].pipeline != 5)
+        return fail("model: odd K, no K-contiguous operand");
     std::printf("select ok\n");
     return 0;
 }

@@ -303,6 +303,71 @@ def test_batch_entries_dealt_by_xcd_agree_with_oracle(loader):
                                          f"layouts C{lc} A{la} B{lb} {tname}: {e}") from None
 
 
+def test_partial_last_k_tile_on_the_persistent_kernel(loader):
+    """K that is not a multiple of the 64-wide K tile, rows 16-byte aligned: the
+    one-wave-per-SIMD kernel reads the operands where they lie and takes the rest of the
+    last K tile as zeros (a K-contiguous operand: the lanes that would fetch columns
+    past K load out of range; an M/N-contiguous one: the rows past K lie past the end of
+    the batch entry's range).  Cases: the partial tile as tile 0, as tile 1 (both go out
+    in the prologue) and later; ragged M and N on top; batch entries; a K split and the
+    walk by K tile on top; K not a multiple of 8 where no operand is K-contiguous."""
+    solo = [v for v in loader.variants() if v.pipeline == 5]
+    assert solo, "no one-wave-per-SIMD variant compiled"
+    cases = [  # M, N, K, batch, split field
+        (512, 512, 1000, 1, 1),
+        (304, 520, 200, 1, 1),     # ragged M and N too
+        (256, 256, 8, 1, 1),       # the only K tile is partial
+        (256, 512, 72, 1, 1),      # the second
+        (256, 256, 136, 5, 1),     # batch entries: each one's range ends at its own K
+        (512, 768, 1096, 2, 2),    # every tile in two K slices, the second ends in the partial tile
+        (768, 512, 648, 3, -1),    # walk by K tile
+        (4352, 256, 40, 1, 1),     # several items per workgroup, each one partial tile
+    ]
+    for i, v in enumerate(solo):
+        for n, (M, N, K, batch, split) in enumerate(cases):
+            tname = "f16_f16" if (n + i) % 2 == 0 else "f32_bf16"
+            din, dout = TYPE_PAIRS[tname]
+            for (lc, la, lb) in [l for l in [(0, 0, 1), (1, 1, 0), (0, 0, 0), (1, 1, 1)] if built_for(v, *l)]:
+                k = K + 1 if (la, lb) == (1, 0) and n % 2 == 0 else K  # odd K: no K-contiguous operand
+                A = np.concatenate([O.init_matrix(M, k, la, din, seed=230 + b) for b in range(batch)])
+                B = np.concatenate([O.init_matrix(k, N, lb, din, seed=260 + b) for b in range(batch)])
+                gpu = run_gpu(loader, A, B, M, N, k, lc, la, lb, din, dout, batch=batch,
+                              variant=(v.index, 4, split))
+                for b in range(batch):
+                    try:
+                        check_against_oracle(gpu[b * M * N:(b + 1) * M * N], A[b * M * k:(b + 1) * M * k],
+                                             B[b * k * N:(b + 1) * k * N], M, N, k, lc, la, lb, din, dout)
+                    except AssertionError as e:
+                        raise AssertionError(f"variant {v.index} {M}x{N}x{k} batch {b}/{batch} split {split} "
+                                             f"layouts C{lc} A{la} B{lb} {tname}: {e}") from None
+
+
+def test_what_lies_past_k_does_not_reach_c(loader):
+    """The columns of the last K tile past K must be zeros, not whatever follows in memory
+    times zero: with infinities right behind a row's K columns (the next row's first
+    elements, the next batch entry) every other row of C stays finite and correct."""
+    solo = next(v for v in loader.variants() if v.pipeline == 5 and (v.block_m, v.block_n) == (256, 256))
+    din, dout = TYPE_PAIRS["f16_f16"]
+    inf = np.uint16(0x7C00)
+    # A row-major (K-contiguous): row 5 starts with infinities, which the loads of row 4's
+    # partial tile would reach
+    M, N, K = 256, 256, 200
+    for lb in (0, 1):
+        A = O.init_matrix(M, K, 0, din, seed=301)
+        B = O.init_matrix(K, N, lb, din, seed=302)
+        A[5 * K:5 * K + 64] = inf
+        gpu = run_gpu(loader, A, B, M, N, K, 0, 0, lb, din, dout, variant=(solo.index, 4, 1))
+        check_against_oracle(gpu, A, B, M, N, K, 0, 0, lb, din, dout, rows=(0, 5))
+        check_against_oracle(gpu, A, B, M, N, K, 0, 0, lb, din, dout, rows=(6, M))
+    # A column-major, B row-major (K rows each): the second batch entry is all
+    # infinities and starts where the first entry's rows past K would be
+    K = 203
+    A = np.concatenate([O.init_matrix(M, K, 1, din, seed=303), np.full(M * K, inf, np.uint16)])
+    B = np.concatenate([O.init_matrix(K, N, 0, din, seed=304), np.full(K * N, inf, np.uint16)])
+    gpu = run_gpu(loader, A, B, M, N, K, 0, 1, 0, din, dout, batch=2, variant=(solo.index, 4, 1))
+    check_against_oracle(gpu[:M * N], A[:M * K], B[:K * N], M, N, K, 0, 1, 0, din, dout)
+
+
 def test_degenerate_arguments(loader):
     import torch
 
