@@ -84,37 +84,98 @@ constexpr int    max_devices           = 64;
 std::mutex       workspace_mutex;
 char*            workspace_ptr[max_devices]  = {};
 size_t           workspace_size[max_devices] = {};
+// The call that used the buffer last: its stream, and an event recorded behind its last
+// kernel.
+hipStream_t workspace_stream[max_devices]   = {};
+hipEvent_t  workspace_released[max_devices] = {};
+bool        workspace_used[max_devices]     = {};
 
-char* workspace_for_current_device(size_t bytes)
+// One call's hold on the current device's buffer, from before its first kernel that
+// touches the buffer is enqueued until after its last one is.  Calls that need the
+// buffer are put in a queue on the device, whatever streams they are on: a call on
+// another stream than the previous holder's makes its stream wait (on the device, the
+// host never blocks) for the event recorded behind that holder's last kernel, so two
+// streams may issue split-K or padded-copy GEMMs at the same time, from one host thread
+// or several, as they may with the kernels that need no scratch memory.  A stream under
+// graph capture is left out of this: it records and waits for nothing, and the buffer
+// must then not be shared with work outside the graph.
+class workspace_lease
 {
-    int dev = 0;
-    if(bytes > workspace_limit_bytes || hipGetDevice(&dev) != hipSuccess || dev < 0
-       || dev >= max_devices)
+public:
+    workspace_lease() = default;
+    workspace_lease(const workspace_lease&)            = delete;
+    workspace_lease& operator=(const workspace_lease&) = delete;
+
+    // nullptr: no memory (or too much asked for); the lease then holds nothing
+    char* acquire(size_t bytes, hipStream_t stream)
     {
-        return nullptr;
-    }
-    std::lock_guard<std::mutex> lock(workspace_mutex);
-    if(workspace_size[dev] < bytes)
-    {
-        size_t want = std::max(bytes + bytes / 4, workspace_first_bytes);
-        if(workspace_ptr[dev] != nullptr)
+        if(bytes > workspace_limit_bytes || hipGetDevice(&dev_) != hipSuccess || dev_ < 0
+           || dev_ >= max_devices)
         {
-            (void)hipDeviceSynchronize();
-            (void)hipFree(workspace_ptr[dev]);
-            workspace_ptr[dev]  = nullptr;
-            workspace_size[dev] = 0;
-        }
-        void* p = nullptr;
-        if(hipMalloc(&p, want) != hipSuccess)
-        {
-            (void)hipGetLastError();
             return nullptr;
         }
-        workspace_ptr[dev]  = static_cast<char*>(p);
-        workspace_size[dev] = want;
+        lock_ = std::unique_lock<std::mutex>(workspace_mutex);
+        if(workspace_size[dev_] < bytes)
+        {
+            size_t want = std::max(bytes + bytes / 4, workspace_first_bytes);
+            if(workspace_ptr[dev_] != nullptr)
+            {
+                (void)hipDeviceSynchronize();
+                (void)hipFree(workspace_ptr[dev_]);
+                workspace_ptr[dev_]  = nullptr;
+                workspace_size[dev_] = 0;
+                workspace_used[dev_] = false;
+            }
+            void* p = nullptr;
+            if(hipMalloc(&p, want) != hipSuccess)
+            {
+                (void)hipGetLastError();
+                lock_.unlock();
+                return nullptr;
+            }
+            workspace_ptr[dev_]  = static_cast<char*>(p);
+            workspace_size[dev_] = want;
+        }
+        stream_ = stream;
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        if(hipStreamIsCapturing(stream, &capture) != hipSuccess)
+        {
+            (void)hipGetLastError();
+            capture = hipStreamCaptureStatusNone;
+        }
+        ordered_ = capture == hipStreamCaptureStatusNone;
+        if(ordered_ && workspace_released[dev_] == nullptr
+           && hipEventCreateWithFlags(&workspace_released[dev_], hipEventDisableTiming) != hipSuccess)
+        {
+            (void)hipGetLastError();
+            workspace_released[dev_] = nullptr;
+            ordered_                 = false;
+        }
+        if(ordered_ && workspace_used[dev_] && workspace_stream[dev_] != stream)
+        {
+            (void)hipStreamWaitEvent(stream, workspace_released[dev_], 0);
+        }
+        held_ = true;
+        return workspace_ptr[dev_];
     }
-    return workspace_ptr[dev];
-}
+
+    ~workspace_lease()
+    {
+        if(held_ && ordered_)
+        {
+            (void)hipEventRecord(workspace_released[dev_], stream_);
+            workspace_stream[dev_] = stream_;
+            workspace_used[dev_]   = true;
+        }
+    }
+
+private:
+    std::unique_lock<std::mutex> lock_;
+    hipStream_t                  stream_  = nullptr;
+    int                          dev_     = 0;
+    bool                         held_    = false;
+    bool                         ordered_ = false;
+};
 
 bool aligned16(const void* p)
 {
@@ -473,10 +534,11 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
                                      ? 2 * stream_groups * v.block_m * v.block_n * sizeof(float)
                                      : (split_k > 1 ? plane_bytes * split_k * batches_per_launch : 0);
 
-    char* workspace = nullptr;
+    char*           workspace = nullptr;
+    workspace_lease lease; // held until the last kernel of this call is enqueued
     if(pack_bytes + partial_bytes > 0)
     {
-        workspace = workspace_for_current_device(pack_bytes + partial_bytes);
+        workspace = lease.acquire(pack_bytes + partial_bytes, stream);
         if(workspace == nullptr)
         {
             if(packed)

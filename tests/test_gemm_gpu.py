@@ -406,6 +406,40 @@ def test_runs_on_the_callers_stream(loader):
     check_against_oracle(to_host(dC, O.F16), A, B, M, N, K, 0, 0, 1, O.F16, O.F16)
 
 
+def test_two_streams_share_the_scratch_memory(loader):
+    """Split-K and padded-copy GEMMs issued from two streams at the same time (reference
+    contract: concurrent calls are safe when each has its own stream).  Both kinds keep
+    fp32 partial sums or operand copies in the library's one per-device buffer; every
+    result must equal, bit for bit, what the same call gives when nothing else runs."""
+    import torch
+
+    cases = [  # (M, N, K, lc, la, lb): split-K (skinny, long K) and padded copies (odd K)
+        (64, 8192, 8192, 0, 0, 1),
+        (1024, 1024, 16384, 0, 0, 1),
+        (128, 8192, 8192, 1, 0, 0),
+        (1025, 1031, 2049, 0, 0, 1),
+    ]
+    dev = []
+    for (M, N, K, lc, la, lb) in cases:
+        A, B = make_inputs(M, N, K, la, lb, O.F16)
+        dA, dB = to_device(A, O.F16), to_device(B, O.F16)
+        want = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+        loader.gemm(want, dA, dB, M, N, K, lc, la, lb)
+        torch.cuda.synchronize()
+        dev.append((dA, dB, want))
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    rounds = 6
+    got = [[torch.zeros_like(dev[i][2]) for _ in range(rounds)] for i in range(len(cases))]
+    for r in range(rounds):
+        for i, (M, N, K, lc, la, lb) in enumerate(cases):
+            s = streams[(i + r) % 2]
+            loader.gemm(got[i][r], dev[i][0], dev[i][1], M, N, K, lc, la, lb, stream=s)
+    torch.cuda.synchronize()
+    for i in range(len(cases)):
+        for r in range(rounds):
+            assert torch.equal(got[i][r], dev[i][2]), (cases[i], r)
+
+
 def test_cpp_client_through_this_repositorys_loader_header():
     """A C++ client of rocm_wmma_gemm::loader (all type pairs, all layouts, batched),
     bit-exact against a host loop on inputs whose sums are exact."""
