@@ -440,6 +440,40 @@ def test_two_streams_share_the_scratch_memory(loader):
             assert torch.equal(got[i][r], dev[i][2]), (cases[i], r)
 
 
+def test_replays_from_a_hip_graph(loader):
+    """GEMM calls recorded into a HIP graph (whole tiles on the persistent kernel, a ragged
+    shape, and a split-K call whose scratch memory was sized by an eager call before) give
+    the eager results on every replay, with eager work and synchronisations in between."""
+    import torch
+
+    cases = [(512, 768, 1024, 0, 0, 1), (1000, 1000, 1000, 0, 1, 0), (64, 8192, 8192, 0, 0, 1)]
+    ops = []
+    for (M, N, K, lc, la, lb) in cases:
+        A, B = make_inputs(M, N, K, la, lb, O.F16)
+        dA, dB = to_device(A, O.F16), to_device(B, O.F16)
+        want = torch.zeros(M * N, dtype=torch.float16, device="cuda")
+        loader.gemm(want, dA, dB, M, N, K, lc, la, lb)  # eager; also sizes the scratch memory
+        ops.append((dA, dB, want, torch.zeros_like(want)))
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for (M, N, K, lc, la, lb), (dA, dB, _, out) in zip(cases, ops):
+            loader.gemm(out, dA, dB, M, N, K, lc, la, lb)  # torch's current stream is capturing
+    for replay in range(3):
+        for (_, _, _, out) in ops:
+            out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for case, (dA, dB, want, out) in zip(cases, ops):
+            assert torch.equal(out, want), (case, replay)
+        # eager work between replays, through the same scratch memory
+        M, N, K, lc, la, lb = cases[2]
+        loader.gemm(ops[2][3], ops[2][0], ops[2][1], M, N, K, lc, la, lb)
+        torch.cuda.synchronize()
+        assert torch.equal(ops[2][3], ops[2][2])
+
+
 def test_cpp_client_through_this_repositorys_loader_header():
     """A C++ client of rocm_wmma_gemm::loader (all type pairs, all layouts, batched),
     bit-exact against a host loop on inputs whose sums are exact."""
