@@ -150,6 +150,83 @@ def test_split_fields_of_a_config_entry():
     assert G.split_field({"split_k": 4, "stream_k": 0}) == 4
 
 
+def _race_module():
+    sys.path.insert(0, os.path.join(ROOT, "rocm_wmma_gemm_amd", "config"))
+    import race
+
+    return race
+
+
+def _entry(M, N, K, la, lb, lc, **cfg):
+    base = {"warps_m": 2, "warps_n": 2, "warp_tile_m": 4, "warp_tile_n": 4, "swizzle": 4, "bits": 128,
+            "block_k": 64, "pipeline": 5, "split_k": 1}
+    base.update(cfg)
+    return {"range": {"M": M, "N": N, "K": K}, "layout": {"A": la, "B": lb, "C": lc}, "config": base}
+
+
+def test_race_keeps_the_faster_configuration_per_entry():
+    """File against file (reference config/race.py:160-226): a fake timer that makes
+    swizzle 8 faster than swizzle 4 and lets one configuration fail."""
+    race = _race_module()
+    r, c = "row_major", "col_major"
+    e_same = _entry(256, 256, 256, r, c, r)
+    t1 = {race.key_of(e): e for e in [e_same, _entry(4096, 4096, 4096, r, c, r, swizzle=4),
+                                      _entry(512, 512, 512, r, r, r, swizzle=4),
+                                      _entry(128, 128, 128, r, r, r)]}
+    t2 = {race.key_of(e): e for e in [e_same, _entry(4096, 4096, 4096, r, c, r, swizzle=8),
+                                      _entry(512, 512, 512, r, r, r, swizzle=16),
+                                      _entry(1024, 1024, 1024, c, c, c)]}
+    calls = []
+
+    def timer(key, cfg):
+        calls.append((key, cfg["swizzle"]))
+        return {4: 1.0, 8: 0.9, 16: None}[cfg["swizzle"]]
+
+    out = race.race_files(t1, t2, timer, rounds=5, log=lambda *_: None)
+    assert out[(4096, 4096, 4096, r, c, r)]["config"]["swizzle"] == 8     # faster one wins
+    assert out[(512, 512, 512, r, r, r)]["config"]["swizzle"] == 4         # the one that runs wins
+    assert (128, 128, 128, r, r, r) in out and (1024, 1024, 1024, c, c, c) in out  # kept
+    assert not any(k == (256, 256, 256, r, c, r) for k, _ in calls)        # equal: no race
+    # alternating order inside a race: first round starts with file 1, second with file 2
+    first = [sw for k, sw in calls if k[0] == 4096]
+    assert first[:4] == [4, 8, 8, 4] and len(first) == 10
+
+
+def test_race_head_to_head_tie_goes_to_the_lower_median():
+    race = _race_module()
+    seq = iter([1.0, 1.2, 1.3, 1.0, 1.0, 1.4, 1.5, 1.0])  # cfg1, cfg2 | cfg2, cfg1 | ...
+
+    def timer(key, cfg):
+        return next(seq)
+
+    # rounds: (1.0 vs 1.2) cfg1, (cfg2 1.3 vs cfg1 1.0) cfg1, (1.0 vs 1.4) cfg1, (cfg2 1.5, cfg1 1.0) cfg1
+    assert race.head_to_head(timer, None, {"a": 1}, {"a": 2}, 4)[:3] == (1, 4, 0)
+    both = iter([1.0, 2.0, 1.0, 3.0])  # cfg1 wins round 1, cfg2 (timed first, 1.0) wins round 2
+
+    w = race.head_to_head(lambda k, c: next(both), None, {"a": 1}, {"a": 2}, 2)
+    assert w[1:3] == (1, 1) and w[0] == 2 and w[3:] == (2.0, 1.5)
+    assert race.head_to_head(lambda k, c: None, None, {}, {"x": 1}, 3)[0] == 0
+
+
+def test_race_cross_check_pairs_a_column_major_c_problem_with_its_transposed_twin():
+    """(M, N, K, A=a, B=b, C=col) is, in kernel space, (N, M, K, A=not b, B=not a, C=row)."""
+    race = _race_module()
+    r, c = "row_major", "col_major"
+    assert race.twin_of((4096, 5120, 1024, r, r, c)) == (5120, 4096, 1024, c, c, r)
+    assert race.twin_of((64, 8192, 8192, r, c, c)) == (8192, 64, 8192, r, c, r)
+    assert race.twin_of((64, 8192, 8192, r, c, r)) is None
+    table = {race.key_of(e): e for e in [_entry(2048, 2048, 2048, r, c, c, swizzle=4),
+                                         _entry(2048, 2048, 2048, r, c, r, swizzle=16),
+                                         _entry(1000, 1000, 1000, r, r, c, swizzle=4)]}
+    out = race.cross_check(table, lambda key, cfg: {4: 2.0, 16: 1.0}[cfg["swizzle"]], 3,
+                           log=lambda *_: None)
+    assert out[(2048, 2048, 2048, r, c, c)]["config"]["swizzle"] == 16   # took the twin's
+    assert out[(2048, 2048, 2048, r, c, r)]["config"]["swizzle"] == 16
+    assert out[(1000, 1000, 1000, r, r, c)]["config"]["swizzle"] == 4    # no twin in the file
+    assert race.hook_split({"split_k": 4}) == 4 and race.hook_split({"split_k": 1, "tail_split": 3}) == -3
+    assert race.hook_split({"split_k": 1, "stream_k": 1}) == -1
+
+
 def test_shipped_json_matches_reference_schema():
     import json
 
