@@ -579,7 +579,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
             const unsigned nb = static_cast<unsigned>(std::min<size_t>(65535, p.batch - b0));
             if(copy_a)
             {
-                const dim3 ga(static_cast<unsigned>(std::min<size_t>((lda / 2 + 255) / 256, 64)),
+                const dim3 ga(static_cast<unsigned>(std::min<size_t>((lda / 8 + 255) / 256, 64)),
                               static_cast<unsigned>(std::min<size_t>(a_outer_pad, 65535)), nb);
                 device::pack_padded<unsigned short><<<ga, dim3(256), 0, stream>>>(
                     static_cast<const unsigned short*>(p.A) + b0 * p.stride_a, wa + b0 * stride_a,
@@ -589,7 +589,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
             }
             if(copy_b)
             {
-                const dim3 gb(static_cast<unsigned>(std::min<size_t>((ldb / 2 + 255) / 256, 64)),
+                const dim3 gb(static_cast<unsigned>(std::min<size_t>((ldb / 8 + 255) / 256, 64)),
                               static_cast<unsigned>(std::min<size_t>(b_outer_pad, 65535)), nb);
                 device::pack_padded<unsigned short><<<gb, dim3(256), 0, stream>>>(
                     static_cast<const unsigned short*>(p.B) + b0 * p.stride_b, wb + b0 * stride_b,

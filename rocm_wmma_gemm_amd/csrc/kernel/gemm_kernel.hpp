@@ -791,10 +791,14 @@ __global__ void __launch_bounds__(256) reduce_stream_tiles(OutT* __restrict__ C,
 }
 
 // Copies a dense 2-D array of 16-bit elements (`outer` rows of `inner` contiguous
-// elements, any alignment) into a zero-padded one whose rows are `inner_pad` long and
-// 16-byte aligned and which has `outer_pad` rows.  Lets ragged or misaligned operands
-// take the direct-to-LDS kernels, which need whole tiles and aligned rows; the zero
-// padding along K adds nothing to the products.
+// elements, any alignment down to 2 bytes) into a zero-padded one whose rows are
+// `inner_pad` long (a multiple of 8) and 16-byte aligned and which has `outer_pad` rows.
+// Lets ragged or misaligned operands take the direct-to-LDS kernels, which need whole
+// tiles and aligned rows; the zero padding along K adds nothing to the products.
+// A thread writes one 16-byte piece.  It reads the two aligned 16-byte blocks that hold
+// the piece's 8 source elements (the second only if it starts before the end of the
+// source row) and shifts them into place; an aligned block that holds an element of the
+// array lies in that element's page, so nothing is read from a page the array is not on.
 template<class Elem16>
 __global__ void __launch_bounds__(256) pack_padded(const Elem16* __restrict__ src,
                                                    Elem16* __restrict__ dst,
@@ -806,27 +810,48 @@ __global__ void __launch_bounds__(256) pack_padded(const Elem16* __restrict__ sr
                                                    long long dst_batch_stride)
 {
     static_assert(sizeof(Elem16) == 2, "16-bit elements only");
-    const Elem16* s = src + blockIdx.z * src_batch_stride;
-    unsigned int*         d = reinterpret_cast<unsigned int*>(dst + blockIdx.z * dst_batch_stride);
-    const int             pairs = inner_pad / 2; // inner_pad is even
+    const Elem16* s      = src + blockIdx.z * src_batch_stride;
+    u32x4*        d      = reinterpret_cast<u32x4*>(dst + blockIdx.z * dst_batch_stride);
+    const int     pieces = inner_pad / 8;
     for(int o = blockIdx.y; o < outer_pad; o += gridDim.y)
     {
-        const Elem16* row = s + (long long)o * inner;
-        for(int i = blockIdx.x * blockDim.x + threadIdx.x; i < pairs; i += gridDim.x * blockDim.x)
+        for(int i = blockIdx.x * blockDim.x + threadIdx.x; i < pieces; i += gridDim.x * blockDim.x)
         {
-            unsigned int lo = 0u, hi = 0u;
-            if(o < outer)
+            u32x4 out = {0u, 0u, 0u, 0u};
+            if(o < outer && 8 * i < inner)
             {
-                if(2 * i < inner)
+                const unsigned long long first = reinterpret_cast<unsigned long long>(s + (long long)o * inner + 8 * i);
+                const unsigned long long end   = reinterpret_cast<unsigned long long>(s + (long long)(o + 1) * inner);
+                const u32x4*             block = reinterpret_cast<const u32x4*>(first & ~15ull);
+                const u32x4              b0    = block[0];
+                u32x4                    b1    = {0u, 0u, 0u, 0u};
+                if((first & 15ull) != 0 && reinterpret_cast<unsigned long long>(block + 1) < end)
                 {
-                    lo = row[2 * i];
+                    b1 = block[1];
                 }
-                if(2 * i + 1 < inner)
+                const unsigned int w[8] = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+                const int          q    = static_cast<int>(first & 15ull) >> 2; // whole words to skip
+                const bool         half = (first & 2ull) != 0; // and half a word more
+                const int          valid = inner - 8 * i; // elements of the piece that the row holds
+#pragma unroll
+                for(int k = 0; k < 4; ++k)
                 {
-                    hi = row[2 * i + 1];
+                    unsigned int lo = w[k], hi = w[k + 1];
+#pragma unroll
+                    for(int t = 1; t < 4; ++t)
+                    {
+                        lo = q == t ? w[k + t] : lo;
+                        hi = q == t ? w[k + t + 1] : hi;
+                    }
+                    unsigned int v = half ? (lo >> 16) | (hi << 16) : lo;
+                    if(2 * k + 1 >= valid)
+                    {
+                        v &= 2 * k >= valid ? 0u : 0xffffu;
+                    }
+                    out[k] = v;
                 }
             }
-            d[(long long)o * pairs + i] = lo | (hi << 16);
+            d[(long long)o * pieces + i] = out;
         }
     }
 }
