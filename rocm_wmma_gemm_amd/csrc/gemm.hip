@@ -579,8 +579,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
             const unsigned nb = static_cast<unsigned>(std::min<size_t>(65535, p.batch - b0));
             if(copy_a)
             {
-                const dim3 ga(static_cast<unsigned>(std::min<size_t>((lda / 8 + 255) / 256, 64)),
-                              static_cast<unsigned>(std::min<size_t>(a_outer_pad, 65535)), nb);
+                const dim3 ga(static_cast<unsigned>(std::min<size_t>((a_outer_pad * (lda / 8) + 255) / 256, 8192)), 1, nb);
                 device::pack_padded<unsigned short><<<ga, dim3(256), 0, stream>>>(
                     static_cast<const unsigned short*>(p.A) + b0 * p.stride_a, wa + b0 * stride_a,
                     static_cast<int>(a_outer), static_cast<int>(a_inner), static_cast<int>(a_outer_pad),
@@ -589,8 +588,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
             }
             if(copy_b)
             {
-                const dim3 gb(static_cast<unsigned>(std::min<size_t>((ldb / 8 + 255) / 256, 64)),
-                              static_cast<unsigned>(std::min<size_t>(b_outer_pad, 65535)), nb);
+                const dim3 gb(static_cast<unsigned>(std::min<size_t>((b_outer_pad * (ldb / 8) + 255) / 256, 8192)), 1, nb);
                 device::pack_padded<unsigned short><<<gb, dim3(256), 0, stream>>>(
                     static_cast<const unsigned short*>(p.B) + b0 * p.stride_b, wb + b0 * stride_b,
                     static_cast<int>(b_outer), static_cast<int>(b_inner), static_cast<int>(b_outer_pad),

@@ -813,10 +813,14 @@ __global__ void __launch_bounds__(256) pack_padded(const Elem16* __restrict__ sr
     const Elem16* s      = src + blockIdx.z * src_batch_stride;
     u32x4*        d      = reinterpret_cast<u32x4*>(dst + blockIdx.z * dst_batch_stride);
     const int     pieces = inner_pad / 8;
-    for(int o = blockIdx.y; o < outer_pad; o += gridDim.y)
+    // (all pieces of the copy in one sequence, so that small arrays still fill workgroups)
+    const long long total = (long long)outer_pad * pieces;
+    for(long long at = (long long)blockIdx.x * blockDim.x + threadIdx.x; at < total;
+        at += (long long)gridDim.x * blockDim.x)
     {
-        for(int i = blockIdx.x * blockDim.x + threadIdx.x; i < pieces; i += gridDim.x * blockDim.x)
         {
+            const int o = static_cast<int>(at / pieces);
+            const int i = static_cast<int>(at - (long long)o * pieces);
             u32x4 out = {0u, 0u, 0u, 0u};
             if(o < outer && 8 * i < inner)
             {
