@@ -110,6 +110,68 @@ def test_ragged_and_tiny_shapes(loader, type_name, lc, la, lb):
         check_against_oracle(gpu, A, B, M, N, K, lc, la, lb, din, dout)
 
 
+def _random_problems(seed, count):
+    """Seeded shapes across the dispatcher's classes: extents that are multiples of 64, of
+    8, even, odd; tiny to a few tiles; every layout and type pair; some strided batches."""
+    rng = np.random.RandomState(seed)
+
+    def extent(hi):
+        kind = rng.randint(4)
+        if kind == 0:
+            return 64 * rng.randint(1, hi // 64 + 1)
+        if kind == 1:
+            return 8 * rng.randint(1, hi // 8 + 1)
+        if kind == 2:
+            return 2 * rng.randint(1, hi // 2 + 1)
+        return rng.randint(1, hi + 1)
+
+    names = list(TYPE_PAIRS)
+    out = []
+    for _ in range(count):
+        M, N, K = extent(1400), extent(1400), extent(2600)
+        lc, la, lb = LAYOUTS8[rng.randint(8)]
+        batch = 1 if M * N > 300000 else int(rng.choice([1, 1, 2, 3]))
+        out.append((M, N, K, lc, la, lb, names[rng.randint(4)], batch))
+    return out
+
+
+@pytest.mark.parametrize("chunk", range(4))
+def test_seeded_random_shapes_through_the_default_dispatch(loader, chunk):
+    """48 seeded problems that have no tuned entry, so the time-estimate model or the
+    nearest entry picks kernel, tile, split and copies for them; each checked element by
+    element against the oracle (strided batches: every entry against its own slice)."""
+    for (M, N, K, lc, la, lb, tname, batch) in _random_problems(20240 + chunk, 12):
+        din, dout = TYPE_PAIRS[tname]
+        As, Bs = [], []
+        for b in range(batch):
+            A, B = make_inputs(M, N, K, la, lb, din, seed_a=11 + 2 * b, seed_b=12 + 2 * b)
+            As.append(A)
+            Bs.append(B)
+        print(f"random problem {M}x{N}x{K} layouts(C,A,B)=({lc},{la},{lb}) {tname} batch {batch}", flush=True)
+        gpu = run_gpu(loader, np.concatenate(As), np.concatenate(Bs), M, N, K, lc, la, lb, din, dout, batch=batch)
+        for b in range(batch):
+            check_against_oracle(gpu[b * M * N:(b + 1) * M * N], As[b], Bs[b], M, N, K, lc, la, lb, din, dout)
+
+
+def test_seeded_random_large_shapes_through_the_default_dispatch(loader):
+    """The same for 10 problems of many tiles (extents 1500..5200, K 500..4200, all
+    alignment classes): every element through the row/column checksums, two 32-row bands
+    element by element."""
+    rng = np.random.RandomState(777)
+    names = list(TYPE_PAIRS)
+    for n in range(10):
+        step = [64, 8, 2, 1][n % 4]
+        M = step * rng.randint(1500 // step, 5200 // step + 1)
+        N = [64, 8, 1, 2][rng.randint(4)] * 1
+        N = N * rng.randint(1500 // N, 5200 // N + 1)
+        kstep = [64, 8, 1][rng.randint(3)]
+        K = kstep * rng.randint(500 // kstep, 4200 // kstep + 1)
+        lc, la, lb = LAYOUTS8[rng.randint(8)]
+        tname = names[rng.randint(4)]
+        print(f"random problem {M}x{N}x{K} layouts(C,A,B)=({lc},{la},{lb}) {tname}", flush=True)
+        _full_size_case(loader, M, N, K, lc, la, lb, tname, (0, M - 32), seed_a=21 + n, seed_b=40 + n)
+
+
 @pytest.mark.parametrize("type_name", ["f16_f16", "f32_bf16"])
 def test_unaligned_base_pointers(loader, type_name):
     """A, B and C starting one element past a 16-byte boundary: vector loads are not
