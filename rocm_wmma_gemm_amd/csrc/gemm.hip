@@ -577,24 +577,35 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         for(size_t b0 = 0; b0 < p.batch; b0 += 65535)
         {
             const unsigned nb = static_cast<unsigned>(std::min<size_t>(65535, p.batch - b0));
+            device::pack_job jobs[2];
+            unsigned         count = 0, blocks = 0;
+            auto add = [&](const void* src, unsigned short* dst, size_t outer, size_t inner, size_t outer_pad,
+                           size_t inner_pad, size_t src_stride, size_t dst_stride) {
+                jobs[count++] = {static_cast<const unsigned short*>(src) + b0 * src_stride,
+                                 dst + b0 * dst_stride,
+                                 static_cast<int>(outer),
+                                 static_cast<int>(inner),
+                                 static_cast<int>(outer_pad),
+                                 static_cast<int>(inner_pad),
+                                 static_cast<long long>(src_stride),
+                                 static_cast<long long>(dst_stride)};
+                blocks = std::max(blocks,
+                                  static_cast<unsigned>(std::min<size_t>((outer_pad * (inner_pad / 8) + 255) / 256, 8192)));
+            };
             if(copy_a)
             {
-                const dim3 ga(static_cast<unsigned>(std::min<size_t>((a_outer_pad * (lda / 8) + 255) / 256, 8192)), 1, nb);
-                device::pack_padded<unsigned short><<<ga, dim3(256), 0, stream>>>(
-                    static_cast<const unsigned short*>(p.A) + b0 * p.stride_a, wa + b0 * stride_a,
-                    static_cast<int>(a_outer), static_cast<int>(a_inner), static_cast<int>(a_outer_pad),
-                    static_cast<int>(lda), static_cast<long long>(p.stride_a),
-                    static_cast<long long>(stride_a));
+                add(p.A, wa, a_outer, a_inner, a_outer_pad, lda, p.stride_a, stride_a);
             }
             if(copy_b)
             {
-                const dim3 gb(static_cast<unsigned>(std::min<size_t>((b_outer_pad * (ldb / 8) + 255) / 256, 8192)), 1, nb);
-                device::pack_padded<unsigned short><<<gb, dim3(256), 0, stream>>>(
-                    static_cast<const unsigned short*>(p.B) + b0 * p.stride_b, wb + b0 * stride_b,
-                    static_cast<int>(b_outer), static_cast<int>(b_inner), static_cast<int>(b_outer_pad),
-                    static_cast<int>(ldb), static_cast<long long>(p.stride_b),
-                    static_cast<long long>(stride_b));
+                add(p.B, wb, b_outer, b_inner, b_outer_pad, ldb, p.stride_b, stride_b);
             }
+            if(count == 1)
+            {
+                jobs[1] = jobs[0];
+            }
+            // one launch for both operands: a dependent launch costs as much as a small copy
+            device::pack_padded<unsigned short><<<dim3(blocks, count, nb), dim3(256), 0, stream>>>(jobs[0], jobs[1]);
         }
         if(copy_a)
         {

@@ -799,19 +799,29 @@ __global__ void __launch_bounds__(256) reduce_stream_tiles(OutT* __restrict__ C,
 // the piece's 8 source elements (the second only if it starts before the end of the
 // source row) and shifts them into place; an aligned block that holds an element of the
 // array lies in that element's page, so nothing is read from a page the array is not on.
+// One array to copy: see pack_padded.
+struct pack_job
+{
+    const void* src;
+    void*       dst;
+    int         outer, inner; // source rows and row length
+    int         outer_pad, inner_pad; // the same of the copy
+    long long   src_batch_stride, dst_batch_stride; // elements
+};
+
+// blockIdx.y picks the job (both operands of a GEMM go in one launch), blockIdx.z the
+// batch entry.
 template<class Elem16>
-__global__ void __launch_bounds__(256) pack_padded(const Elem16* __restrict__ src,
-                                                   Elem16* __restrict__ dst,
-                                                   int       outer,
-                                                   int       inner,
-                                                   int       outer_pad,
-                                                   int       inner_pad,
-                                                   long long src_batch_stride,
-                                                   long long dst_batch_stride)
+__global__ void __launch_bounds__(256) pack_padded(const pack_job first_job, const pack_job second_job)
 {
     static_assert(sizeof(Elem16) == 2, "16-bit elements only");
-    const Elem16* s      = src + blockIdx.z * src_batch_stride;
-    u32x4*        d      = reinterpret_cast<u32x4*>(dst + blockIdx.z * dst_batch_stride);
+    const pack_job& job       = blockIdx.y == 0 ? first_job : second_job;
+    const int       outer     = job.outer;
+    const int       inner     = job.inner;
+    const int       outer_pad = job.outer_pad;
+    const int       inner_pad = job.inner_pad;
+    const Elem16*   s = static_cast<const Elem16*>(job.src) + blockIdx.z * job.src_batch_stride;
+    u32x4*          d = reinterpret_cast<u32x4*>(static_cast<Elem16*>(job.dst) + blockIdx.z * job.dst_batch_stride);
     const int     pieces = inner_pad / 8;
     // (all pieces of the copy in one sequence, so that small arrays still fill workgroups)
     const long long total = (long long)outer_pad * pieces;
