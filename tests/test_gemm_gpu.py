@@ -502,6 +502,52 @@ def test_two_streams_share_the_scratch_memory(loader):
             assert torch.equal(got[i][r], dev[i][2]), (cases[i], r)
 
 
+def test_two_host_threads_each_on_its_own_stream(loader):
+    """The reference's threading contract (no mutable state behind the loader: concurrent
+    gemm calls from several host threads are safe when each uses its own stream), on
+    shapes that share the library's scratch buffer and on one that does not."""
+    import threading
+
+    import torch
+
+    cases = [(64, 8192, 8192, 0, 0, 1), (1025, 1031, 2049, 0, 0, 1), (512, 768, 1024, 0, 0, 1)]
+    dev = []
+    for (M, N, K, lc, la, lb) in cases:
+        A, B = make_inputs(M, N, K, la, lb, O.F16)
+        dA, dB = to_device(A, O.F16), to_device(B, O.F16)
+        want = torch.zeros(M * N, dtype=torch.float16, device="cuda")
+        loader.gemm(want, dA, dB, M, N, K, lc, la, lb)
+        dev.append((dA, dB, want))
+    torch.cuda.synchronize()
+    rounds, errors = 8, []
+    outs = [[[torch.zeros_like(dev[i][2]) for _ in range(rounds)] for i in range(len(cases))] for _ in range(2)]
+
+    def worker(t):
+        try:
+            torch.cuda.set_device(0)
+            s = torch.cuda.Stream()
+            for r in range(rounds):
+                for i in range(len(cases)):
+                    j = (i + t) % len(cases)
+                    M, N, K, lc, la, lb = cases[j]
+                    loader.gemm(outs[t][j][r], dev[j][0], dev[j][1], M, N, K, lc, la, lb, stream=s)
+            s.synchronize()
+        except Exception as e:  # surfaced in the main thread below
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=120)
+    assert not errors and not any(th.is_alive() for th in threads), errors
+    torch.cuda.synchronize()
+    for t in range(2):
+        for i in range(len(cases)):
+            for r in range(rounds):
+                assert torch.equal(outs[t][i][r], dev[i][2]), (t, cases[i], r)
+
+
 def test_replays_from_a_hip_graph(loader):
     """GEMM calls recorded into a HIP graph (whole tiles on the persistent kernel, a ragged
     shape, and a split-K call whose scratch memory was sized by an eager call before) give
