@@ -74,7 +74,8 @@ int rocm_wmma_gemm_variant_info_get(int variant, rocm_wmma_gemm_variant_info* in
 
 /* Which variant the dispatcher would pick for this problem (the table built from
  * gemm_config_gfx950_*.json, then shape heuristics).  type_idx as above.
- * Also reports the swizzle (tile-row group height) and the split field: s > 1 = every
+ * Also reports the swizzle (band height of the tile walk: g > 0 bands of g tile rows,
+ * g < 0 bands of -g tile columns) and the split field: s > 1 = every
  * tile's K range is cut into s slices; -s < -1 = only the tiles of the last, partial
  * wave over the compute units are cut into s slices; -1 = the persistent kernel's
  * workgroups each take the same number of K tiles of the sequence of all K tiles of the

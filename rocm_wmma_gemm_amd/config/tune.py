@@ -81,7 +81,8 @@ def candidates(variants, M, N, K, lc):
         # a tile much larger than the problem only wastes work
         if (v.block_m >= 192 and rows < 192) or (v.block_n >= 192 and cols < 192):
             continue
-        swizzles = [1] if tiles <= 8 else [4, 8, 16]
+        # band height of the tile walk; negative: bands of tile columns instead of rows
+        swizzles = [1] if tiles <= 8 else [4, 8, 16, -4, -8]
         splits = [1]
         if tiles < 256 and k_steps >= 16:
             for s in (2, 4, 8, 16, 32):

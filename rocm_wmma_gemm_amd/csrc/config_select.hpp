@@ -25,7 +25,7 @@ namespace host
 struct launch_plan
 {
     int variant; // index into the compiled variant table
-    int swizzle; // tile-row band height of the tile map
+    int swizzle; // band height of the tile map: s > 0 bands of s tile rows, s < 0 bands of -s tile columns
     int split_k; // K slices (1 = off); -s (s > 1) = split only the last, partial wave of tiles s
                  // ways; -1 = persistent kernel walks by K tile (equal K tiles per workgroup)
 };

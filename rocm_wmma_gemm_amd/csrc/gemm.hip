@@ -641,7 +641,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         args.batch_stride_c = static_cast<long long>(p.stride_c);
         args.grid_m         = static_cast<int>(grid_m);
         args.grid_n         = static_cast<int>(grid_n);
-        args.group          = plan.swizzle < 1 ? 1 : plan.swizzle;
+        args.group          = plan.swizzle == 0 ? 1 : plan.swizzle; // negative: bands of tile columns
         args.k_slices       = split_k;
         args.tail_begin     = static_cast<int>(tail_begin);
         args.partials       = partials;

@@ -582,7 +582,7 @@ struct direct_gemm
             const int entry = item / (int)gridDim.x;
             batch           = entry;
             w               = decode_block(args, item - entry * (int)gridDim.x);
-            t = banded_tile(w.tile_id, args.grid_m, args.grid_n, args.group < 1 ? 1 : args.group);
+            t = banded_tile(w.tile_id, args.grid_m, args.grid_n, args.group);
         }
         else
         {

@@ -61,7 +61,7 @@ struct gemm_args
                           // K (or the padded K) if K-contiguous, else the row count
     long long   batch_stride_a, batch_stride_b, batch_stride_c; // elements
     int         grid_m, grid_n; // tiles along M and N
-    int         group; // tile-row band height of the tile map
+    int         group; // band height of the tile map (banded_tile): > 0 tile rows, < 0 tile columns
     int         k_slices; // split-K factor of the split tiles (1 = off)
     int         tail_begin; // tiles [0, tail_begin) of the walk order run whole K, the rest are
                             // split k_slices ways; 0 = every tile is split (plain split-K)

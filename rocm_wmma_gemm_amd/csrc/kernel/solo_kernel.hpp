@@ -609,7 +609,7 @@ struct solo_gemm
             x.batch            = item / args.blocks_per_batch;
             const block_work w = decode_block(args, item - x.batch * args.blocks_per_batch);
             const tile_coord t = args.batch_by_xcd
-                                     ? banded_tile(w.tile_id, args.grid_m, args.grid_n, args.group < 1 ? 1 : args.group)
+                                     ? banded_tile(w.tile_id, args.grid_m, args.grid_n, args.group)
                                      : map_tile(w.tile_id, args.grid_m, args.grid_n, args.group);
             x.row0             = t.m * BM;
             x.col0             = t.n * BN;

@@ -2,7 +2,7 @@
 // L2 each.  The hardware deals consecutive workgroup ids round-robin over the
 // XCDs, so ids that are congruent mod 8 share an L2.  The map first renumbers
 // the ids so that every XCD owns one contiguous run of "logical" ids, then walks
-// the tile grid in bands of `group` tile rows, column by column inside a band,
+// the tile grid in bands of `group` tile rows (or columns), column by column inside a band,
 // so that a run of logical ids covers a compact group x (run/group) rectangle of
 // C and re-uses the same A row panels and B column panels out of that L2.
 //
@@ -46,28 +46,32 @@ RWG_HD inline int xcd_remap(int wg, int total)
     return tall * per_xcd + (xcd - tall) * (per_xcd - 1) + local;
 }
 
-// Banded walk: bands of `group` tile rows; inside a band, down a column first.
+// Banded walk.  group > 0: bands of `group` tile rows; inside a band, down a column
+// first.  group < 0: the mirror image, bands of -group tile columns, along a row first
+// (a grid that is wider than tall then gives an XCD the rectangle that the upright walk
+// gives it on the transposed grid).  group 0 counts as 1.
 RWG_HD inline tile_coord banded_tile(int id, int grid_m, int grid_n, int group)
 {
-    const int per_band = group * grid_n;
-    const int band     = id / per_band;
-    const int first_m  = band * group;
-    const int rows     = (grid_m - first_m) < group ? (grid_m - first_m) : group;
-    const int in_band  = id - band * per_band;
+    const bool mirrored = group < 0;
+    const int  g        = mirrored ? -group : (group == 0 ? 1 : group);
+    const int  tall     = mirrored ? grid_n : grid_m; // the dimension the bands cut
+    const int  wide     = mirrored ? grid_m : grid_n;
+    const int  per_band = g * wide;
+    const int  band     = id / per_band;
+    const int  first    = band * g;
+    const int  rows     = (tall - first) < g ? (tall - first) : g;
+    const int  in_band  = id - band * per_band;
+    const int  along    = first + in_band % rows;
+    const int  across   = in_band / rows;
     tile_coord t;
-    t.m = first_m + in_band % rows;
-    t.n = in_band / rows;
+    t.m = mirrored ? across : along;
+    t.n = mirrored ? along : across;
     return t;
 }
 
 RWG_HD inline tile_coord map_tile(int wg, int grid_m, int grid_n, int group)
 {
-    const int total = grid_m * grid_n;
-    if(group < 1)
-    {
-        group = 1;
-    }
-    return banded_tile(xcd_remap(wg, total), grid_m, grid_n, group);
+    return banded_tile(xcd_remap(wg, grid_m * grid_n), grid_m, grid_n, group);
 }
 
 } // namespace device

@@ -20,7 +20,7 @@ static int fail(const char* what)
 
 static int check_tilemap()
 {
-    const int groups[] = {1, 2, 4, 8, 16, 100};
+    const int groups[] = {0, 1, 2, 4, 8, 16, 100, -1, -2, -4, -8, -16, -100}; // negative: bands of tile columns
     for(int gm = 1; gm <= 40; ++gm)
         for(int gn = 1; gn <= 40; ++gn)
             for(int g : groups)
@@ -65,6 +65,14 @@ static int check_xcd()
         }
         if(rows.size() != 4 || cols.size() != 8)
             return fail("XCD footprint is not a 4x8 rectangle");
+    }
+    // mirrored walk (negative group): on a 16 x 32 grid with bands of 4 tile columns an
+    // XCD's 64 tiles cover what the upright walk gives it on the 32 x 16 grid, transposed
+    for(int wg = 0; wg < 512; ++wg)
+    {
+        const tile_coord a = map_tile(wg, 16, 32, -4), b = map_tile(wg, 32, 16, 4);
+        if(a.m != b.n || a.n != b.m)
+            return fail("mirrored walk is not the transpose of the upright walk");
     }
     std::printf("xcd ok\n");
     return 0;

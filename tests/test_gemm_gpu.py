@@ -283,6 +283,39 @@ def test_split_tail_wave_agrees_with_oracle(loader):
                                          f"C{lc} A{la} B{lb}: {e}") from None
 
 
+def test_mirrored_tile_walk_agrees_with_oracle(loader):
+    """Negative swizzle: the tile walk runs in bands of tile columns instead of tile rows.
+    Every pipeline, whole K, every tile split, split tail wave and (persistent kernel) the
+    walk by K tile, whose reduce kernels must find the tiles by the same mirrored walk; a
+    batched call on top (the persistent kernel then deals entries by XCD)."""
+    by_pipe = {}
+    for v in loader.variants():
+        if (v.block_m, v.block_n) in ((256, 256), (128, 128)):
+            by_pipe.setdefault(v.pipeline, v)
+    assert len(by_pipe) >= 6
+    for pipe, v in sorted(by_pipe.items()):
+        # 9 x 29 tiles of 256 (261 > 256 CUs: a tail wave of 5) or 18 x 29 of 128
+        M, N, K = (2304, 7424, 512) if v.block_m == 256 else (2304, 3700, 512)
+        splits = [1, 2, -2] + ([-1] if pipe == 5 else [])
+        for split in splits:
+            for swz in (-4, -8):
+                lc, la, lb = (0, 0, 1) if swz == -4 else (1, 0, 1)
+                din, dout = TYPE_PAIRS["f16_f16" if split > 0 else "f32_bf16"]
+                A, B = make_inputs(M, N, K, la, lb, din, seed_a=7, seed_b=8)
+                print(f"mirrored walk: variant {v.index} pipeline {pipe} split {split} swizzle {swz}", flush=True)
+                gpu = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout, variant=(v.index, swz, split))
+                checksum_check(gpu, A, B, M, N, K, lc, la, lb, din, dout)
+                check_against_oracle(gpu, A, B, M, N, K, lc, la, lb, din, dout, rows=(M - 40, M))
+    v = by_pipe[5]
+    M, N, K, batch = 512, 1280, 256, 3
+    A = np.concatenate([O.init_matrix(M, K, 0, O.F16, seed=30 + b) for b in range(batch)])
+    B = np.concatenate([O.init_matrix(K, N, 1, O.F16, seed=40 + b) for b in range(batch)])
+    gpu = run_gpu(loader, A, B, M, N, K, 0, 0, 1, O.F16, O.F16, batch=batch, variant=(v.index, -2, 1))
+    for b in range(batch):
+        check_against_oracle(gpu[b * M * N:(b + 1) * M * N], A[b * M * K:(b + 1) * M * K],
+                             B[b * K * N:(b + 1) * K * N], M, N, K, 0, 0, 1, O.F16, O.F16)
+
+
 def test_workgroups_that_take_several_tiles_agree_with_oracle(loader):
     """The one-wave-per-SIMD kernel launches one workgroup per CU, and each walks over
     work items CU count apart with ONE load stream running through them.  Cases: more
