@@ -247,8 +247,11 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
         {
             if(tiles > cus && tiles % cus != 0 && kt / s >= 4 && (tiles % cus) * s <= cus * 5 / 4)
             {
+                // (the slices of the split tiles take one more pass over the CUs, or two
+                // when there are more of them than CUs)
                 consider(launch_us + static_cast<double>(tiles / cus) * (kt * step + item)
-                             + ceil_div(kt, s) * step + item + reduce_us
+                             + static_cast<double>(ceil_div((tiles % cus) * s, cus)) * (ceil_div(kt, s) * step + item)
+                             + reduce_us
                              + (tiles % cus) * s * tile_bytes * 2.0 / tile_bytes_per_us,
                          -static_cast<int>(s));
             }

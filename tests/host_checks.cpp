@@ -158,6 +158,11 @@ static int check_select()
         return fail("model: tail split");
     // a partial last K tile with aligned rows: the persistent kernel takes it as it is,
     // every other kernel would pay padded copies of both operands
+    // 400 tiles: the 144 tiles of the tail wave cut in two would be 288 slices, two more
+    // passes over the CUs for what one pass of whole tiles does (measured 0.255 ms against
+    // 0.210 ms whole)
+    if(!model_plan(5120, 5120, 5120, 0, 0, 1, &p) || p.split_k != 1)
+        return fail("model: a tail wave whose slices need two passes stays whole");
     if(!model_plan(4096, 4096, 1000, 0, 0, 1, &p) || tiles[p.variant].pipeline != 5)
         return fail("model: ragged K with aligned rows belongs to the persistent kernel");
     // K-contiguous rows that are not 16-byte aligned, odd extents: not its business ...
