@@ -1,6 +1,7 @@
 // Implementation of the shape -> launch plan lookup (plain C++, no device code).
 #include "config_select.hpp"
 
+#include <initializer_list>
 #include <limits>
 
 #include "config_generated.hpp"
@@ -243,8 +244,12 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
         // whole tiles
         consider(launch_us + static_cast<double>(ceil_div(tiles, cus)) * (kt * step + item), 1);
         // only the last, partial wave of tiles split
-        for(size_t s = 2; s <= 4 && v.pipeline == 5; ++s)
+        for(const size_t s : {size_t{2}, size_t{3}, size_t{4}, size_t{6}, size_t{8}})
         {
+            if(v.pipeline != 5)
+            {
+                break;
+            }
             if(tiles > cus && tiles % cus != 0 && kt / s >= 4 && (tiles % cus) * s <= cus * 5 / 4)
             {
                 // (the slices of the split tiles take one more pass over the CUs, or two
