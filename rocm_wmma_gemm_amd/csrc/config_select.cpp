@@ -190,6 +190,13 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
     constexpr double reduce_us     = 4.0;
     constexpr double plane_bytes_per_us = 2.2e6; // partial planes: written, then read by reduce_partials
     constexpr double tile_bytes_per_us  = 3.7e6; // partial tiles (split tail, walk by K tile)
+    // (small planes are paid for in latency, not bandwidth: past 32 MB the rest moves at
+    // twice the rate; 8192x1024x8192 cut in two moves 134 MB in ~30 us)
+    auto plane_traffic_us = [&](double bytes) {
+        constexpr double knee = 32.0 * 1024 * 1024;
+        return bytes <= knee ? bytes / plane_bytes_per_us
+                             : knee / plane_bytes_per_us + (bytes - knee) / (2.0 * plane_bytes_per_us);
+    };
     const size_t     kt            = ceil_div(k, size_t{64});
     double           best          = 0.0;
     bool             found         = false;
@@ -271,7 +278,7 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
                     break;
                 }
                 consider(launch_us + static_cast<double>(ceil_div(tiles * s, cus)) * (ceil_div(kt, s) * step + item)
-                             + reduce_us + s * tiles * tile_bytes * 2.0 / plane_bytes_per_us,
+                             + reduce_us + plane_traffic_us(s * tiles * tile_bytes * 2.0),
                          static_cast<int>(s));
             }
         }
