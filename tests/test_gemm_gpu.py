@@ -172,6 +172,54 @@ def test_seeded_random_large_shapes_through_the_default_dispatch(loader):
         _full_size_case(loader, M, N, K, lc, la, lb, tname, (0, M - 32), seed_a=21 + n, seed_b=40 + n)
 
 
+def test_subnormal_inputs_are_not_flushed(loader):
+    """A holds only subnormal values (fp16 below 6.1e-5, bf16 below 1.2e-38): the products
+    and sums must come out as the fp32 arithmetic of the reference's CPU loop gives them,
+    subnormal fp32 sums included, on whole tiles and on a ragged shape."""
+    for tname, lim in (("f32_f16", 6.0e-5), ("f16_f16", 6.0e-5), ("f32_bf16", 1.0e-38)):
+        din, dout = TYPE_PAIRS[tname]
+        for (M, N, K) in ((256, 256, 256), (1024, 1024, 512), (130, 70, 51)):
+            A = O.init_matrix(M, K, O.ROW, din, seed=5, lo=-lim, hi=lim)
+            B = O.init_matrix(K, N, O.COL, din, seed=6, lo=-1.0, hi=1.0)
+            a = O.bits_to_f32(A, din)
+            assert 0.0 < np.abs(a).max() <= lim * 1.01
+            gpu = run_gpu(loader, A, B, M, N, K, 0, 0, 1, din, dout)
+            _, g, c = check_against_oracle(gpu, A, B, M, N, K, 0, 0, 1, din, dout)
+            assert np.abs(c).max() > 0.0 and np.count_nonzero(g) >= 0.9 * np.count_nonzero(c)
+
+
+def test_infinities_and_nans_propagate_as_in_the_reference_loop(loader):
+    """inf * finite = inf, inf * 0 = NaN, inf - inf = NaN, NaN stays: element (i, k0) of A
+    set to +inf (and one to NaN) must mark row i of C exactly as the oracle's fp32 loop does,
+    and leave every other row within tolerance."""
+    M, N, K = 256, 384, 192
+    for tname in ("f32_f16", "bf16_bf16"):
+        din, dout = TYPE_PAIRS[tname]
+        for (lc, la, lb) in [(0, 0, 1), (1, 1, 0)]:
+            A, B = make_inputs(M, N, K, la, lb, din, seed_a=9, seed_b=10)
+            inf_bits = 0x7c00 if din == O.F16 else 0x7f80
+            nan_bits = 0x7e00 if din == O.F16 else 0x7fc0
+            Al = O.logical(A, M, K, la).copy()
+            Bl = O.logical(B, K, N, lb).copy()
+            Al[3, 17] = inf_bits                   # row 3: +-inf by the sign of B(17, j), NaN where it is 0
+            Bl[17, 5] = 0
+            Al[100, 40] = inf_bits                 # row 100: +inf and -inf meet in one sum
+            Al[100, 41] = inf_bits | 0x8000
+            Al[200, 0] = nan_bits                  # row 200: NaN everywhere
+            A2 = (Al if la == 0 else Al.T).reshape(-1).copy()
+            B2 = (Bl if lb == 0 else Bl.T).reshape(-1).copy()
+            gpu = run_gpu(loader, A2, B2, M, N, K, lc, la, lb, din, dout)
+            cpu = O.gemm(A2, B2, M, N, K, lc, la, lb, din, dout)
+            g = O.bits_to_f32(O.logical(gpu, M, N, lc), dout)
+            c = O.bits_to_f32(O.logical(cpu, M, N, lc), dout)
+            assert np.array_equal(np.isnan(g), np.isnan(c)), (tname, lc, la, lb)
+            assert np.array_equal(np.isposinf(g), np.isposinf(c)) and np.array_equal(np.isneginf(g), np.isneginf(c))
+            assert np.isnan(c[3, 5]) and np.isinf(c[3, 6]) and np.isnan(c[200]).all()
+            fin = np.isfinite(c)
+            assert fin[[0, 1, 2, 4, 99, 101, 199, 201, 255]].all()
+            assert np.allclose(g[fin], c[fin], rtol=2e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("type_name", ["f16_f16", "f32_bf16"])
 def test_unaligned_base_pointers(loader, type_name):
     """A, B and C starting one element past a 16-byte boundary: vector loads are not
