@@ -549,6 +549,32 @@ def test_runs_on_the_callers_stream(loader):
     check_against_oracle(to_host(dC, O.F16), A, B, M, N, K, 0, 0, 1, O.F16, O.F16)
 
 
+def test_repeated_calls_give_identical_bits(loader):
+    """Every reduction runs in a fixed order (K slices ascending, parts of a tile by
+    workgroup number), so a call repeated with other work in between returns the same
+    bits: whole tiles, every tile split, split tail wave, walk by K tile, padded copies."""
+    import torch
+
+    shapes = [(4096, 4096, 4096), (64, 8192, 8192), (4096, 5120, 5120), (1024, 1024, 65536),
+              (4095, 5121, 3001), (1000, 1000, 1000)]
+    other = torch.ones(512 * 512, dtype=torch.float16, device="cuda")
+    other_c = torch.empty(512 * 512, dtype=torch.float32, device="cuda")
+    for (M, N, K) in shapes:
+        for (lc, la, lb) in [(0, 0, 1), (1, 1, 0)]:
+            dA = (torch.rand(M * K, device="cuda") * 2 - 1).to(torch.float16)
+            dB = (torch.rand(K * N, device="cuda") * 2 - 1).to(torch.float16)
+            outs = []
+            for _ in range(3):
+                c = torch.full((M * N,), float("nan"), dtype=torch.float32, device="cuda")
+                loader.gemm(c, dA, dB, M, N, K, lc, la, lb)
+                loader.gemm(other_c, other, other, 512, 512, 512, 0, 0, 1)
+                loader.gemm(other_c, other, other, 16, 128, 2048, 0, 0, 1)  # a split-K call in between
+                outs.append(c)
+            torch.cuda.synchronize()
+            assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2]), (M, N, K, lc, la, lb)
+            assert not torch.isnan(outs[0]).any()
+
+
 def test_two_streams_share_the_scratch_memory(loader):
     """Split-K and padded-copy GEMMs issued from two streams at the same time (reference
     contract: concurrent calls are safe when each has its own stream).  Both kinds keep
