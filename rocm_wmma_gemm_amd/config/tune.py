@@ -42,6 +42,11 @@ DEFAULT_SHAPES = [
     (128, 128, 128), (256, 256, 256), (512, 512, 512),
     # square sizes whose tile count does not divide by the CU count
     (1536, 1536, 1536), (3072, 3072, 3072), (6144, 6144, 6144),
+    # transformer projection shapes (hidden 4096 / 8192, feed-forward 11008 / 14336 / 28672)
+    (4096, 11008, 4096), (4096, 4096, 11008), (8192, 8192, 4096), (4096, 12288, 4096),
+    (8192, 1024, 8192), (4096, 4096, 14336), (2048, 8192, 2048), (12288, 4096, 4096),
+    (5120, 5120, 5120), (8192, 3584, 7168), (7168, 7168, 7168), (8192, 28672, 8192),
+    (8192, 8192, 28672),
 ]
 
 
