@@ -32,6 +32,10 @@ SETS = {
     # projection, decode-like, ragged and long-K shapes
     "other": "8192,4096,2048:4096,14336,4096:16,8192,8192:64,8192,8192:128,8192,8192:"
              "4095,5121,3001:1000,1000,1000:1024,1024,65536:3072,3072,3072:6144,6144,6144",
+    # transformer projection shapes (hidden 4096 / 8192 against 11008 / 12288 / 14336 / 28672)
+    "projection": "4096,11008,4096:4096,4096,11008:8192,8192,4096:4096,12288,4096:8192,1024,8192:"
+                  "4096,4096,14336:2048,8192,2048:12288,4096,4096:5120,5120,5120:8192,3584,7168:"
+                  "7168,7168,7168:8192,28672,8192:8192,8192,28672",
     # many small problems in one strided-batch call (run with --batch_count, default 64)
     "batched": "128,128,128:256,256,256:512,512,512:1024,1024,1024:256,256,4096:"
                "384,640,512:1000,1000,1000:2048,2048,2048",
@@ -134,6 +138,7 @@ def main(argv=None) -> int:
     res = run_bench(a.type, shapes, a.reps, batch)
     title = {"square": "Square matrices", "rectangle": "Rectangular matrices",
              "other": "Projection, skinny, ragged and long-K shapes",
+             "projection": "Transformer projection shapes",
              "batched": f"Strided batches of {batch} small problems"}.get(a.set, "Selected shapes")
     flops = "2·M·N·K" if batch == 1 else f"{batch}·2·M·N·K"
     lines = [f"# {title}: this library and rocBLAS on one MI355X\n",
