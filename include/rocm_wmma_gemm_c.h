@@ -54,6 +54,15 @@ void rocm_wmma_gemm_f32_bf16(void* C, void* A, void* B, size_t M, size_t N, size
 #define ROCM_WMMA_GEMM_TYPE_BF16_BF16 2
 #define ROCM_WMMA_GEMM_TYPE_F32_BF16 3
 
+/* Status codes of the additions that return int (the four reference entry points return
+ * void, as in the reference). */
+#define ROCM_WMMA_GEMM_OK 0
+#define ROCM_WMMA_GEMM_ERR_VARIANT (-1)  /* the forced variant cannot run this problem */
+#define ROCM_WMMA_GEMM_ERR_ARGUMENT (-2) /* type index, variant index or layout code out of range */
+#define ROCM_WMMA_GEMM_ERR_SCRATCH (-3)  /* the call needs more scratch memory than the fixed buffer holds */
+#define ROCM_WMMA_GEMM_ERR_RUNTIME (-4)  /* the HIP runtime reported an error (symbol lookup, launch) */
+#define ROCM_WMMA_GEMM_ERR_LIMIT (-5)    /* M, N or K beyond 31 bits, tile grid too large, or no kernel built */
+
 /* Description of one compiled kernel variant. */
 typedef struct rocm_wmma_gemm_variant_info
 {
@@ -92,12 +101,22 @@ int rocm_wmma_gemm_select_batched(size_t M, size_t N, size_t K, size_t batch_cou
                                   int* split_k);
 
 /* Same computation as the four entry points above, but with the tile variant,
- * swizzle and split field (see above) forced (tuner hook).  Returns 0 on success, -1 if the
- * variant cannot run this problem, -2 for invalid arguments. */
+ * swizzle and split field (see above) forced (tuner hook).  Returns ROCM_WMMA_GEMM_OK,
+ * ROCM_WMMA_GEMM_ERR_VARIANT if the variant cannot run this problem, or another of the
+ * status codes above. */
 int rocm_wmma_gemm_run_variant(int type_idx, int variant, int swizzle, int split_k, void* C,
                                void* A, void* B, size_t M, size_t N, size_t K,
                                size_t batch_count, int layout_c, int layout_a, int layout_b,
                                void* stream);
+
+/* Gives the current device's library-owned scratch buffer back (split-K partial sums and
+ * padded operand copies live there: 256 MiB from the first call that needs it, more when a
+ * call needs more).  Waits for the device to finish first.  Returns 0 when the buffer is
+ * gone or was never there, 1 when it was kept because a call on a capturing stream has
+ * used it (a graph may hold its address), ROCM_WMMA_GEMM_ERR_RUNTIME without a device.
+ * The next call that needs scratch memory allocates again.  No counterpart in the
+ * reference, which owns no memory. */
+int rocm_wmma_gemm_workspace_release(void);
 
 #ifdef __cplusplus
 }

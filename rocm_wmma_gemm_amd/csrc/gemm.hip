@@ -15,6 +15,7 @@
 
 #include "config_select.hpp"
 #include "kernel_table.hpp"
+#include "workspace_policy.hpp"
 
 namespace rocm_wmma_gemm
 {
@@ -77,13 +78,16 @@ size_t out_bytes(int type_idx)
 // Library-owned scratch memory, one buffer per device: fp32 partial planes of split-K
 // and zero-padded copies of ragged or misaligned operands.  Allocated on first use,
 // grown when a call needs more (after a device-wide synchronisation, since kernels of
-// earlier calls may still be reading the old buffer), never shrunk.
+// earlier calls may still be reading the old buffer), never shrunk.  What a call may do
+// with the buffer is decided by workspace_decide (workspace_policy.hpp).
 constexpr size_t workspace_first_bytes = size_t{256} << 20;
 constexpr size_t workspace_limit_bytes = size_t{16} << 30;
 constexpr int    max_devices           = 64;
 std::mutex       workspace_mutex;
 char*            workspace_ptr[max_devices]  = {};
 size_t           workspace_size[max_devices] = {};
+// whether the buffer's address may sit in a captured graph: such a buffer is never freed
+bool workspace_lent_to_capture[max_devices] = {};
 // The call that used the buffer last: its stream, and an event recorded behind its last
 // kernel.
 hipStream_t workspace_stream[max_devices]   = {};
@@ -97,8 +101,9 @@ bool        workspace_used[max_devices]     = {};
 // host never blocks) for the event recorded behind that holder's last kernel, so two
 // streams may issue split-K or padded-copy GEMMs at the same time, from one host thread
 // or several, as they may with the kernels that need no scratch memory.  A stream under
-// graph capture is left out of this: it records and waits for nothing, and the buffer
-// must then not be shared with work outside the graph.
+// graph capture is left out of this: it records and waits for nothing (the caller orders
+// the replays of such a graph against other work that uses the buffer), it never
+// allocates, frees or synchronises, and a buffer it was given stays allocated for good.
 class workspace_lease
 {
 public:
@@ -106,7 +111,8 @@ public:
     workspace_lease(const workspace_lease&)            = delete;
     workspace_lease& operator=(const workspace_lease&) = delete;
 
-    // nullptr: no memory (or too much asked for); the lease then holds nothing
+    // nullptr: no memory (or too much asked for, or the stream is capturing and the
+    // buffer is not there yet or too small); the lease then holds nothing
     char* acquire(size_t bytes, hipStream_t stream)
     {
         if(bytes > workspace_limit_bytes || hipGetDevice(&dev_) != hipSuccess || dev_ < 0
@@ -114,19 +120,36 @@ public:
         {
             return nullptr;
         }
-        lock_ = std::unique_lock<std::mutex>(workspace_mutex);
-        if(workspace_size[dev_] < bytes)
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        if(hipStreamIsCapturing(stream, &capture) != hipSuccess)
         {
-            size_t want = std::max(bytes + bytes / 4, workspace_first_bytes);
-            if(workspace_ptr[dev_] != nullptr)
+            (void)hipGetLastError();
+            capture = hipStreamCaptureStatusNone;
+        }
+        const bool capturing = capture != hipStreamCaptureStatusNone;
+        lock_                = std::unique_lock<std::mutex>(workspace_mutex);
+        const workspace_action action = workspace_decide(workspace_size[dev_], bytes, workspace_limit_bytes,
+                                                         capturing, workspace_lent_to_capture[dev_]);
+        if(action == workspace_action::refuse)
+        {
+            lock_.unlock();
+            return nullptr;
+        }
+        if(action != workspace_action::use_existing)
+        {
+            if(action == workspace_action::grow_free_old)
             {
                 (void)hipDeviceSynchronize();
                 (void)hipFree(workspace_ptr[dev_]);
-                workspace_ptr[dev_]  = nullptr;
-                workspace_size[dev_] = 0;
-                workspace_used[dev_] = false;
             }
-            void* p = nullptr;
+            // (grow_retire_old: the old buffer stays allocated until the process ends,
+            // for the graphs that hold its address)
+            workspace_ptr[dev_]             = nullptr;
+            workspace_size[dev_]            = 0;
+            workspace_used[dev_]            = false;
+            workspace_lent_to_capture[dev_] = false;
+            const size_t want = workspace_grown_size(bytes, workspace_first_bytes);
+            void*        p    = nullptr;
             if(hipMalloc(&p, want) != hipSuccess)
             {
                 (void)hipGetLastError();
@@ -136,14 +159,12 @@ public:
             workspace_ptr[dev_]  = static_cast<char*>(p);
             workspace_size[dev_] = want;
         }
-        stream_ = stream;
-        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-        if(hipStreamIsCapturing(stream, &capture) != hipSuccess)
+        stream_  = stream;
+        ordered_ = !capturing;
+        if(capturing)
         {
-            (void)hipGetLastError();
-            capture = hipStreamCaptureStatusNone;
+            workspace_lent_to_capture[dev_] = true;
         }
-        ordered_ = capture == hipStreamCaptureStatusNone;
         if(ordered_ && workspace_released[dev_] == nullptr
            && hipEventCreateWithFlags(&workspace_released[dev_], hipEventDisableTiming) != hipSuccess)
         {
@@ -175,6 +196,15 @@ private:
     int                          dev_     = 0;
     bool                         held_    = false;
     bool                         ordered_ = false;
+};
+
+// Scratch memory that a call brings along instead of leasing the library's buffer (the
+// entry point that allocates nothing): the call takes what it needs from the front, or
+// fails when it needs more than there is.
+struct fixed_scratch
+{
+    char*  ptr;
+    size_t bytes;
 };
 
 bool aligned16(const void* p)
@@ -320,7 +350,8 @@ bool spans_fit(const variant_desc& v, bool a_kmajor, bool b_kmajor, size_t lda, 
 }
 
 template<class OutT>
-int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hipStream_t stream)
+int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hipStream_t stream,
+           const fixed_scratch* fixed)
 {
     launch_plan plan = plan_in;
     if(plan.variant < 0 || plan.variant >= num_variants)
@@ -536,7 +567,15 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
 
     char*           workspace = nullptr;
     workspace_lease lease; // held until the last kernel of this call is enqueued
-    if(pack_bytes + partial_bytes > 0)
+    if(pack_bytes + partial_bytes > 0 && fixed != nullptr)
+    {
+        if(pack_bytes + partial_bytes > fixed->bytes)
+        {
+            return ROCM_WMMA_GEMM_ERR_SCRATCH;
+        }
+        workspace = fixed->ptr;
+    }
+    else if(pack_bytes + partial_bytes > 0)
     {
         workspace = lease.acquire(pack_bytes + partial_bytes, stream);
         if(workspace == nullptr)
@@ -551,7 +590,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
                 {
                     retry.variant = 0;
                 }
-                return launch<OutT>(type_idx, retry, p, stream);
+                return launch<OutT>(type_idx, retry, p, stream, fixed);
             }
             split_k          = 1;
             tail_begin       = 0;
@@ -704,7 +743,8 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
 
 template<class OutT>
 int run(int type_idx, const launch_plan* forced, void* C, void* A, void* B, size_t M, size_t N,
-        size_t K, size_t batch, int layout_c, int layout_a, int layout_b, hipStream_t stream)
+        size_t K, size_t batch, int layout_c, int layout_a, int layout_b, hipStream_t stream,
+        const fixed_scratch* fixed)
 {
     if((layout_c | layout_a | layout_b) & ~1)
     {
@@ -746,7 +786,7 @@ int run(int type_idx, const launch_plan* forced, void* C, void* A, void* B, size
             plan.variant = 0;
         }
     }
-    return launch<OutT>(type_idx, plan, p, stream);
+    return launch<OutT>(type_idx, plan, p, stream, fixed);
 }
 
 template<class T, class U>
@@ -764,16 +804,41 @@ constexpr int type_index()
 }
 
 int run_by_type(int type_idx, const launch_plan* forced, void* C, void* A, void* B, size_t M,
-                size_t N, size_t K, size_t batch, int lc, int la, int lb, hipStream_t stream)
+                size_t N, size_t K, size_t batch, int lc, int la, int lb, hipStream_t stream,
+                const fixed_scratch* fixed = nullptr)
 {
     switch(type_idx)
     {
-        case 0: return run<_Float16>(0, forced, C, A, B, M, N, K, batch, lc, la, lb, stream);
-        case 1: return run<float>(1, forced, C, A, B, M, N, K, batch, lc, la, lb, stream);
-        case 2: return run<__bf16>(2, forced, C, A, B, M, N, K, batch, lc, la, lb, stream);
-        case 3: return run<float>(3, forced, C, A, B, M, N, K, batch, lc, la, lb, stream);
-        default: return -2;
+        case 0: return run<_Float16>(0, forced, C, A, B, M, N, K, batch, lc, la, lb, stream, fixed);
+        case 1: return run<float>(1, forced, C, A, B, M, N, K, batch, lc, la, lb, stream, fixed);
+        case 2: return run<__bf16>(2, forced, C, A, B, M, N, K, batch, lc, la, lb, stream, fixed);
+        case 3: return run<float>(3, forced, C, A, B, M, N, K, batch, lc, la, lb, stream, fixed);
+        default: return ROCM_WMMA_GEMM_ERR_ARGUMENT;
     }
+}
+
+// The same, for callers that take a status code instead of an exception (the entry points
+// that return int): a problem beyond the library's size limits, or a kernel that is not
+// there, becomes ROCM_WMMA_GEMM_ERR_LIMIT, and a launch that the runtime rejected
+// ROCM_WMMA_GEMM_ERR_RUNTIME.
+int run_with_status(int type_idx, const launch_plan* forced, void* C, void* A, void* B, size_t M,
+                    size_t N, size_t K, size_t batch, int lc, int la, int lb, hipStream_t stream,
+                    const fixed_scratch* fixed)
+{
+    int rc;
+    try
+    {
+        rc = run_by_type(type_idx, forced, C, A, B, M, N, K, batch, lc, la, lb, stream, fixed);
+    }
+    catch(const std::exception&)
+    {
+        return ROCM_WMMA_GEMM_ERR_LIMIT;
+    }
+    if(rc == 0 && hipPeekAtLastError() != hipSuccess)
+    {
+        rc = ROCM_WMMA_GEMM_ERR_RUNTIME;
+    }
+    return rc;
 }
 
 } // namespace
@@ -932,14 +997,39 @@ int rocm_wmma_gemm_run_variant(int type_idx, int variant, int swizzle, int split
     using namespace rocm_wmma_gemm::host;
     if(type_idx < 0 || type_idx >= num_types || variant < 0 || variant >= num_variants)
     {
-        return -2;
+        return ROCM_WMMA_GEMM_ERR_ARGUMENT;
     }
     launch_plan plan;
     plan.variant = variant;
     plan.swizzle = swizzle;
     plan.split_k = split_k;
-    return run_by_type(type_idx, &plan, C, A, B, M, N, K, batch_count, layout_c, layout_a,
-                       layout_b, stream_of(stream));
+    return run_with_status(type_idx, &plan, C, A, B, M, N, K, batch_count, layout_c, layout_a,
+                           layout_b, stream_of(stream), nullptr);
+}
+
+int rocm_wmma_gemm_workspace_release(void)
+{
+    using namespace rocm_wmma_gemm::host;
+    int dev = -1;
+    if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= max_devices)
+    {
+        return ROCM_WMMA_GEMM_ERR_RUNTIME;
+    }
+    std::lock_guard<std::mutex> lock(workspace_mutex);
+    if(workspace_ptr[dev] == nullptr)
+    {
+        return 0;
+    }
+    if(workspace_lent_to_capture[dev])
+    {
+        return 1; // a captured graph may hold its address
+    }
+    (void)hipDeviceSynchronize();
+    (void)hipFree(workspace_ptr[dev]);
+    workspace_ptr[dev]  = nullptr;
+    workspace_size[dev] = 0;
+    workspace_used[dev] = false;
+    return 0;
 }
 
 } // extern "C"

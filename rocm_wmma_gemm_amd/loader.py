@@ -25,6 +25,9 @@ _DEFAULT_LIB_DIR = os.path.join(_HERE, "lib")
 
 ENTRY_SUFFIXES = ("f16_f16", "f32_f16", "bf16_bf16", "f32_bf16")
 
+# status codes and the fixed scratch size of include/rocm_wmma_gemm_c.h
+OK, ERR_VARIANT, ERR_ARGUMENT, ERR_SCRATCH, ERR_RUNTIME, ERR_LIMIT = 0, -1, -2, -3, -4, -5
+
 
 class GemmLibraryError(RuntimeError):
     """Library or symbol could not be loaded (the C++ loader throws std::runtime_error)."""
@@ -152,6 +155,9 @@ class Loader:
             ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
         L.rocm_wmma_gemm_run_variant.restype = ctypes.c_int
         L.rocm_wmma_gemm_run_variant.argtypes = [ctypes.c_int] * 4 + self._ENTRY_ARGS
+        if hasattr(L, "rocm_wmma_gemm_workspace_release"):
+            L.rocm_wmma_gemm_workspace_release.restype = ctypes.c_int
+            L.rocm_wmma_gemm_workspace_release.argtypes = []
 
     def library_arch(self) -> str:
         return self._lib.rocm_wmma_gemm_arch().decode()
@@ -195,6 +201,13 @@ class Loader:
                 raise ValueError(f"{name} holds {t.numel()} elements, the problem needs {need}")
         if A.dtype != B.dtype:
             raise TypeError("A and B must share an element type")
+        # the library's own limits: beyond them its C++ side throws, which a caller that
+        # came in through ctypes could not catch
+        for name, v in (("M", M), ("N", N), ("K", K)):
+            if v < 0 or v > 0x7FFFFFFF:
+                raise ValueError(f"{name} = {v} does not fit in 31 bits")
+        if batch < 0:
+            raise ValueError("batch_count must not be negative")
 
     def gemm(self, C, A, B, M: int, N: int, K: int, layout_c=row_major, layout_a=row_major,
              layout_b=row_major, batch_count: int = 1, stream=None) -> None:
@@ -214,6 +227,11 @@ class Loader:
         handle = ctypes.c_void_p(stream_handle)
         self._entries[slot](c_ptr, a_ptr, b_ptr, M, N, K, batch_count, layout_c, layout_a,
                             layout_b, ctypes.byref(handle))
+
+    def workspace_release(self) -> int:
+        """Frees the current device's library-owned scratch buffer (0), unless a captured
+        graph may hold its address (1)."""
+        return self._lib.rocm_wmma_gemm_workspace_release()
 
     def run_variant(self, variant: int, swizzle: int, split_k: int, C, A, B, M: int, N: int,
                     K: int, layout_c=row_major, layout_a=row_major, layout_b=row_major,

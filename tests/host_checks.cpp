@@ -8,6 +8,7 @@
 
 #include "config_select.hpp"
 #include "kernel/tile_map.hpp"
+#include "workspace_policy.hpp"
 
 using namespace rocm_wmma_gemm::device;
 using namespace rocm_wmma_gemm::host;
@@ -175,6 +176,55 @@ static int check_select()
     return 0;
 }
 
+// The scratch-buffer rules: nothing allocates, frees or synchronises for a call on a
+// capturing stream, and a buffer such a call has used is never freed.
+static int check_workspace()
+{
+    using A            = workspace_action;
+    const size_t MiB   = size_t{1} << 20;
+    const size_t limit = size_t{16} << 30;
+    struct
+    {
+        size_t have, need;
+        bool   capturing, lent;
+        A      want;
+        const char* what;
+    } cases[] = {
+        {0, 4 * MiB, false, false, A::allocate, "first eager call allocates"},
+        {0, 4 * MiB, true, false, A::refuse, "first call under capture gets nothing"},
+        {256 * MiB, 4 * MiB, false, false, A::use_existing, "fits, eager"},
+        {256 * MiB, 4 * MiB, true, false, A::use_existing, "fits, capturing"},
+        {256 * MiB, 256 * MiB, true, true, A::use_existing, "fits exactly"},
+        {256 * MiB, 300 * MiB, true, false, A::refuse, "too small under capture: no growth"},
+        {256 * MiB, 300 * MiB, true, true, A::refuse, "too small under capture, lent before"},
+        {256 * MiB, 300 * MiB, false, false, A::grow_free_old, "eager growth frees the old buffer"},
+        {256 * MiB, 300 * MiB, false, true, A::grow_retire_old, "a buffer a graph may hold is kept"},
+        {256 * MiB, limit + 1, false, false, A::refuse, "beyond the limit"},
+        {0, limit + 1, false, false, A::refuse, "beyond the limit, nothing there"},
+        {0, 0, false, false, A::allocate, "a zero-byte request still gets a buffer"},
+    };
+    for(const auto& c : cases)
+    {
+        if(workspace_decide(c.have, c.need, limit, c.capturing, c.lent) != c.want)
+            return fail(c.what);
+    }
+    // whatever the state, a capturing stream never triggers an allocation or a free
+    for(size_t have : {size_t{0}, MiB, 256 * MiB})
+        for(size_t need : {size_t{1}, MiB, 257 * MiB})
+            for(bool lent : {false, true})
+            {
+                const A a = workspace_decide(have, need, limit, true, lent);
+                if(a != A::use_existing && a != A::refuse)
+                    return fail("capture must not allocate or free");
+                if(a == A::use_existing && have < need)
+                    return fail("handed out a buffer that is too small");
+            }
+    if(workspace_grown_size(4 * MiB, 256 * MiB) != 256 * MiB || workspace_grown_size(400 * MiB, 256 * MiB) != 500 * MiB)
+        return fail("grown size");
+    std::printf("workspace ok\n");
+    return 0;
+}
+
 int main(int argc, char** argv)
 {
     if(argc < 2)
@@ -185,5 +235,7 @@ int main(int argc, char** argv)
         return check_xcd();
     if(!std::strcmp(argv[1], "select"))
         return check_select();
+    if(!std::strcmp(argv[1], "workspace"))
+        return check_workspace();
     return 2;
 }
