@@ -155,8 +155,8 @@ def test_seeded_random_shapes_through_the_default_dispatch(loader, chunk):
 
 def test_seeded_random_large_shapes_through_the_default_dispatch(loader):
     """The same for 10 problems of many tiles (extents 1500..5200, K 500..4200, all
-    alignment classes): every element through the row/column checksums, two 32-row bands
-    element by element."""
+    alignment classes): every element through the row/column checksums, a 32-row band in
+    every block of 128 rows element by element."""
     rng = np.random.RandomState(777)
     names = list(TYPE_PAIRS)
     for n in range(10):
@@ -169,7 +169,7 @@ def test_seeded_random_large_shapes_through_the_default_dispatch(loader):
         lc, la, lb = LAYOUTS8[rng.randint(8)]
         tname = names[rng.randint(4)]
         print(f"random problem {M}x{N}x{K} layouts(C,A,B)=({lc},{la},{lb}) {tname}", flush=True)
-        _full_size_case(loader, M, N, K, lc, la, lb, tname, (0, M - 32), seed_a=21 + n, seed_b=40 + n)
+        _full_size_case(loader, M, N, K, lc, la, lb, tname, seed_a=21 + n, seed_b=40 + n)
 
 
 def test_subnormal_inputs_are_not_flushed(loader):
@@ -655,6 +655,65 @@ def test_two_host_threads_each_on_its_own_stream(loader):
                 assert torch.equal(outs[t][i][r], dev[i][2]), (t, cases[i], r)
 
 
+def test_scratch_buffer_outlives_a_graph_that_holds_its_address(loader):
+    """A split-K call recorded into a HIP graph bakes the library's scratch buffer into the
+    graph.  A later eager call that needs a larger buffer must not free the old one (the
+    replays would write partial sums into freed memory), and a call recorded while the buffer
+    is too small must neither allocate nor synchronise inside the capture: it runs without
+    scratch memory instead.  Every replay gives the eager result."""
+    import torch
+
+    assert loader.workspace_release() == 0, "run before any other test that captures a graph"
+    M, N, K, lc, la, lb = 64, 8192, 8192, 0, 0, 1
+    A, B = make_inputs(M, N, K, la, lb, O.F16)
+    dA, dB = to_device(A, O.F16), to_device(B, O.F16)
+    want = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+    loader.gemm(want, dA, dB, M, N, K, lc, la, lb)  # eager: allocates the first buffer
+    torch.cuda.synchronize()
+    check_against_oracle(to_host(want, O.F32), A, B, M, N, K, lc, la, lb, O.F16, O.F32)
+    out = torch.zeros_like(want)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        loader.gemm(out, dA, dB, M, N, K, lc, la, lb)
+    assert loader.workspace_release() == 1, "a buffer lent to a capture must be kept"
+
+    # an eager call that needs 512 MiB of partial planes: the buffer is replaced
+    small = next(v.index for v in loader.variants() if v.pipeline == 1 and v.block_m == 128 and v.block_n == 128)
+    M2, N2, K2 = 2048, 2048, 8192
+    A2, B2 = make_inputs(M2, N2, K2, 0, 1, O.F16, seed_b=2)
+    dA2, dB2 = to_device(A2, O.F16), to_device(B2, O.F16)
+    big = torch.full((M2 * N2,), float("nan"), dtype=torch.float32, device="cuda")
+    assert loader.run_variant(small, 8, 32, big, dA2, dB2, M2, N2, K2, 0, 0, 1) == 0
+    torch.cuda.synchronize()
+    check_against_oracle(to_host(big, O.F32), A2, B2, M2, N2, K2, 0, 0, 1, O.F16, O.F32)
+    # memory allocated now lands where a freed buffer would have been
+    filler = [torch.full((64 << 20,), 7, dtype=torch.uint8, device="cuda") for _ in range(6)]
+    for replay in range(3):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), replay
+        assert all(bool((f == 7).all()) for f in filler), "a replay wrote into memory the library had freed"
+        loader.gemm(big, dA2, dB2, M2, N2, K2, 0, 0, 1)  # eager work in between
+        torch.cuda.synchronize()
+
+    # recorded while the buffer is too small for it: no growth inside the capture
+    M3, N3, K3 = 4096, 2048, 8192
+    A3, B3 = make_inputs(M3, N3, K3, 0, 1, O.F16, seed_b=3)
+    dA3, dB3 = to_device(A3, O.F16), to_device(B3, O.F16)
+    out3 = torch.full((M3 * N3,), float("nan"), dtype=torch.float32, device="cuda")
+    graph3 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph3):
+        assert loader.run_variant(small, 8, 28, out3, dA3, dB3, M3, N3, K3, 0, 0, 1) == 0
+    for replay in range(2):
+        out3.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph3.replay()
+        torch.cuda.synchronize()
+        check_against_oracle(to_host(out3, O.F32), A3, B3, M3, N3, K3, 0, 0, 1, O.F16, O.F32)
+
+
 def test_replays_from_a_hip_graph(loader):
     """GEMM calls recorded into a HIP graph (whole tiles on the persistent kernel, a ragged
     shape, and a split-K call whose scratch memory was sized by an eager call before) give
@@ -717,25 +776,46 @@ def test_cpp_client_through_the_references_own_loader_header():
 
 
 # ---------------------------------------------------------------- full-size configurations
-def _full_size_case(loader, M, N, K, lc, la, lb, tname, row_bands, **gen):
+def _full_size_case(loader, M, N, K, lc, la, lb, tname, band_every=128, whole=False, **gen):
+    """One full-size configuration: every element of C through the row/column checksums,
+    and element by element against the oracle either over the whole of C (`whole`, as
+    the reference's tests do, test/gemm/test_float_accum.cpp:118-136) or over one 32-row
+    band in every block of `band_every` rows, so that every tile of C, whatever the
+    kernel's tile size (128, 192 or 256 rows: each holds a whole aligned block of 128) and
+    whichever way round it walks C, has 32 of its rows compared."""
     din, dout = TYPE_PAIRS[tname]
     A, B = make_inputs(M, N, K, la, lb, din, **gen)
     gpu = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout)
-    checksum_check(gpu, A, B, M, N, K, lc, la, lb, din, dout)
-    for r0 in row_bands:
-        check_against_oracle(gpu, A, B, M, N, K, lc, la, lb, din, dout, rows=(r0, min(M, r0 + 32)))
+    sums = checksum_check(gpu, A, B, M, N, K, lc, la, lb, din, dout)
+    if whole:
+        worst, _, _ = check_against_oracle(gpu, A, B, M, N, K, lc, la, lb, din, dout)
+        compared = M * N
+    else:
+        worst, compared = 0.0, 0
+        for block in range(0, M, band_every):
+            # a different place in every block, the last rows of C always among them
+            r0 = min(block + (block // band_every * 96) % max(band_every - 32, 1), max(M - 32, 0))
+            if block + band_every >= M:
+                r0 = max(M - 32, 0)
+            r1 = min(M, r0 + 32)
+            w, _, _ = check_against_oracle(gpu, A, B, M, N, K, lc, la, lb, din, dout, rows=(r0, r1))
+            worst, compared = max(worst, w), compared + (r1 - r0) * N
+    print(f"full-size {tname} {M}x{N}x{K} {layout_id(lc, la, lb)}: {compared} of {M * N} elements "
+          f"compared with the oracle, max |err|/tol = {worst:.3f}; checksums at {sums:.3f} of "
+          f"their tolerance", flush=True)
 
 
 @pytest.mark.parametrize("lc,la,lb", LAYOUTS8, ids=[layout_id(*l) for l in LAYOUTS8])
 def test_half_half_4096_cubed_all_layouts(loader, lc, la, lb):
-    """fp16 -> fp16, M=N=K=4096, uniform[-1,1] seeded: every element through the
-    row/column checksums, three 32-row bands element by element."""
-    _full_size_case(loader, 4096, 4096, 4096, lc, la, lb, "f16_f16", (0, 2048 + 96, 4096 - 32))
+    """fp16 -> fp16, M=N=K=4096, uniform[-1,1] seeded: every element of C against the
+    oracle, and the row/column checksums."""
+    _full_size_case(loader, 4096, 4096, 4096, lc, la, lb, "f16_f16", whole=True)
 
 
 def test_float_bf16_8192_cubed(loader):
-    """bf16 -> fp32, M=N=K=8192, A row / B col / C row, normal(0,1) seeded."""
-    _full_size_case(loader, 8192, 8192, 8192, 0, 0, 1, "f32_bf16", (0, 4096 + 160, 8192 - 32),
+    """bf16 -> fp32, M=N=K=8192, A row / B col / C row, normal(0,1) seeded: every element
+    of C against the oracle."""
+    _full_size_case(loader, 8192, 8192, 8192, 0, 0, 1, "f32_bf16", whole=True,
                     dist="normal", lo=0.0, hi=1.0)
 
 
@@ -743,7 +823,7 @@ def test_float_bf16_8192_cubed(loader):
                                    (16, 8192, 8192), (64, 8192, 8192), (128, 8192, 8192)])
 def test_llm_projection_shapes(loader, M, N, K):
     for (lc, la, lb) in [(0, 0, 1), (1, 0, 0)]:
-        _full_size_case(loader, M, N, K, lc, la, lb, "f32_f16", (0, max(0, M - 32)))
+        _full_size_case(loader, M, N, K, lc, la, lb, "f32_f16", whole=M <= 128)
 
 
 @pytest.mark.parametrize("M,N,K", [(4095, 5121, 3001), (1000, 1000, 1000), (1024, 1024, 65536),
@@ -753,5 +833,5 @@ def test_edge_tile_and_long_k(loader, M, N, K):
     workspace's first allocation, so it also covers the workspace growing."""
     layouts = [(0, 0, 1), (1, 0, 0), (0, 1, 0), (1, 1, 1)] if M < 8000 else [(0, 0, 1), (1, 1, 0)]
     for (lc, la, lb) in layouts:
-        _full_size_case(loader, M, N, K, lc, la, lb, "bf16_bf16", (0, max(0, M - 32)),
+        _full_size_case(loader, M, N, K, lc, la, lb, "bf16_bf16", whole=M <= 1024 and K <= 1024,
                         lo=-0.5, hi=0.5)

@@ -106,6 +106,55 @@ def test_config_selection_order(host_tool):
     assert r.returncode == 0, r.stdout + r.stderr
 
 
+def test_scratch_buffer_rules_under_graph_capture(host_tool):
+    r = subprocess.run([host_tool, "workspace"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+
+
+def test_cmake_consumer_links_through_the_loader_target(tmp_path, built_library):
+    """A consumer project that only does add_subdirectory + target_link_libraries(app
+    rocm_wmma_gemm_loader), as a user of the reference does (reference
+    rocm_wmma_gemm/CMakeLists.txt:96-105): it must get the include path, HIP, libdl and the
+    ROCM_WMMA_GEMM_LIB_DIR definition, and the arch library target must exist when the
+    library is built from CMake."""
+    import shutil
+
+    if shutil.which("cmake") is None or shutil.which("ninja") is None:
+        pytest.skip("cmake / ninja not installed")
+    compiler = "/opt/rocm/bin/amdclang++"  # the public headers use _Float16 / __bf16 (HIP's types)
+    proj = tmp_path / "consumer"
+    proj.mkdir()
+    (proj / "CMakeLists.txt").write_text(
+        "cmake_minimum_required(VERSION 3.16)\n"
+        "project(consumer LANGUAGES CXX)\n"
+        f"add_subdirectory({ROOT} rocm_wmma_gemm)\n"
+        f"add_executable(dropin_check {ROOT}/tests/dropin_check.cpp)\n"
+        "target_link_libraries(dropin_check PRIVATE rocm_wmma_gemm_loader)\n")
+    # prebuilt library: nothing is compiled but the client
+    build = proj / "build"
+    r = subprocess.run(["cmake", "-S", str(proj), "-B", str(build), "-G", "Ninja",
+                        "-DCMAKE_CXX_COMPILER=" + compiler, "-DROCM_WMMA_GEMM_BUILD_LIBRARY=OFF",
+                        "-DROCM_WMMA_GEMM_LIB_DIR=" + os.path.dirname(built_library)],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    r = subprocess.run(["cmake", "--build", str(build)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    exe = build / "dropin_check"
+    assert exe.exists()
+    assert os.path.dirname(built_library).encode() in exe.read_bytes(), "ROCM_WMMA_GEMM_LIB_DIR not injected"
+    # library built from CMake: the per-arch target is there and the loader depends on it
+    build2 = proj / "build2"
+    r = subprocess.run(["cmake", "-S", str(proj), "-B", str(build2), "-G", "Ninja",
+                        "-DCMAKE_CXX_COMPILER=" + compiler], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    r = subprocess.run(["ninja", "-C", str(build2), "-t", "targets", "all"], capture_output=True, text=True)
+    assert "rocm_wmma_gemm_gfx950" in r.stdout and "librocm_wmma_gemm_gfx950.so" in r.stdout, r.stdout
+    r = subprocess.run(["cmake", "-S", str(proj), "-B", str(proj / "build3"), "-G", "Ninja",
+                        "-DCMAKE_CXX_COMPILER=" + compiler, "-DWMMA_GPU_TARGETS=gfx1100"],
+                       capture_output=True, text=True)
+    assert r.returncode != 0 and "gfx950 is the only target" in r.stderr
+
+
 def test_generator_rejects_unknown_variant_and_roundtrips(tmp_path):
     sys.path.insert(0, os.path.join(ROOT, "rocm_wmma_gemm_amd", "config"))
     import generate_config as G

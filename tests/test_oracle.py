@@ -30,13 +30,69 @@ def test_uniform_first_six_match_reference_generator():
     assert np.array_equal(got, want), (got, want)
 
 
-def test_uniform_range_and_affine_map():
+def test_uniform_draws_match_the_standard_librarys_generator(tmp_path):
+    """The reference draws its inputs with libstdc++'s mt19937 and
+    uniform_real_distribution<float> (test/test.hpp:36-38).  tests/golden/
+    record_uniform_draws.cpp is that pair and nothing else; the oracle's generator must give
+    the same floats, bit for bit, for the reference's range, the harness's other range and
+    an asymmetric one, and the fixture's six values are the head of the first."""
+    import subprocess
+
+    src = os.path.join(os.path.dirname(__file__), "golden", "record_uniform_draws.cpp")
+    exe = str(tmp_path / "record_uniform_draws")
+    subprocess.run(["g++", "-O1", "-std=c++17", src, "-o", exe], check=True)
+    for seed, lo, hi, count in [(1, -1.0, 1.0, 100000), (1, -0.5, 0.5, 100000), (7, 0.25, 3.0, 20000)]:
+        r = subprocess.run([exe, str(seed), repr(lo), repr(hi), str(count)], capture_output=True,
+                           text=True, check=True)
+        want = np.array([float.fromhex(t) for t in r.stdout.split()], dtype=np.float32)
+        got = O.uniform_draws(seed, lo, hi, count)
+        assert want.size == count and np.array_equal(got, want), (seed, lo, hi)
+        if (seed, lo, hi) == (1, -1.0, 1.0):
+            assert np.array_equal(want[:6], np.array(GOLD["uniform_seed1_first6"], dtype=np.float32))
+
+
+def test_uniform_range_and_moments():
     u = O.uniform_draws(1, -1.0, 1.0, 100000)
     assert u.min() >= -1.0 and u.max() < 1.0
     assert abs(float(u.mean())) < 0.01 and abs(float(u.var()) - 1.0 / 3.0) < 0.01
-    h = O.uniform_draws(1, -0.5, 0.5, 1000)
-    raw = O.raw_draws(1, 1000).astype(np.float32) / np.float32(4294967296.0)
-    assert np.array_equal(h, raw * np.float32(1.0) + np.float32(-0.5))
+
+
+def test_normal_draws_are_standard_normal():
+    """dist='normal' (Box-Muller; harness-only, the 8192^3 configuration's inputs) is what
+    it says: moments and a Kolmogorov-Smirnov test against the normal distribution on a
+    million values, mean and deviation applied as given, both members of every pair used
+    (an odd count keeps the order), and the storage layout does not change the values."""
+    from scipy import stats
+
+    n = 1 << 20
+    x = O.init_matrix(1024, 1024, O.ROW, O.F32, seed=1, dist="normal", lo=0.0, hi=1.0).astype(np.float64)
+    assert abs(x.mean()) < 5.0 / np.sqrt(n)
+    assert abs(x.var() - 1.0) < 5.0 * np.sqrt(2.0 / n)
+    assert abs(stats.skew(x)) < 5.0 * np.sqrt(6.0 / n)
+    assert abs(stats.kurtosis(x)) < 5.0 * np.sqrt(24.0 / n)
+    assert stats.kstest(x, "norm").pvalue > 1e-3
+    # even and odd members of the pairs are each normal and uncorrelated with each other
+    assert stats.kstest(x[0::2], "norm").pvalue > 1e-3 and stats.kstest(x[1::2], "norm").pvalue > 1e-3
+    assert abs(np.corrcoef(x[0::2], x[1::2])[0, 1]) < 5.0 / np.sqrt(n / 2)
+    assert abs(np.corrcoef(x[:-1], x[1:])[0, 1]) < 5.0 / np.sqrt(n)
+    assert 4.5 < np.abs(x).max() < 6.5  # tails are there, and nothing is infinite
+    # mean and deviation
+    y = O.init_matrix(1024, 1024, O.ROW, O.F32, seed=1, dist="normal", lo=3.0, hi=0.5).astype(np.float64)
+    assert np.allclose(y, 3.0 + 0.5 * x, rtol=0, atol=1e-6)
+    # a different seed gives different values; the same seed the same ones
+    assert not np.array_equal(O.init_matrix(8, 8, O.ROW, O.F32, seed=2, dist="normal", lo=0.0, hi=1.0),
+                              x[:64].astype(np.float32))
+    # draw order is logical (row by row) whatever the storage, as for the uniform inputs
+    r = O.init_matrix(5, 7, O.ROW, O.F32, seed=1, dist="normal", lo=0.0, hi=1.0)
+    c = O.init_matrix(5, 7, O.COL, O.F32, seed=1, dist="normal", lo=0.0, hi=1.0)
+    assert np.array_equal(r.reshape(5, 7), c.reshape(7, 5).T)
+    assert np.array_equal(r, x[:35].astype(np.float32))
+    # narrowing is the oracle's own round-to-nearest-even conversion
+    b = O.init_matrix(5, 7, O.ROW, O.BF16, seed=1, dist="normal", lo=0.0, hi=1.0)
+    import torch
+
+    want = torch.from_numpy(r).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(b, want)
 
 
 def test_f16_conversion_exhaustive_against_numpy():
@@ -230,3 +286,38 @@ def test_fnv1a64_known_vectors():
     # published FNV-1a test vectors
     assert O.fnv1a64(np.frombuffer(b"a", dtype=np.uint8)) == "af63dc4c8601ec8c"
     assert O.fnv1a64(np.frombuffer(b"foobar", dtype=np.uint8)) == "85944171f73967e8"
+
+
+def test_checksums_see_one_wrong_tile():
+    """The row/column checksum check of the GPU tests (tests/gemm_harness.py) on the CPU:
+    the oracle's own result passes, and so does a result from a different summation order;
+    a result with one K tile of 64 missing from one 128 x 128 tile, or with one tile from
+    another problem, fails."""
+    import sys
+
+    sys.path.insert(0, os.path.dirname(__file__))
+    from gemm_harness import checksum_check
+
+    M, N, K = 512, 384, 2048
+    for din, dout in [(O.F16, O.F16), (O.BF16, O.F32)]:
+        A = O.init_matrix(M, K, O.ROW, din, seed=1)
+        B = O.init_matrix(K, N, O.COL, din, seed=2)
+        good = O.gemm(A, B, M, N, K, O.ROW, O.ROW, O.COL, din, dout)
+        assert checksum_check(good, A, B, M, N, K, O.ROW, O.ROW, O.COL, din, dout) < 0.5
+        Af = O.bits_to_f32(A, din).reshape(M, K).astype(np.float64)
+        Bf = O.bits_to_f32(B, din).reshape(N, K).T.astype(np.float64)
+        exact = Af @ Bf
+        def narrow(x):
+            if dout == O.F32:
+                return x.astype(np.float32).ravel()
+            return x.astype(np.float16).view(np.uint16).ravel()
+        other_order = narrow(exact)  # float64 sums, rounded once: another legal result
+        assert checksum_check(other_order, A, B, M, N, K, O.ROW, O.ROW, O.COL, din, dout) < 0.5
+        dropped = exact.copy()
+        dropped[128:256, 256:384] -= Af[128:256, 64:128] @ Bf[64:128, 256:384]
+        with pytest.raises(AssertionError, match="checksum outside tolerance"):
+            checksum_check(narrow(dropped), A, B, M, N, K, O.ROW, O.ROW, O.COL, din, dout)
+        swapped = exact.copy()
+        swapped[0:128, 0:128] = exact[256:384, 128:256]
+        with pytest.raises(AssertionError, match="checksum outside tolerance"):
+            checksum_check(narrow(swapped), A, B, M, N, K, O.ROW, O.ROW, O.COL, din, dout)
