@@ -4,7 +4,8 @@
 //   gemm_bench --type f16_f16 --shapes 4096,4096,4096:8192,8192,8192 --layouts all
 //              [--reps 20] [--warmup 3] [--batch_count 1]
 //              [--variant V --swizzle S --split_k K]   force one compiled variant
-//              [--rocblas]                             also time rocblas_gemm_ex
+//              [--rocblas] [--hipblaslt]               also time rocblas_gemm_ex / hipblasLtMatmul
+//                                                      (through libvendor_gemm.so)
 //              [--data cyclic|random]
 //              [--names]   also print each result under the reference's benchmark name,
 //                          "{A:m_layout::...,B:...,C:...,m:M,n:N,k:K}/manual_time ...", in
@@ -28,8 +29,14 @@
 #include <string>
 #include <vector>
 
-#ifdef WITH_ROCBLAS
-#include <rocblas/rocblas.h>
+#include <vendor_gemm/vendor_gemm.h>
+
+// The type pair a binary times when --type is not given: the Makefile builds this file
+// once per pair under the reference's benchmark names (reference benchmark/gemm/
+// bench_half_half.cpp, bench_float_half.cpp, bench_bf16_bf16.cpp, bench_float_bf16.cpp)
+// and once as gemm_bench.
+#ifndef GEMM_BENCH_DEFAULT_TYPE
+#define GEMM_BENCH_DEFAULT_TYPE "f16_f16"
 #endif
 
 #define CHECK(x)                                                                                   \
@@ -147,11 +154,11 @@ int type_index(const std::string& t)
 
 int main(int argc, char** argv)
 {
-    std::string type = "f16_f16", shapes_arg = "4096,4096,4096", layouts_arg = "rcr",
+    std::string type = GEMM_BENCH_DEFAULT_TYPE, shapes_arg = "4096,4096,4096", layouts_arg = "rcr",
                 data = "random";
     int    reps = 20, warmup = 3, variant = -1, swizzle = 4, split_k = 1;
     size_t batch = 1;
-    bool   with_rocblas = false;
+    bool   with_rocblas = false, with_hipblaslt = false;
     bool   names        = false;
     for(int i = 1; i < argc; ++i)
     {
@@ -186,6 +193,8 @@ int main(int argc, char** argv)
             data = next("--data");
         else if(a == "--rocblas")
             with_rocblas = true;
+        else if(a == "--hipblaslt")
+            with_hipblaslt = true;
         else if(a == "--names")
             names = true;
         else
@@ -224,14 +233,11 @@ int main(int argc, char** argv)
         return 2;
     }
 
-#ifdef WITH_ROCBLAS
-    rocblas_handle blas = nullptr;
-    if(with_rocblas)
-        rocblas_create_handle(&blas);
-#else
-    if(with_rocblas)
-        std::fprintf(stderr, "built without rocBLAS; --rocblas ignored\n");
-#endif
+    if((with_rocblas || with_hipblaslt) && vendor_gemm_init() != 0)
+    {
+        std::fprintf(stderr, "vendor_gemm_init failed\n");
+        return 2;
+    }
 
     hipStream_t stream;
     CHECK(hipStreamCreate(&stream));
@@ -303,50 +309,16 @@ int main(int argc, char** argv)
                             lc ? "col_major" : "row_major", sh.m, sh.n, sh.k, med, med, reps, tf, gib_s);
             }
             std::fflush(stdout);
-#ifdef WITH_ROCBLAS
-            if(with_rocblas && blas)
+            for(int backend = 0; backend < 2; ++backend)
             {
-                // rocBLAS is column-major: C(col) = op(A) op(B); a row-major operand is
-                // the transpose of a column-major one.  A row-major C (M x N) is the
-                // column-major N x M matrix C^T = B^T A^T: same buffers, operands swapped.
-                rocblas_set_stream(blas, stream);
-                const rocblas_datatype in_t = bf16 ? rocblas_datatype_bf16_r : rocblas_datatype_f16_r;
-                const rocblas_datatype out_t
-                    = c_is_32 ? rocblas_datatype_f32_r : in_t;
-                const float alpha = 1.0f, beta = 0.0f;
-                // as a column-major matrix: A is M x K (ld M) if col-major, else K x M (ld K)
-                const rocblas_int lda = la ? sh.m : sh.k, ldb = lb ? sh.k : sh.n;
-                // the matrices of a batch follow one another without gaps
-                const rocblas_stride sa = sh.m * sh.k, sb = sh.k * sh.n, sc = sh.m * sh.n;
+                if(!(backend == VENDOR_GEMM_ROCBLAS ? with_rocblas : with_hipblaslt))
+                    continue;
                 auto blas_call = [&]() {
-                    if(lc == 1)
+                    const int rc = vendor_gemm(backend, tidx, C, A, B, sh.m, sh.n, sh.k, batch, lc, la, lb, &stream);
+                    if(rc != 0)
                     {
-                        const rocblas_operation ta = la ? rocblas_operation_none : rocblas_operation_transpose;
-                        const rocblas_operation tb = lb ? rocblas_operation_none : rocblas_operation_transpose;
-                        if(batch == 1)
-                            rocblas_gemm_ex(blas, ta, tb, sh.m, sh.n, sh.k, &alpha, A, in_t, lda, B,
-                                            in_t, ldb, &beta, C, out_t, sh.m, C, out_t, sh.m,
-                                            rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
-                        else
-                            rocblas_gemm_strided_batched_ex(
-                                blas, ta, tb, sh.m, sh.n, sh.k, &alpha, A, in_t, lda, sa, B, in_t, ldb,
-                                sb, &beta, C, out_t, sh.m, sc, C, out_t, sh.m, sc, (rocblas_int)batch,
-                                rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
-                    }
-                    else
-                    {
-                        // C^T (N x M, ld N) = op(B) op(A) with op(B) = B^T (N x K), op(A) = A^T (K x M)
-                        const rocblas_operation tb = lb ? rocblas_operation_transpose : rocblas_operation_none;
-                        const rocblas_operation ta = la ? rocblas_operation_transpose : rocblas_operation_none;
-                        if(batch == 1)
-                            rocblas_gemm_ex(blas, tb, ta, sh.n, sh.m, sh.k, &alpha, B, in_t, ldb, A,
-                                            in_t, lda, &beta, C, out_t, sh.n, C, out_t, sh.n,
-                                            rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
-                        else
-                            rocblas_gemm_strided_batched_ex(
-                                blas, tb, ta, sh.n, sh.m, sh.k, &alpha, B, in_t, ldb, sb, A, in_t, lda,
-                                sa, &beta, C, out_t, sh.n, sc, C, out_t, sh.n, sc, (rocblas_int)batch,
-                                rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+                        std::fprintf(stderr, "vendor_gemm failed: %d\n", rc);
+                        std::exit(3);
                     }
                 };
                 for(int w = 0; w < warmup; ++w)
@@ -362,11 +334,11 @@ int main(int argc, char** argv)
                 }
                 std::sort(ms.begin(), ms.end());
                 const double btf = 2.0 * sh.m * sh.n * sh.k * batch / (ms[reps / 2] * 1e-3) / 1e12;
-                std::printf("%-10s %-22s %-4s %8s %6s %10.4f %10.4f %8.1f %7.1f%%\n", "rocblas", dims,
-                            lay.c_str(), "-", "-", ms[reps / 2], ms[0], btf, 100.0 * btf / peak_tf);
+                std::printf("%-10s %-22s %-4s %8s %6s %10.4f %10.4f %8.1f %7.1f%%\n",
+                            backend == VENDOR_GEMM_ROCBLAS ? "rocblas" : "hipblaslt", dims, lay.c_str(), "-", "-",
+                            ms[reps / 2], ms[0], btf, 100.0 * btf / peak_tf);
                 std::fflush(stdout);
             }
-#endif
         }
         CHECK(hipFree(A));
         CHECK(hipFree(B));

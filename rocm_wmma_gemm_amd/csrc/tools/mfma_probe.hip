@@ -248,286 +248,6 @@ __global__ void __launch_bounds__(256) read_kernel(unsigned* __restrict__ out, c
     out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = acc.x ^ acc.y ^ acc.z ^ acc.w;
 }
 
-// ---- 6. LDS read throughput under a given per-lane address pattern ------------
-// Every lane issues `iters` x 8 reads at its own fixed byte address (plus a per-read
-// immediate offset); the time against the linear pattern shows bank conflicts.
-template<bool TR>
-__global__ void __launch_bounds__(512) lds_pattern(const int* lane_addr, float* out, int iters)
-{
-    __shared__ u32x4 lds[4096]; // 64 KiB
-    for(int i = threadIdx.x; i < 4096; i += blockDim.x)
-    {
-        lds[i] = u32x4{1u, 2u, 3u, 4u};
-    }
-    __syncthreads();
-    const unsigned addr = (unsigned)lane_addr[threadIdx.x & 63]
-                          + (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
-    u32x4 acc = {0u, 0u, 0u, 0u};
-    for(int it = 0; it < iters; ++it)
-    {
-        if constexpr(TR)
-        {
-            uint2 v[16];
-            asm volatile(
-                "ds_read_b64_tr_b16 %0, %16\n ds_read_b64_tr_b16 %1, %16 offset:4096\n"
-                "ds_read_b64_tr_b16 %2, %16 offset:8192\n ds_read_b64_tr_b16 %3, %16 offset:12288\n"
-                "ds_read_b64_tr_b16 %4, %16 offset:16384\n ds_read_b64_tr_b16 %5, %16 offset:20480\n"
-                "ds_read_b64_tr_b16 %6, %16 offset:24576\n ds_read_b64_tr_b16 %7, %16 offset:28672\n"
-                "ds_read_b64_tr_b16 %8, %16 offset:32768\n ds_read_b64_tr_b16 %9, %16 offset:36864\n"
-                "ds_read_b64_tr_b16 %10, %16 offset:40960\n ds_read_b64_tr_b16 %11, %16 offset:45056\n"
-                "ds_read_b64_tr_b16 %12, %16 offset:49152\n ds_read_b64_tr_b16 %13, %16 offset:53248\n"
-                "ds_read_b64_tr_b16 %14, %16 offset:57344\n ds_read_b64_tr_b16 %15, %16 offset:61440\n"
-                "s_waitcnt lgkmcnt(0)"
-                : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]),
-                  "=&v"(v[6]), "=&v"(v[7]), "=&v"(v[8]), "=&v"(v[9]), "=&v"(v[10]), "=&v"(v[11]),
-                  "=&v"(v[12]), "=&v"(v[13]), "=&v"(v[14]), "=&v"(v[15])
-                : "v"(addr));
-            for(int i = 0; i < 16; ++i)
-                acc.x ^= v[i].x ^ v[i].y;
-        }
-        else
-        {
-            u32x4 v[16];
-            asm volatile(
-                "ds_read_b128 %0, %16\n ds_read_b128 %1, %16 offset:4096\n"
-                "ds_read_b128 %2, %16 offset:8192\n ds_read_b128 %3, %16 offset:12288\n"
-                "ds_read_b128 %4, %16 offset:16384\n ds_read_b128 %5, %16 offset:20480\n"
-                "ds_read_b128 %6, %16 offset:24576\n ds_read_b128 %7, %16 offset:28672\n"
-                "ds_read_b128 %8, %16 offset:32768\n ds_read_b128 %9, %16 offset:36864\n"
-                "ds_read_b128 %10, %16 offset:40960\n ds_read_b128 %11, %16 offset:45056\n"
-                "ds_read_b128 %12, %16 offset:49152\n ds_read_b128 %13, %16 offset:53248\n"
-                "ds_read_b128 %14, %16 offset:57344\n ds_read_b128 %15, %16 offset:61440\n"
-                "s_waitcnt lgkmcnt(0)"
-                : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]),
-                  "=&v"(v[6]), "=&v"(v[7]), "=&v"(v[8]), "=&v"(v[9]), "=&v"(v[10]), "=&v"(v[11]),
-                  "=&v"(v[12]), "=&v"(v[13]), "=&v"(v[14]), "=&v"(v[15])
-                : "v"(addr));
-            for(int i = 0; i < 16; ++i)
-                acc.x ^= v[i].x ^ v[i].w;
-        }
-    }
-    if(acc.x == 0x12345678u)
-    {
-        out[0] = 1.0f;
-    }
-}
-
-
-// ---- 7. LDS reads and global->LDS loads side by side ----------------------------
-// MODE 0: 16 ds_read_b128 per step; MODE 1: 4 global_load_lds_dwordx4 per step (from
-// a window of global memory small enough to stay in L2); MODE 2: both.  Shows what
-// the LDS sustains when the MFMA operand reads and the tile loads share it.
-template<int MODE, int DMA_BYTES>
-__global__ void __launch_bounds__(512) lds_dma_mix(const char* src, float* out, int iters)
-{
-    __shared__ __attribute__((aligned(1024))) char lds[131072];
-    for(int i = threadIdx.x; i < 131072 / 16; i += blockDim.x)
-    {
-        ((u32x4*)lds)[i] = u32x4{1u, 2u, 3u, 4u};
-    }
-    __syncthreads();
-    const int      lane  = threadIdx.x & 63;
-    const int      wave  = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const unsigned raddr = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds
-                           + (unsigned)(((lane % 32) * 128 + (((lane / 32) ^ ((lane >> 1) & 7)) * 16)));
-    // each workgroup walks its own 64 KiB window; each wave its own 1 KiB stripes
-    const char* base = src + (size_t)(blockIdx.x % 64) * 65536 + lane * DMA_BYTES;
-    u32x4 acc = {0u, 0u, 0u, 0u};
-    for(int it = 0; it < iters; ++it)
-    {
-        if constexpr(MODE != 0)
-        {
-#pragma unroll
-            for(int q = 0; q < 4; ++q)
-            {
-                const int stripe = ((it * 4 + q) * 8 + wave) & 63;
-                auto* g = (const __attribute__((address_space(1))) void*)(base + stripe * (64 * DMA_BYTES));
-                auto* l = (__attribute__((address_space(3))) void*)(lds + 65536 + stripe * 1024);
-                if constexpr(DMA_BYTES == 16)
-                    __builtin_amdgcn_global_load_lds(g, l, 16, 0, 0);
-                else
-                    __builtin_amdgcn_global_load_lds(g, l, 4, 0, 0);
-            }
-        }
-        if constexpr(MODE != 1)
-        {
-            u32x4 v[16];
-            asm volatile(
-                "ds_read_b128 %0, %16\n ds_read_b128 %1, %16 offset:4096\n"
-                "ds_read_b128 %2, %16 offset:8192\n ds_read_b128 %3, %16 offset:12288\n"
-                "ds_read_b128 %4, %16 offset:16384\n ds_read_b128 %5, %16 offset:20480\n"
-                "ds_read_b128 %6, %16 offset:24576\n ds_read_b128 %7, %16 offset:28672\n"
-                "ds_read_b128 %8, %16 offset:32768\n ds_read_b128 %9, %16 offset:36864\n"
-                "ds_read_b128 %10, %16 offset:40960\n ds_read_b128 %11, %16 offset:45056\n"
-                "ds_read_b128 %12, %16 offset:49152\n ds_read_b128 %13, %16 offset:53248\n"
-                "ds_read_b128 %14, %16 offset:57344\n ds_read_b128 %15, %16 offset:61440\n"
-                "s_waitcnt lgkmcnt(0)"
-                : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]),
-                  "=&v"(v[6]), "=&v"(v[7]), "=&v"(v[8]), "=&v"(v[9]), "=&v"(v[10]), "=&v"(v[11]),
-                  "=&v"(v[12]), "=&v"(v[13]), "=&v"(v[14]), "=&v"(v[15])
-                : "v"(raddr));
-            for(int i = 0; i < 16; ++i)
-                acc.x ^= v[i].x ^ v[i].w;
-        }
-        if constexpr(MODE != 0)
-        {
-            __builtin_amdgcn_s_waitcnt(0x0070 | 4 | (0 << 8)); // vmcnt(4): one step in flight
-        }
-    }
-    __builtin_amdgcn_s_waitcnt(0);
-    if(acc.x == 0x12345678u)
-    {
-        out[0] = 1.0f;
-    }
-}
-
-
-// ---- 8. MFMA throughput with a memory stream running beside it ---------------------
-// Each wave runs 16 independent MFMAs per step on pseudo-random operands and, beside
-// them, LOADS memory operations of one kind:
-//   KIND 0 none, 1 global_load_lds_dwordx4 (L2-resident source), 2 global_load_dwordx4
-//   into VGPRs, 3 ds_read_b128, 4 global_load_lds from a large (HBM-resident) source
-template<int KIND, int LOADS>
-__global__ void __launch_bounds__(256) mfma_with_stream(const char* src, size_t src_bytes, float* out, int iters)
-{
-    __shared__ __attribute__((aligned(1024))) char lds[65536];
-    for(int i = threadIdx.x; i < 65536 / 16; i += blockDim.x)
-        ((u32x4*)lds)[i] = u32x4{(unsigned)i * 2654435761u, 0x3c003c00u ^ (unsigned)i, 0xbc00u * (unsigned)i, 0x12345u * (unsigned)i};
-    __syncthreads();
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    f32x16    acc[16];
-    for(int c = 0; c < 16; ++c)
-        for(int v = 0; v < 16; ++v)
-            acc[c][v] = 0.0f;
-    u32x4 fa[4], fb[4];
-    for(int i = 0; i < 4; ++i)
-    {
-        fa[i] = ((u32x4*)lds)[(lane * 4 + i) & 4095];
-        fb[i] = ((u32x4*)lds)[(lane * 4 + i + 1024) & 4095];
-    }
-    const unsigned long long clk0 = __builtin_amdgcn_s_memtime();
-    const unsigned long long rt0  = __builtin_amdgcn_s_memrealtime();
-    const size_t window = KIND == 4 ? src_bytes : (size_t)(4 << 20);
-    size_t       pos    = ((size_t)blockIdx.x * 65536 + (size_t)wave * 16384) % window;
-    u32x4        sink   = {0u, 0u, 0u, 0u};
-    const unsigned raddr = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds + lane * 16;
-    for(int it = 0; it < iters; ++it)
-    {
-#pragma unroll
-        for(int q = 0; q < LOADS; ++q)
-        {
-            const char* g = src + pos + q * 1024 + lane * 16;
-            if constexpr(KIND == 6)
-            {
-                // buffer form: 128-bit resource in SGPRs, 32-bit per-lane offset, scalar offset
-                auto rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, 0x7fffffff, 0x00020000);
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc,
-                                                         (__attribute__((address_space(3))) void*)(lds + 32768 + ((wave * LOADS + q) & 31) * 1024),
-                                                         16, lane * 16, (int)(pos + q * 1024), 0, 0);
-            }
-            else if constexpr(KIND == 5)
-            {
-                // uniform 64-bit base in SGPRs + 32-bit per-lane byte offset
-                const char* ubase = src + pos + q * 1024;
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ubase + (unsigned)(lane * 16)),
-                                                 (__attribute__((address_space(3))) void*)(lds + 32768 + ((wave * LOADS + q) & 31) * 1024),
-                                                 16, 0, 0);
-            }
-            else if constexpr(KIND == 1 || KIND == 4)
-            {
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
-                                                 (__attribute__((address_space(3))) void*)(lds + 32768 + ((wave * LOADS + q) & 31) * 1024),
-                                                 16, 0, 0);
-            }
-            else if constexpr(KIND == 2)
-            {
-                u32x4 v = __builtin_nontemporal_load((const u32x4*)g);
-                sink ^= v;
-            }
-            else if constexpr(KIND == 3)
-            {
-                u32x4 v;
-                asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(raddr + q * 1024));
-                sink ^= v;
-            }
-        }
-        pos = (pos + 256 * 1024) % window;
-#pragma unroll
-        for(int c = 0; c < 16; ++c)
-            acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fa[c / 4]), __builtin_bit_cast(f16x8, fb[c % 4]), acc[c], 0, 0, 0);
-        if constexpr(KIND == 1 || KIND == 4 || KIND == 5 || KIND == 6)
-            __builtin_amdgcn_s_waitcnt(0x0070 | (3 * LOADS > 15 ? 15 : 3 * LOADS)); // keep ~3 steps in flight
-    }
-    __builtin_amdgcn_s_waitcnt(0);
-    float s = 0.0f;
-    for(int c = 0; c < 16; ++c)
-        for(int v = 0; v < 16; ++v)
-            s += acc[c][v];
-    if(s == 12345.678f || sink.x == 0x7654321u)
-        out[0] = s;
-    if(blockIdx.x == 0 && threadIdx.x == 0)
-    {
-        // shader-clock ticks and constant 100 MHz ticks over the loop -> average core clock
-        out[1] = (float)(__builtin_amdgcn_s_memtime() - clk0);
-        out[2] = (float)(__builtin_amdgcn_s_memrealtime() - rt0);
-    }
-}
-
-
-// ---- 6b. ds_read_b128 with only some lanes active (address < 0 = lane sits out) -----
-template<bool B64>
-__global__ void __launch_bounds__(512) lds_pattern_masked(const int* lane_addr, float* out, int iters)
-{
-    __shared__ u32x4 lds[4096]; // 64 KiB
-    for(int i = threadIdx.x; i < 4096; i += blockDim.x)
-    {
-        lds[i] = u32x4{1u, 2u, 3u, 4u};
-    }
-    __syncthreads();
-    const int      la   = lane_addr[threadIdx.x & 63];
-    const unsigned addr = (unsigned)la + (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
-    u32x4 acc = {0u, 0u, 0u, 0u};
-    if(la >= 0)
-    {
-        for(int it = 0; it < iters; ++it)
-        {
-            u32x4 v[8];
-            if constexpr(B64)
-            {
-                uint2 w[8];
-                asm volatile(
-                    "ds_read_b64_tr_b16 %0, %8\n ds_read_b64_tr_b16 %1, %8 offset:4096\n"
-                    "ds_read_b64_tr_b16 %2, %8 offset:8192\n ds_read_b64_tr_b16 %3, %8 offset:12288\n"
-                    "ds_read_b64_tr_b16 %4, %8 offset:16384\n ds_read_b64_tr_b16 %5, %8 offset:20480\n"
-                    "ds_read_b64_tr_b16 %6, %8 offset:24576\n ds_read_b64_tr_b16 %7, %8 offset:28672\n"
-                    "s_waitcnt lgkmcnt(0)"
-                    : "=&v"(w[0]), "=&v"(w[1]), "=&v"(w[2]), "=&v"(w[3]), "=&v"(w[4]), "=&v"(w[5]),
-                      "=&v"(w[6]), "=&v"(w[7])
-                    : "v"(addr));
-                for(int i = 0; i < 8; ++i)
-                    v[i] = u32x4{w[i].x, w[i].y, 0u, 0u};
-            }
-            else
-            {
-                asm volatile(
-                    "ds_read_b128 %0, %8\n ds_read_b128 %1, %8 offset:4096\n"
-                    "ds_read_b128 %2, %8 offset:8192\n ds_read_b128 %3, %8 offset:12288\n"
-                    "ds_read_b128 %4, %8 offset:16384\n ds_read_b128 %5, %8 offset:20480\n"
-                    "ds_read_b128 %6, %8 offset:24576\n ds_read_b128 %7, %8 offset:28672\n"
-                    "s_waitcnt lgkmcnt(0)"
-                    : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]),
-                      "=&v"(v[6]), "=&v"(v[7])
-                    : "v"(addr));
-            }
-            for(int i = 0; i < 8; ++i)
-                acc ^= v[i];
-        }
-    }
-    if(acc.x == 0x12345u)
-        out[0] = 1.0f;
-}
-
 // ---- 9. MFMA shape vs sustained rate on pseudo-random operands ----------------------
 // SHAPE 0: v_mfma_f32_32x32x16_f16 (16 accumulator registers per instruction),
 // SHAPE 1: v_mfma_f32_16x16x32_f16 (4 accumulator registers per instruction).
@@ -655,7 +375,6 @@ int main(int argc, char** argv)
 {
     bool   dump     = false;
     bool   ceiling  = false;
-    bool   lds_groups = false;
     size_t copy_mib = 0, read_mib = 0;
     bool   range_check = false;
     for(int i = 1; i < argc; ++i)
@@ -664,8 +383,6 @@ int main(int argc, char** argv)
             dump = true;
         if(!std::strcmp(argv[i], "--ceiling"))
             ceiling = true;
-        if(!std::strcmp(argv[i], "--lds-groups"))
-            lds_groups = true;
         if(!std::strcmp(argv[i], "--copy") && i + 1 < argc)
             copy_mib = std::strtoull(argv[++i], nullptr, 10);
         if(!std::strcmp(argv[i], "--range"))
@@ -713,136 +430,6 @@ int main(int argc, char** argv)
         };
         run("ceiling", mfma_shape_rate<1>);
         run("ceiling_32x32x16", mfma_shape_rate<0>);
-        return 0;
-    }
-
-    if(lds_groups)
-    {
-        // Which lanes of a ds_read_b128 are served in the same LDS cycle, and which
-        // address bits pick the bank: start from the conflict-free pattern lane*16 and
-        // move ONE lane j onto another row of lane 0's 16-byte column (experiment 1), or
-        // move lane 1 to byte offset X of another row (experiment 2); a slower run means
-        // the two lanes met in one cycle on one bank.
-        int*   dAddr;
-        float* dOut;
-        CHECK(hipMalloc(&dAddr, 256));
-        CHECK(hipMalloc(&dOut, 4));
-        const int iters = 3000, blocks = prop.multiProcessorCount;
-        auto run = [&](const std::vector<int>& addr) {
-            CHECK(hipMemcpy(dAddr, addr.data(), 256, hipMemcpyHostToDevice));
-            lds_pattern<false><<<blocks, 512>>>(dAddr, dOut, 100);
-            CHECK(hipDeviceSynchronize());
-            CHECK(hipEventRecord(e0));
-            lds_pattern<false><<<blocks, 512>>>(dAddr, dOut, iters);
-            CHECK(hipEventRecord(e1));
-            CHECK(hipEventSynchronize(e1));
-            return time_ms(e0, e1);
-        };
-        auto run_masked = [&](const std::vector<int>& addr) {
-            CHECK(hipMemcpy(dAddr, addr.data(), 256, hipMemcpyHostToDevice));
-            lds_pattern_masked<false><<<blocks, 512>>>(dAddr, dOut, 100);
-            CHECK(hipDeviceSynchronize());
-            CHECK(hipEventRecord(e0));
-            lds_pattern_masked<false><<<blocks, 512>>>(dAddr, dOut, iters);
-            CHECK(hipEventRecord(e1));
-            CHECK(hipEventSynchronize(e1));
-            return time_ms(e0, e1);
-        };
-        (void)run;
-        // Experiment 1: lanes i and j alone, same 16-byte bank column, different rows.
-        for(int i : {0, 8, 16, 32})
-        {
-            std::vector<int> one(64, -1);
-            one[i]         = 0;
-            const float t1 = run_masked(one);
-            std::printf("lanes %d and j active on one bank column (time relative to lane %d alone, %.3f ms):\n", i, i, t1);
-            for(int j = 0; j < 64; ++j)
-            {
-                if(j == i)
-                {
-                    std::printf("  --:----%s", j % 8 == 7 ? "\n" : "");
-                    continue;
-                }
-                std::vector<int> a(64, -1);
-                a[i] = 0;
-                a[j] = 2048;
-                std::printf("  %2d:%.2f%s", j, run_masked(a) / t1, j % 8 == 7 ? "\n" : "");
-            }
-        }
-        // Experiment 2: lanes 0 and 1 alone; lane 0 at byte 0, lane 1 at byte X.
-        {
-            std::vector<int> one(64, -1);
-            one[0]         = 0;
-            const float t1 = run_masked(one);
-            std::printf("lane 0 at byte 0, lane 1 at byte X (relative time):\n");
-            int n = 0;
-            for(int x : {16, 32, 64, 128, 256, 512, 1024, 2048, 4096, 8192, 256 + 16, 512 + 16, 1024 + 16, 2048 + 16, 4096 + 16, 128 + 256, 128 + 512, 64 + 1024})
-            {
-                std::vector<int> a(64, -1);
-                a[0] = 0;
-                a[1] = x;
-                std::printf("  %5d:%.2f%s", x, run_masked(a) / t1, ++n % 6 == 0 ? "\n" : "");
-            }
-            std::printf("\n");
-        }
-        // Experiment 1b/2b: the same for ds_read_b64_tr_b16 (8 bytes per lane)
-        auto run_masked64 = [&](const std::vector<int>& addr) {
-            CHECK(hipMemcpy(dAddr, addr.data(), 256, hipMemcpyHostToDevice));
-            lds_pattern_masked<true><<<blocks, 512>>>(dAddr, dOut, 100);
-            CHECK(hipDeviceSynchronize());
-            CHECK(hipEventRecord(e0));
-            lds_pattern_masked<true><<<blocks, 512>>>(dAddr, dOut, iters);
-            CHECK(hipEventRecord(e1));
-            CHECK(hipEventSynchronize(e1));
-            return time_ms(e0, e1);
-        };
-        for(int i : {0, 16, 32})
-        {
-            std::vector<int> one(64, -1);
-            one[i]         = 0;
-            const float t1 = run_masked64(one);
-            std::printf("b64_tr: lanes %d and j active on one 8-byte bank column (relative to lane %d alone, %.3f ms):\n", i, i, t1);
-            for(int j = 0; j < 64; ++j)
-            {
-                if(j == i)
-                {
-                    std::printf("  --:----%s", j % 8 == 7 ? "\n" : "");
-                    continue;
-                }
-                std::vector<int> a(64, -1);
-                a[i] = 0;
-                a[j] = 2048;
-                std::printf("  %2d:%.2f%s", j, run_masked64(a) / t1, j % 8 == 7 ? "\n" : "");
-            }
-        }
-        {
-            std::vector<int> one(64, -1);
-            one[0]         = 0;
-            const float t1 = run_masked64(one);
-            std::printf("b64_tr: lane 0 at byte 0, lane 1 at byte X (relative time):\n");
-            int n = 0;
-            for(int x : {8, 16, 32, 64, 128, 256, 512, 1024, 2048, 4096, 256 + 8, 512 + 8, 2048 + 8, 128 + 256})
-            {
-                std::vector<int> a(64, -1);
-                a[0] = 0;
-                a[1] = x;
-                std::printf("  %5d:%.2f%s", x, run_masked64(a) / t1, ++n % 7 == 0 ? "\n" : "");
-            }
-            std::printf("\n");
-        }
-        // Experiment 3: how many lanes of a 16-lane block can run before time goes up
-        {
-            std::printf("lanes 0..n-1 active at lane*16 (ms):");
-            for(int n : {1, 2, 4, 8, 16, 24, 32, 48, 64})
-            {
-                std::vector<int> a(64, -1);
-                for(int l = 0; l < n; ++l)
-                    a[l] = l * 16;
-                std::printf("  %d:%.3f", n, run_masked(a));
-            }
-            std::printf("\n");
-        }
-        std::printf("\n");
         return 0;
     }
 
@@ -1048,118 +635,6 @@ int main(int argc, char** argv)
             std::printf("mfma ceiling, %d waves/CU: %.1f TFLOP/s  (=> %.0f MHz at 1024 FLOP/clk/SIMD)\n", 4 * wg_per_cu, tf,
                         tf * 1e12 / (prop.multiProcessorCount * 4.0 * 1024.0) / 1e6);
         }
-    }
-
-
-    // LDS read patterns (4 waves per CU, all CUs)
-    {
-        struct pat { const char* name; bool tr; int (*f)(int); };
-        static const pat pats[] = {
-            {"b128 linear lane*16", false, [](int l) { return l * 16; }},
-            {"b128 row*128, chunk=hi (no swizzle)", false, [](int l) { return (l % 32) * 128 + (l / 32) * 16; }},
-            {"b128 slot = c ^ (r&7)", false, [](int l) { int r = l % 32, c = l / 32; return r * 128 + ((c ^ (r & 7)) * 16); }},
-            {"b128 slot = c ^ ((r>>1)&7)", false, [](int l) { int r = l % 32, c = l / 32; return r * 128 + ((c ^ ((r >> 1) & 7)) * 16); }},
-            {"b128 slot = c ^ (r&7) ^ ((r>>3)&1)", false, [](int l) { int r = l % 32, c = l / 32; return r * 128 + ((c ^ (r & 7) ^ ((r >> 3) & 1)) * 16); }},
-            {"b128 row*64 (BK=32), slot = c ^ ((r>>1)&3)", false, [](int l) { int r = l % 32, c = l / 32; return r * 64 + ((c ^ ((r >> 1) & 3)) * 16); }},
-            {"b128 16x16x32: row*128, slot = g ^ ((r>>1)&7)", false, [](int l) { int r = l % 16, g = l / 16; return r * 128 + ((g ^ ((r >> 1) & 7)) * 16); }},
-            {"b128 16x16x32: row*64, slot = g ^ ((r>>2)&3)", false, [](int l) { int r = l % 16, g = l / 16; return r * 64 + ((g ^ ((r >> 2) & 3)) * 16); }},
-            {"b128 16 lanes linear, groups 4096 B apart", false, [](int l) { return (l % 16) * 16 + (l / 16) * 4096; }},
-            {"b128 16 lanes linear, groups 256 B apart", false, [](int l) { return (l % 16) * 16 + (l / 16) * 256; }},
-            {"b128 16x16x32: row*128, slot = (g + 4*(r&1)) ^ (r>>1)", false, [](int l) { int r = l % 16, g = l / 16; return r * 128 + (((g + 4 * (r & 1)) ^ ((r >> 1) & 7)) * 16); }},
-            {"b128 16x16x32: row*128, slot = (2g) ^ (r>>1), +16B odd g", false, [](int l) { int r = l % 16, g = l / 16; return r * 128 + (((2 * (g & 1) + (g >> 1)) ^ ((r >> 1) & 7)) * 16); }},
-            {"tr64 linear lane*8", true, [](int l) { return l * 8; }},
-            {"tr64 [k][m] rows of 512 B, no swizzle", true, [](int l) { int b = l / 16, s = l % 16; return (8 * (b / 2) + s / 4) * 512 + (16 * (b % 2) + (s % 4) * 4) * 2; }},
-            {"tr64 4k x 128m blocks, chunk ^ 4j", true, [](int l) { int b = l / 16, s = l % 16, j = s / 4; int mm = 16 * (b % 2) + (s % 4) * 4; int c = mm / 8; return (2 * (b / 2)) * 2048 + (j * 16 + (c ^ (4 * j))) * 16 + (mm % 8) * 2; }},
-            {"tr64 4k x 128m blocks, no swizzle", true, [](int l) { int b = l / 16, s = l % 16, j = s / 4; int mm = 16 * (b % 2) + (s % 4) * 4; int c = mm / 8; return (2 * (b / 2)) * 2048 + (j * 16 + c) * 16 + (mm % 8) * 2; }},
-        };
-        int*   dAddr;
-        float* dOut;
-        CHECK(hipMalloc(&dAddr, 256));
-        CHECK(hipMalloc(&dOut, 4));
-        const int iters = 5000;
-        for(const pat& p : pats)
-        {
-            std::vector<int> addr(64);
-            for(int l = 0; l < 64; ++l)
-                addr[l] = p.f(l);
-            CHECK(hipMemcpy(dAddr, addr.data(), 256, hipMemcpyHostToDevice));
-            const int blocks = prop.multiProcessorCount;
-            for(int threads = 256; threads <= 512; threads *= 2)
-            {
-                if(p.tr) lds_pattern<true><<<blocks, threads>>>(dAddr, dOut, 100); else lds_pattern<false><<<blocks, threads>>>(dAddr, dOut, 100);
-                CHECK(hipDeviceSynchronize());
-                CHECK(hipEventRecord(e0));
-                if(p.tr) lds_pattern<true><<<blocks, threads>>>(dAddr, dOut, iters); else lds_pattern<false><<<blocks, threads>>>(dAddr, dOut, iters);
-                CHECK(hipEventRecord(e1));
-                CHECK(hipEventSynchronize(e1));
-                const float  ms    = time_ms(e0, e1);
-                const double bytes = (double)iters * 16 * threads * (p.tr ? 8 : 16); // per CU
-                std::printf("lds %-46s %d waves/CU %8.3f ms  %7.1f B/ns/CU\n", p.name, threads / 64, ms, bytes / (ms * 1e6));
-            }
-        }
-    }
-
-
-    // LDS reads vs global->LDS loads (8 waves per CU, all CUs, source resident in L2)
-    {
-        char*  dSrc;
-        float* dOut;
-        CHECK(hipMalloc(&dSrc, 64 * 65536 + 65536));
-        CHECK(hipMemset(dSrc, 1, 64 * 65536 + 65536));
-        CHECK(hipMalloc(&dOut, 4));
-        const int iters = 4000, blocks = prop.multiProcessorCount;
-        auto run = [&](const char* name, auto kernel, double rd_bytes, double dma_bytes) {
-            kernel<<<blocks, 512>>>(dSrc, dOut, 50);
-            CHECK(hipDeviceSynchronize());
-            CHECK(hipEventRecord(e0));
-            kernel<<<blocks, 512>>>(dSrc, dOut, iters);
-            CHECK(hipEventRecord(e1));
-            CHECK(hipEventSynchronize(e1));
-            const float ms = time_ms(e0, e1);
-            std::printf("mix %-34s %8.3f ms  reads %7.1f B/ns/CU  loads %7.1f B/ns/CU\n", name, ms,
-                        rd_bytes * iters / (ms * 1e6), dma_bytes * iters / (ms * 1e6));
-        };
-        run("ds_read_b128 only", lds_dma_mix<0, 16>, 8.0 * 16 * 1024, 0.0);
-        run("global_load_lds_dwordx4 only", lds_dma_mix<1, 16>, 0.0, 8.0 * 4 * 1024);
-        run("both (dwordx4)", lds_dma_mix<2, 16>, 8.0 * 16 * 1024, 8.0 * 4 * 1024);
-        run("global_load_lds_dword only", lds_dma_mix<1, 4>, 0.0, 8.0 * 4 * 256);
-        run("both (dword)", lds_dma_mix<2, 4>, 8.0 * 16 * 1024, 8.0 * 4 * 256);
-    }
-
-
-    // MFMA beside a memory stream (4 waves per CU, all CUs)
-    {
-        const size_t big = size_t{1} << 30;
-        char*        dSrc;
-        float*       dOut;
-        CHECK(hipMalloc(&dSrc, big + (1 << 20)));
-        CHECK(hipMemset(dSrc, 0x3c, big + (1 << 20)));
-        CHECK(hipMalloc(&dOut, 16));
-        const int iters = 4000, blocks = prop.multiProcessorCount;
-        auto run = [&](const char* name, auto kernel, int loads) {
-            kernel<<<blocks, 256>>>(dSrc, big, dOut, 50);
-            CHECK(hipDeviceSynchronize());
-            CHECK(hipEventRecord(e0));
-            kernel<<<blocks, 256>>>(dSrc, big, dOut, iters);
-            CHECK(hipEventRecord(e1));
-            CHECK(hipEventSynchronize(e1));
-            const float  ms = time_ms(e0, e1);
-            const double tf = 2.0 * 32 * 32 * 16 * 16 * (double)iters * 4 * blocks / (ms * 1e-3) / 1e12;
-            float clk[3];
-            CHECK(hipMemcpy(clk, dOut, 12, hipMemcpyDeviceToHost));
-            const double mhz = clk[2] > 0 ? clk[1] / clk[2] * 100.0 : 0.0;
-            std::printf("mfma+%-44s %8.3f ms %8.1f TFLOP/s  stream %6.1f B/ns/CU  core clock %5.0f MHz  MFMA busy %4.1f %%\n", name, ms, tf,
-                        loads * 1024.0 * 4 * iters / (ms * 1e6), mhz,
-                        mhz > 0 ? 100.0 * tf * 1e12 / (prop.multiProcessorCount * 4.0 * 1024.0 * mhz * 1e6) : 0.0);
-        };
-        run("nothing (random operands)", mfma_with_stream<0, 0>, 0);
-        run("global_load_lds x4 per 16 MFMA, L2-resident", mfma_with_stream<1, 4>, 4);
-        run("global_load_lds x2 per 16 MFMA, L2-resident", mfma_with_stream<1, 2>, 2);
-        run("global_load_lds x4, SGPR base + 32-bit offset", mfma_with_stream<5, 4>, 4);
-        run("buffer_load ... lds x4 (32-bit voffset + soffset)", mfma_with_stream<6, 4>, 4);
-        run("global_load_lds x4 per 16 MFMA, 1 GiB source", mfma_with_stream<4, 4>, 4);
-        run("global_load_dwordx4 x4 per 16 MFMA, L2-resident", mfma_with_stream<2, 4>, 4);
-        run("ds_read_b128 x8 per 16 MFMA", mfma_with_stream<3, 8>, 8);
     }
 
 
