@@ -118,6 +118,34 @@ int rocm_wmma_gemm_run_variant(int type_idx, int variant, int swizzle, int split
  * reference, which owns no memory. */
 int rocm_wmma_gemm_workspace_release(void);
 
+/* Size of the fixed per-GPU scratch buffer behind rocm_wmma_gemm_noalloc. */
+#define ROCM_WMMA_GEMM_NOALLOC_SCRATCH_BYTES (64u << 20)
+
+/* The same computation as the four reference entry points (type_idx picks the type pair),
+ * for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference, whose
+ * kernels need no scratch memory at all.  Here split-K partial sums and zero-padded copies
+ * of ragged operands do; the other entry points keep them in a buffer that the library
+ * allocates and grows on demand, this one keeps them in a fixed array of
+ * ROCM_WMMA_GEMM_NOALLOC_SCRATCH_BYTES that is part of the library's code object on every
+ * GPU (held from the first use of the library on that GPU until the process ends), and
+ * calls neither hipMalloc nor hipFree nor anything else that allocates.
+ *   - A call whose plan needs more scratch memory than the array holds fails with
+ *     ROCM_WMMA_GEMM_ERR_SCRATCH and enqueues nothing (of the shapes the library is
+ *     tuned for: K = 65536 at M = N = 1024, which wants 128 MiB of partial tiles, and
+ *     (4095, 5121, 3001), which wants 56 MiB of padded copies plus its partial tiles).
+ *     Calls that need no scratch memory (whole tiles, no split) have no size limit.
+ *   - The first call on a GPU looks the array's address up (hipGetSymbolAddress); make that
+ *     call outside graph capture.
+ *   - Every call on a GPU uses that GPU's one array, which keeps the previous call's
+ *     contents; nothing has to start at zero (each kernel writes what a later one reads).
+ *     Calls that overlap on one GPU (two streams, two threads) race on it: order them.
+ * Returns ROCM_WMMA_GEMM_OK or one of the codes above; a layout code outside {0, 1} is
+ * ROCM_WMMA_GEMM_ERR_ARGUMENT here rather than a silent no-op. */
+int rocm_wmma_gemm_noalloc(int type_idx, void* C, void* A, void* B, size_t M, size_t N, size_t K,
+                           size_t batch_count, int layout_c, int layout_a, int layout_b,
+                           void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -841,6 +841,38 @@ int run_with_status(int type_idx, const launch_plan* forced, void* C, void* A, v
     return rc;
 }
 
+// Scratch memory of the entry point that allocates nothing: one array per GPU, part of
+// the library's code object, so it is there from the moment the library is loaded on a
+// device until the process ends.  In host code the array's name only stands in for the
+// symbol; the memory's address on a device comes from hipGetSymbolAddress, asked once per
+// device with that device current, and only that address is ever handed to kernels.
+__attribute__((used)) static __device__ __align__(256) unsigned char scratch[ROCM_WMMA_GEMM_NOALLOC_SCRATCH_BYTES];
+std::mutex scratch_mutex;
+char*      scratch_address[max_devices] = {};
+
+int scratch_of_current_device(fixed_scratch* out)
+{
+    int dev = -1;
+    if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= max_devices)
+    {
+        return ROCM_WMMA_GEMM_ERR_RUNTIME;
+    }
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if(scratch_address[dev] == nullptr)
+    {
+        void* p = nullptr;
+        if(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr)
+        {
+            (void)hipGetLastError();
+            return ROCM_WMMA_GEMM_ERR_RUNTIME;
+        }
+        scratch_address[dev] = static_cast<char*>(p);
+    }
+    out->ptr   = scratch_address[dev];
+    out->bytes = ROCM_WMMA_GEMM_NOALLOC_SCRATCH_BYTES;
+    return 0;
+}
+
 } // namespace
 } // namespace host
 
@@ -1030,6 +1062,25 @@ int rocm_wmma_gemm_workspace_release(void)
     workspace_size[dev] = 0;
     workspace_used[dev] = false;
     return 0;
+}
+
+int rocm_wmma_gemm_noalloc(int type_idx, void* C, void* A, void* B, size_t M, size_t N, size_t K,
+                           size_t batch_count, int layout_c, int layout_a, int layout_b,
+                           void* stream)
+{
+    using namespace rocm_wmma_gemm::host;
+    if(type_idx < 0 || type_idx >= num_types || ((layout_c | layout_a | layout_b) & ~1))
+    {
+        return ROCM_WMMA_GEMM_ERR_ARGUMENT;
+    }
+    fixed_scratch own;
+    const int     rc = scratch_of_current_device(&own);
+    if(rc != 0)
+    {
+        return rc;
+    }
+    return run_with_status(type_idx, nullptr, C, A, B, M, N, K, batch_count, layout_c, layout_a,
+                           layout_b, stream_of(stream), &own);
 }
 
 } // extern "C"

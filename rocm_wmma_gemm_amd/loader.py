@@ -27,6 +27,7 @@ ENTRY_SUFFIXES = ("f16_f16", "f32_f16", "bf16_bf16", "f32_bf16")
 
 # status codes and the fixed scratch size of include/rocm_wmma_gemm_c.h
 OK, ERR_VARIANT, ERR_ARGUMENT, ERR_SCRATCH, ERR_RUNTIME, ERR_LIMIT = 0, -1, -2, -3, -4, -5
+NOALLOC_SCRATCH_BYTES = 64 << 20
 
 
 class GemmLibraryError(RuntimeError):
@@ -158,6 +159,9 @@ class Loader:
         if hasattr(L, "rocm_wmma_gemm_workspace_release"):
             L.rocm_wmma_gemm_workspace_release.restype = ctypes.c_int
             L.rocm_wmma_gemm_workspace_release.argtypes = []
+        if hasattr(L, "rocm_wmma_gemm_noalloc"):
+            L.rocm_wmma_gemm_noalloc.restype = ctypes.c_int
+            L.rocm_wmma_gemm_noalloc.argtypes = [ctypes.c_int] + self._ENTRY_ARGS
 
     def library_arch(self) -> str:
         return self._lib.rocm_wmma_gemm_arch().decode()
@@ -232,6 +236,19 @@ class Loader:
         """Frees the current device's library-owned scratch buffer (0), unless a captured
         graph may hold its address (1)."""
         return self._lib.rocm_wmma_gemm_workspace_release()
+
+    def gemm_noalloc(self, C, A, B, M: int, N: int, K: int, layout_c=row_major,
+                     layout_a=row_major, layout_b=row_major, batch_count: int = 1,
+                     stream=None) -> int:
+        """gemm() through the entry point that allocates nothing: scratch memory comes from
+        a fixed per-GPU array of NOALLOC_SCRATCH_BYTES.  Returns the library's status code
+        (0 = enqueued, ERR_SCRATCH = the call needs more scratch memory than that)."""
+        self._check(C, A, B, M, N, K, batch_count)
+        slot = _type_slot(C.dtype, A.dtype)
+        handle = ctypes.c_void_p(self._stream_handle(stream))
+        return self._lib.rocm_wmma_gemm_noalloc(
+            slot, C.data_ptr(), A.data_ptr(), B.data_ptr(), M, N, K, batch_count,
+            int(layout_c), int(layout_a), int(layout_b), ctypes.byref(handle))
 
     def run_variant(self, variant: int, swizzle: int, split_k: int, C, A, B, M: int, N: int,
                     K: int, layout_c=row_major, layout_a=row_major, layout_b=row_major,

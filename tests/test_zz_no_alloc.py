@@ -1,0 +1,83 @@
+"""The entry point that allocates nothing (rocm_wmma_gemm_noalloc) against the ordinary
+entry points, through the C ABI: same problems, same bits, on calls in a row that share
+the fixed per-GPU scratch array, the later ones smaller than the first."""
+import numpy as np
+import pytest
+
+import oracle as O
+from gemm_harness import TYPE_PAIRS, check_against_oracle, make_inputs, to_device, to_host, torch_dtype
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def loader():
+    import torch
+
+    import rocm_wmma_gemm_amd as R
+
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    torch.cuda.set_device(0)
+    return R.Loader()  # raises if the HIP library is missing: no fallback
+
+
+def _both_ways(loader, M, N, K, lc, la, lb, tname, batch=1):
+    import torch
+
+    din, dout = TYPE_PAIRS[tname]
+    A = np.concatenate([O.init_matrix(M, K, la, din, seed=1 + b) for b in range(batch)])
+    B = np.concatenate([O.init_matrix(K, N, lb, din, seed=101 + b) for b in range(batch)])
+    dA, dB = to_device(A, din), to_device(B, din)
+    want = torch.full((M * N * batch,), float("nan"), dtype=torch_dtype(dout), device="cuda")
+    got = torch.full_like(want, float("nan"))
+    loader.gemm(want, dA, dB, M, N, K, lc, la, lb, batch_count=batch)
+    rc = loader.gemm_noalloc(got, dA, dB, M, N, K, lc, la, lb, batch_count=batch)
+    torch.cuda.synchronize()
+    return rc, want, got, A, B
+
+
+def test_noalloc_entry_point_matches_the_ordinary_one_on_calls_in_a_row(loader):
+    import torch
+
+    import rocm_wmma_gemm_amd.loader as RL
+
+    cases = [  # the first is the largest user of the scratch array, the rest are smaller
+        (128, 8192, 8192, 0, 0, 1, "f32_f16", 1),    # split-K: fp32 partial planes
+        (64, 4096, 4096, 1, 0, 0, "f16_f16", 1),     # split-K, fewer and smaller planes
+        (1025, 1031, 2049, 0, 0, 1, "bf16_bf16", 1),  # ragged: padded copies (and partial tiles)
+        (16, 2048, 1024, 0, 1, 1, "f32_bf16", 3),    # small batched split
+        (512, 768, 1024, 0, 0, 1, "f16_f16", 1),     # whole tiles: no scratch memory at all
+    ]
+    for rnd in range(2):  # and once more from the top, over what the last round left behind
+        for (M, N, K, lc, la, lb, tname, batch) in cases:
+            rc, want, got, A, B = _both_ways(loader, M, N, K, lc, la, lb, tname, batch)
+            assert rc == RL.OK, (rc, M, N, K, tname)
+            assert not torch.isnan(got.float()).any()
+            # same plan, same kernels, same order of additions: the same bits
+            assert torch.equal(got, want), (rnd, M, N, K, lc, la, lb, tname)
+            if rnd == 0 and batch == 1:
+                din, dout = TYPE_PAIRS[tname]
+                check_against_oracle(to_host(got, dout), A, B, M, N, K, lc, la, lb, din, dout)
+
+
+def test_noalloc_entry_point_rejects_what_its_scratch_array_cannot_hold(loader):
+    import torch
+
+    import rocm_wmma_gemm_amd.loader as RL
+
+    # ragged in every extent, rows not 16-byte aligned: the plan is padded copies of both
+    # operands, 2 x 8192 x 8192 x 2 bytes = 256 MiB, four times the array
+    M = N = K = 8191
+    dA = torch.zeros(M * K, dtype=torch.float16, device="cuda")
+    dB = torch.zeros(K * N, dtype=torch.float16, device="cuda")
+    dC = torch.full((M * N,), float("nan"), dtype=torch.float16, device="cuda")
+    assert loader.gemm_noalloc(dC, dA, dB, M, N, K, 0, 0, 1) == RL.ERR_SCRATCH
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(dC).all()), "a rejected call must enqueue nothing"
+    # bad arguments are reported, not ignored
+    assert loader._lib.rocm_wmma_gemm_noalloc(7, 0, 0, 0, 16, 16, 16, 1, 0, 0, 0, None) == RL.ERR_ARGUMENT
+    assert loader._lib.rocm_wmma_gemm_noalloc(0, 0, 0, 0, 16, 16, 16, 1, 0, 2, 0, None) == RL.ERR_ARGUMENT
+    # and the array still serves the next call
+    rc, want, got, _, _ = _both_ways(loader, 64, 8192, 8192, 0, 0, 1, "f32_f16")
+    assert rc == RL.OK and torch.equal(got, want)
