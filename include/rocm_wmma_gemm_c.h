@@ -100,6 +100,16 @@ int rocm_wmma_gemm_select_batched(size_t M, size_t N, size_t K, size_t batch_cou
                                   int layout_c, int layout_a, int layout_b, int* swizzle,
                                   int* split_k);
 
+/* rocm_wmma_gemm_select_batched, also reporting the plan's fourth field: touch_ahead d > 0 =
+ * the persistent kernel, beside the loads of a K tile, touches the cache lines of the K tile
+ * d tiles further on (one dword per line from two waves of each workgroup, the workgroups
+ * that share an operand panel touching different quarters), so that those lines are on
+ * their way into the XCD's L2 a tile time before the loads that need them; it pays for a
+ * long K whose operands outgrow the memory-side cache and costs a few percent elsewhere,
+ * so the tuner decides.  0 = off; other kernels ignore it. */
+int rocm_wmma_gemm_select_ex(size_t M, size_t N, size_t K, size_t batch_count, int type_idx, int layout_c,
+                             int layout_a, int layout_b, int* swizzle, int* split_k, int* touch_ahead);
+
 /* Same computation as the four entry points above, but with the tile variant,
  * swizzle and split field (see above) forced (tuner hook).  Returns ROCM_WMMA_GEMM_OK,
  * ROCM_WMMA_GEMM_ERR_VARIANT if the variant cannot run this problem, or another of the
@@ -108,6 +118,32 @@ int rocm_wmma_gemm_run_variant(int type_idx, int variant, int swizzle, int split
                                void* A, void* B, size_t M, size_t N, size_t K,
                                size_t batch_count, int layout_c, int layout_a, int layout_b,
                                void* stream);
+
+/* rocm_wmma_gemm_run_variant with the plan's touch_ahead field forced too (see
+ * rocm_wmma_gemm_select_ex). */
+int rocm_wmma_gemm_run_variant_ex(int type_idx, int variant, int swizzle, int split_k, int touch_ahead,
+                                  void* C, void* A, void* B, size_t M, size_t N, size_t K,
+                                  size_t batch_count, int layout_c, int layout_a, int layout_b,
+                                  void* stream);
+
+/* Adds a tile variant that was compiled outside this library (the tuner builds
+ * rocm_wmma_gemm_amd/csrc/kernel_jit.hip for one tuple, type pair and pair of operand layouts
+ * and passes that library's rwg_jit_kernels here: entry points for the three load modes,
+ * 16-byte unguarded, 16-byte guarded, 2-byte; null where the pipeline has none).  The
+ * variant gets the next index after the compiled ones and runs through
+ * rocm_wmma_gemm_run_variant like any other; registering the same tuple again for another
+ * type pair or layout pair adds those kernels to the same index.  operand *_kmajor: 1 if K is
+ * the operand's contiguous dimension in the kernel's view (C row-major: A row-major, B
+ * column-major; a column-major C swaps the operands).  Returns the variant index,
+ * ROCM_WMMA_GEMM_ERR_VARIANT if the library already holds a compiled variant of this
+ * description, ROCM_WMMA_GEMM_ERR_ARGUMENT for a tuple no kernel can have, or
+ * ROCM_WMMA_GEMM_ERR_LIMIT when 64 variants have been registered.  The library that holds
+ * the kernels must stay loaded.  The role of the reference tuner's run-time compilation
+ * (reference rocm_wmma_gemm/config/tuner.cpp:237-454), split into compile (tuner) and
+ * launch (library). */
+int rocm_wmma_gemm_register_variant(int block_m, int block_n, int block_k, int warps_m, int warps_n,
+                                    int pipeline, int type_idx, int a_kmajor, int b_kmajor,
+                                    const void* const* kernels);
 
 /* Gives the current device's library-owned scratch buffer back (split-K partial sums and
  * padded operand copies live there: 256 MiB from the first call that needs it, more when a

@@ -168,8 +168,8 @@ def gpu_timer(type_name: str, reps: int, warmup: int):
             cache["A"] = (torch.rand(M * K, device="cuda") * 2 - 1).to(in_dtype)
             cache["B"] = (torch.rand(K * N, device="cuda") * 2 - 1).to(in_dtype)
             cache["C"] = torch.empty(M * N, dtype=c_dtype, device="cuda")
-        return time_candidate(L, torch, v, int(cfg.get("swizzle", 1)), hook_split(cfg),
-                              cache["C"], cache["A"], cache["B"], M, N, K,
+        return time_candidate(L, torch, v.index, int(cfg.get("swizzle", 1)), hook_split(cfg),
+                              int(cfg.get("touch_ahead", 0)), cache["C"], cache["A"], cache["B"], M, N, K,
                               LAYOUT_CODE[lc], LAYOUT_CODE[la], LAYOUT_CODE[lb], reps, warmup)
 
     return timer

@@ -92,6 +92,7 @@ launch_plan heuristic_plan(size_t m, size_t n, size_t k, int lc)
     plan.variant           = (rows >= 256 && cols >= 256 && big_tiles >= 128) ? 1 : 0;
     plan.swizzle           = 4;
     plan.split_k           = 1;
+    plan.touch             = 0;
     const size_t bm        = plan.variant == 1 ? 256 : 128;
     const size_t bk        = plan.variant == 1 ? 64 : 32;
     const size_t tiles     = ((rows + bm - 1) / bm) * ((cols + bm - 1) / bm);
@@ -246,6 +247,7 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
                 out->variant = i;
                 out->swizzle = 4;
                 out->split_k = split;
+                out->touch   = 0;
             }
         };
         // whole tiles

@@ -28,6 +28,8 @@ struct launch_plan
     int swizzle; // band height of the tile map: s > 0 bands of s tile rows, s < 0 bands of -s tile columns
     int split_k; // K slices (1 = off); -s (s > 1) = split only the last, partial wave of tiles s
                  // ways; -1 = persistent kernel walks by K tile (equal K tiles per workgroup)
+    int touch = 0; // persistent kernel: d > 0 = touch the cache lines of the K tile d tiles past
+                   // the one being loaded (see gemm_args::warm_ahead); 0 = off
 };
 
 struct tuned_entry

@@ -24,20 +24,54 @@ namespace host
 
 // LDS per workgroup: the staged pipeline double-buffers one tile pair; the direct
 // pipelines keep a ring of 2 (BLOCK_K 64) or 4 (BLOCK_K 32, and pipeline 6) tile pairs.
-#define RWG_VARIANT(IDX, BM, BN, BK, WM, WN, PIPE)                                         \
-    {BM, BN, BK, WM, WN, PIPE, ((PIPE) == 6 || ((PIPE) != 0 && (BK) == 32) ? 4 : 2) * (BM + BN) * BK * 2,   \
-     64 * WM * WN},
+constexpr int ring_bytes(int bm, int bn, int bk, int pipeline)
+{
+    return (pipeline == 6 || (pipeline != 0 && bk == 32) ? 4 : 2) * (bm + bn) * bk * 2;
+}
+
+#define RWG_VARIANT(IDX, BM, BN, BK, WM, WN, PIPE) \
+    {BM, BN, BK, WM, WN, PIPE, ring_bytes(BM, BN, BK, PIPE), 64 * WM * WN},
 const variant_desc variant_table[num_variants] = {
 #include "variants.def"
 };
 #undef RWG_VARIANT
 
+// Variants registered at run time (rocm_wmma_gemm_register_variant: kernels the tuner
+// compiled into a library of its own): indices num_variants, num_variants + 1, ...  A
+// slot is filled completely before registered_count is raised past it, and never changes
+// afterwards except for kernels being added to combinations that had none.
+constexpr int max_registered = 64;
+struct registered_variant
+{
+    variant_desc           desc;
+    std::atomic<kernel_fn> kernels[num_types][2][2][num_modes];
+};
+registered_variant registered[max_registered];
+std::atomic<int>   registered_count{0};
+std::mutex         register_mutex;
+
+int variant_total()
+{
+    return num_variants + registered_count.load(std::memory_order_acquire);
+}
+
+// Description of any variant, compiled or registered (index checked by the caller).
+const variant_desc& variant_at(int variant)
+{
+    return variant < num_variants ? variant_table[variant] : registered[variant - num_variants].desc;
+}
+
 kernel_fn lookup_kernel(int type_idx, bool a_kmajor, bool b_kmajor, int variant, int mode)
 {
-    if(type_idx < 0 || type_idx >= num_types || variant < 0 || variant >= num_variants || mode < 0
+    if(type_idx < 0 || type_idx >= num_types || variant < 0 || variant >= variant_total() || mode < 0
        || mode >= num_modes)
     {
         return nullptr;
+    }
+    if(variant >= num_variants)
+    {
+        return registered[variant - num_variants].kernels[type_idx][a_kmajor ? 1 : 0][b_kmajor ? 1 : 0][mode].load(
+            std::memory_order_acquire);
     }
     const int key = type_idx * 4 + (a_kmajor ? 2 : 0) + (b_kmajor ? 1 : 0);
     switch(key)
@@ -354,7 +388,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
            const fixed_scratch* fixed)
 {
     launch_plan plan = plan_in;
-    if(plan.variant < 0 || plan.variant >= num_variants)
+    if(plan.variant < 0 || plan.variant >= variant_total())
     {
         return -1;
     }
@@ -370,7 +404,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
     size_t      ldb      = p.b_kmajor ? p.K : p.N;
     size_t      k_kernel = p.K;
     size_t      stride_a = p.stride_a, stride_b = p.stride_b;
-    if(variant_table[plan.variant].pipeline == 5)
+    if(variant_at(plan.variant).pipeline == 5)
     {
         // The persistent kernel stores C in 16-byte pieces through a buffer descriptor per
         // tile: every row of C must start on 16 bytes and hold whole pieces, and a tile's
@@ -380,22 +414,22 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
                               && p.N < (size_t{1} << 21);
         if(!c_pieces)
         {
-            plan.variant = elementwise_store_variant(variant_table[plan.variant]);
+            plan.variant = elementwise_store_variant(variant_at(plan.variant));
             if(plan.split_k == -1)
             {
                 plan.split_k = 1;
             }
         }
     }
-    int         mode     = pick_mode(p, variant_table[plan.variant], plan.split_k);
+    int         mode     = pick_mode(p, variant_at(plan.variant), plan.split_k);
     size_t      pack_bytes = 0;
     bool        packed     = false; // the kernel reads a padded copy of ...
     bool        copy_a = false, copy_b = false; // ... this operand
     int         k_tail = 0; // columns of a partial last K tile that the kernel cuts off itself
 
-    if(variant_table[plan.variant].pipeline != 0)
+    if(variant_at(plan.variant).pipeline != 0)
     {
-        const variant_desc& dv = variant_table[plan.variant];
+        const variant_desc& dv = variant_at(plan.variant);
         const bool direct_ok = mode == static_cast<int>(device::load_mode::vec_unguarded)
                                && spans_fit(dv, p.a_kmajor, p.b_kmajor, lda, ldb);
         if(direct_ok)
@@ -455,7 +489,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
             {
                 pack_bytes   = 0;
                 plan.variant = staged_fallback(dv);
-                mode         = pick_mode(p, variant_table[plan.variant], plan.split_k);
+                mode         = pick_mode(p, variant_at(plan.variant), plan.split_k);
                 if(mode == static_cast<int>(device::load_mode::scalar))
                 {
                     // The 2-byte-load path keeps far more values in flight per thread;
@@ -465,7 +499,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
             }
         }
     }
-    const variant_desc& v = variant_table[plan.variant];
+    const variant_desc& v = variant_at(plan.variant);
 
     const size_t grid_m = (p.M + v.block_m - 1) / v.block_m;
     const size_t grid_n = (p.N + v.block_n - 1) / v.block_n;
@@ -585,7 +619,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
                 // no memory for the padded copies: take the general kernel instead
                 launch_plan retry = plan;
                 retry.variant     = staged_fallback(v);
-                if(pick_mode(p, variant_table[retry.variant], retry.split_k)
+                if(pick_mode(p, variant_at(retry.variant), retry.split_k)
                    == static_cast<int>(device::load_mode::scalar))
                 {
                     retry.variant = 0;
@@ -688,6 +722,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         args.batches          = static_cast<int>(nb);
         args.stream_units     = static_cast<int>(stream_units);
         args.k_tail           = k_tail;
+        args.warm_ahead       = persistent && plan.touch > 0 ? std::min(plan.touch, 3) : 0;
         args.batch_by_xcd     = (persistent || v.pipeline == 6) && nb > 1 && split_k == 1 && stream_groups == 0
                                         && blocks_per_batch * nb < (size_t{1} << 31)
                                     ? 1
@@ -762,7 +797,7 @@ int run(int type_idx, const launch_plan* forced, void* C, void* A, void* B, size
     const kernel_problem p = to_kernel_space(C, A, B, M, N, K, batch, layout_c, layout_a, layout_b);
     launch_plan          plan
         = forced ? *forced : select_plan(M, N, K, type_idx, layout_c, layout_a, layout_b, batch);
-    if(variant_table[plan.variant].pipeline != 0
+    if(variant_at(plan.variant).pipeline != 0
        && lookup_kernel(type_idx, p.a_kmajor, p.b_kmajor, plan.variant,
                         static_cast<int>(device::load_mode::vec_unguarded))
               == nullptr)
@@ -773,14 +808,14 @@ int run(int type_idx, const launch_plan* forced, void* C, void* A, void* B, size
         {
             return -1;
         }
-        plan.variant = staged_fallback(variant_table[plan.variant]);
+        plan.variant = staged_fallback(variant_at(plan.variant));
     }
-    if(!forced && variant_table[plan.variant].pipeline == 0)
+    if(!forced && variant_at(plan.variant).pipeline == 0)
     {
         // Same rule as in launch() for a staged variant picked directly: misaligned
         // operands go through the small tile.  A direct variant is left alone here:
         // launch() decides between padded copies and the staged kernels.
-        const int mode = pick_mode(p, variant_table[plan.variant], plan.split_k);
+        const int mode = pick_mode(p, variant_at(plan.variant), plan.split_k);
         if(mode == static_cast<int>(device::load_mode::scalar))
         {
             plan.variant = 0;
@@ -967,17 +1002,17 @@ const char* rocm_wmma_gemm_arch(void)
 
 int rocm_wmma_gemm_variant_count(void)
 {
-    return rocm_wmma_gemm::host::num_variants;
+    return rocm_wmma_gemm::host::variant_total();
 }
 
 int rocm_wmma_gemm_variant_info_get(int variant, rocm_wmma_gemm_variant_info* info)
 {
     using namespace rocm_wmma_gemm::host;
-    if(variant < 0 || variant >= num_variants || info == nullptr)
+    if(variant < 0 || variant >= variant_total() || info == nullptr)
     {
         return -1;
     }
-    const variant_desc& v = variant_table[variant];
+    const variant_desc& v = variant_at(variant);
     info->block_m         = v.block_m;
     info->block_n         = v.block_n;
     info->block_k         = v.block_k;
@@ -1021,13 +1056,48 @@ int rocm_wmma_gemm_select_batched(size_t M, size_t N, size_t K, size_t batch_cou
     return plan.variant;
 }
 
+int rocm_wmma_gemm_select_ex(size_t M, size_t N, size_t K, size_t batch_count, int type_idx, int layout_c,
+                             int layout_a, int layout_b, int* swizzle, int* split_k, int* touch_ahead)
+{
+    using namespace rocm_wmma_gemm::host;
+    if(type_idx < 0 || type_idx >= num_types || ((layout_c | layout_a | layout_b) & ~1)
+       || batch_count == 0)
+    {
+        return -1;
+    }
+    const launch_plan plan
+        = select_plan(M, N, K, type_idx, layout_c, layout_a, layout_b, batch_count);
+    if(swizzle)
+    {
+        *swizzle = plan.swizzle;
+    }
+    if(split_k)
+    {
+        *split_k = plan.split_k;
+    }
+    if(touch_ahead)
+    {
+        *touch_ahead = plan.touch;
+    }
+    return plan.variant;
+}
+
 int rocm_wmma_gemm_run_variant(int type_idx, int variant, int swizzle, int split_k, void* C,
                                void* A, void* B, size_t M, size_t N, size_t K,
                                size_t batch_count, int layout_c, int layout_a, int layout_b,
                                void* stream)
 {
+    return rocm_wmma_gemm_run_variant_ex(type_idx, variant, swizzle, split_k, 0, C, A, B, M, N, K,
+                                         batch_count, layout_c, layout_a, layout_b, stream);
+}
+
+int rocm_wmma_gemm_run_variant_ex(int type_idx, int variant, int swizzle, int split_k, int touch_ahead,
+                                  void* C, void* A, void* B, size_t M, size_t N, size_t K,
+                                  size_t batch_count, int layout_c, int layout_a, int layout_b,
+                                  void* stream)
+{
     using namespace rocm_wmma_gemm::host;
-    if(type_idx < 0 || type_idx >= num_types || variant < 0 || variant >= num_variants)
+    if(type_idx < 0 || type_idx >= num_types || variant < 0 || variant >= variant_total())
     {
         return ROCM_WMMA_GEMM_ERR_ARGUMENT;
     }
@@ -1035,8 +1105,65 @@ int rocm_wmma_gemm_run_variant(int type_idx, int variant, int swizzle, int split
     plan.variant = variant;
     plan.swizzle = swizzle;
     plan.split_k = split_k;
+    plan.touch   = touch_ahead < 0 ? 0 : touch_ahead;
     return run_with_status(type_idx, &plan, C, A, B, M, N, K, batch_count, layout_c, layout_a,
                            layout_b, stream_of(stream), nullptr);
+}
+
+int rocm_wmma_gemm_register_variant(int block_m, int block_n, int block_k, int warps_m, int warps_n,
+                                    int pipeline, int type_idx, int a_kmajor, int b_kmajor,
+                                    const void* const* kernels)
+{
+    using namespace rocm_wmma_gemm::host;
+    if(block_m <= 0 || block_n <= 0 || block_k <= 0 || warps_m <= 0 || warps_n <= 0 || pipeline < 0
+       || pipeline > 6 || block_m % (32 * warps_m) != 0 || block_n % (32 * warps_n) != 0
+       || 64 * warps_m * warps_n > 1024 || type_idx < 0 || type_idx >= num_types || kernels == nullptr
+       || ((a_kmajor | b_kmajor) & ~1) || ring_bytes(block_m, block_n, block_k, pipeline) > 160 * 1024)
+    {
+        return ROCM_WMMA_GEMM_ERR_ARGUMENT;
+    }
+    std::lock_guard<std::mutex> lock(register_mutex);
+    const int count = registered_count.load(std::memory_order_relaxed);
+    int       slot  = -1;
+    // a compiled variant of this description cannot take kernels; a registered one can
+    for(int i = 0; i < num_variants; ++i)
+    {
+        const variant_desc& v = variant_table[i];
+        if(v.block_m == block_m && v.block_n == block_n && v.block_k == block_k && v.waves_m == warps_m
+           && v.waves_n == warps_n && v.pipeline == pipeline)
+        {
+            return ROCM_WMMA_GEMM_ERR_VARIANT;
+        }
+    }
+    for(int i = 0; i < count; ++i)
+    {
+        const variant_desc& v = registered[i].desc;
+        if(v.block_m == block_m && v.block_n == block_n && v.block_k == block_k && v.waves_m == warps_m
+           && v.waves_n == warps_n && v.pipeline == pipeline)
+        {
+            slot = i;
+        }
+    }
+    if(slot < 0)
+    {
+        if(count >= max_registered)
+        {
+            return ROCM_WMMA_GEMM_ERR_LIMIT;
+        }
+        slot                  = count;
+        registered[slot].desc = {block_m, block_n, block_k, warps_m, warps_n, pipeline,
+                                 ring_bytes(block_m, block_n, block_k, pipeline), 64 * warps_m * warps_n};
+    }
+    for(int mode = 0; mode < num_modes; ++mode)
+    {
+        registered[slot].kernels[type_idx][a_kmajor][b_kmajor][mode].store(
+            reinterpret_cast<kernel_fn>(const_cast<void*>(kernels[mode])), std::memory_order_release);
+    }
+    if(slot == count)
+    {
+        registered_count.store(count + 1, std::memory_order_release);
+    }
+    return num_variants + slot;
 }
 
 int rocm_wmma_gemm_workspace_release(void)

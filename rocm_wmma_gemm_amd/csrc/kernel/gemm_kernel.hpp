@@ -81,6 +81,11 @@ struct gemm_args
                               // batch entry) are dealt so that each XCD works through one
                               // contiguous run of batch entries, and the tiles of an entry, which
                               // share its A and B, go through one L2 at about the same time
+    int         warm_ahead; // persistent kernel only.  1: beside the loads of a K tile, two waves
+                            // of a workgroup touch a quarter of the cache lines of the K tile
+                            // after it (one dword per line), so that the line is on its way into
+                            // the XCD's L2 a tile time before the loads that need it; the
+                            // workgroups that share an operand panel touch different quarters
 };
 
 // What one workgroup works on.  blockIdx.x enumerates the whole tiles first, then

@@ -273,6 +273,25 @@ struct solo_gemm
                      : "memory", "scc");
     }
 
+    // One dword per lane from 64 different cache lines, fetched for the sake of the fetch:
+    // the lines travel from memory into this XCD's L2 (and the dwords into 256 bytes of LDS
+    // that nothing reads).  Its range ends with the operand's allocation, so a touch past
+    // the end of a matrix fetches nothing.
+    __device__ __forceinline__ static void touch_lines(unsigned int lds_sink, unsigned int voff,
+                                                       const InT* origin, const InT* end, unsigned int soff)
+    {
+        const unsigned long long p    = (unsigned long long)origin;
+        const unsigned long long left = (unsigned long long)end > p ? (unsigned long long)end - p : 0;
+        const u32x4 rsrc{(unsigned int)p, (unsigned int)(p >> 32) & 0xffffu,
+                         left > RANGE_MAX ? RANGE_MAX : (unsigned int)left, 0x00020000u};
+        asm volatile("s_mov_b32 m0, %[sink]\n\t"
+                     "s_nop 4\n\t"
+                     "buffer_load_dword %[voff], %[rsrc], %[soff] offen lds"
+                     :
+                     : [sink] "s"(lds_sink), [voff] "v"(voff), [rsrc] "s"(rsrc), [soff] "s"(soff)
+                     : "memory");
+    }
+
     // Everything a step works on.
     struct step_ctx
     {
@@ -428,7 +447,8 @@ struct solo_gemm
     static constexpr int ROW_BYTES   = TN * 32; // 256 for the 128-column wave tile
     static constexpr int STRIP_PITCH = ROW_BYTES + 16;
     static constexpr int STRIP_BYTES = (16 * STRIP_PITCH + 1023) / 1024 * 1024;
-    static_assert(LDS_BYTES + WAVES * STRIP_BYTES <= 160 * 1024, "tile ring and store strips must fit the 160 KB LDS");
+    static_assert(LDS_BYTES + WAVES * STRIP_BYTES + WAVES * 256 <= 160 * 1024,
+                  "tile ring, store strips and the sink of the line touches must fit the 160 KB LDS");
 
     // Ties a row of accumulators to its registers at this point of the program: what
     // follows reads the row from there.  Without it the compiler copies all 256
@@ -739,7 +759,7 @@ struct solo_gemm
     // 13 us, nine K tiles' worth, at 256 x 256 x 64.)
     __device__ __forceinline__ static void run(const gemm_args& args)
     {
-        __shared__ __attribute__((aligned(1024))) char lds_raw[LDS_BYTES + WAVES * STRIP_BYTES];
+        __shared__ __attribute__((aligned(1024))) char lds_raw[LDS_BYTES + WAVES * STRIP_BYTES + WAVES * 256];
         lds_char_ptr lds = (lds_char_ptr)lds_raw;
 
         const int tid    = threadIdx.x;
@@ -786,6 +806,29 @@ struct solo_gemm
         int        stream_left = cur.nk;
         int        stream_next = cur.next;
         bool       stream_ends = cur.ends_k;
+        // Line touches (args.warm_ahead = distance in K tiles, + 4 for "every workgroup touches
+        // whole tiles"): which quarter of a K tile's lines this workgroup touches.  The
+        // workgroups that share an A panel differ in their tile column, those that share a B
+        // panel in their tile row, so a run of four neighbours covers a tile; wave 0 touches
+        // A's lines, wave 1 B's.  With whole tiles, wave w touches quarter w of both.
+        const int          warm_dist = args.warm_ahead & 3;
+        const bool         warm_full = (args.warm_ahead & 4) != 0;
+        const unsigned int lds_sink  = (unsigned int)(size_t)lds + LDS_BYTES + WAVES * STRIP_BYTES + wave * 256;
+        // K-contiguous: lane l touches the line of row 4 l + quarter (a row of a K tile is one
+        // line); else lane l touches line `quarter` of k row l (four lines of 128 bytes hold
+        // the 256 elements of a k row)
+        const unsigned int warm_voff_a = (unsigned int)((A_KMAJOR ? 4 * lane : lane) * a_ld * 2);
+        const unsigned int warm_voff_b = (unsigned int)((B_KMAJOR ? 4 * lane : lane) * b_ld * 2);
+        const InT* warm_end_a = scalar_pointer(static_cast<const InT*>(args.A) + (args.batches - 1) * args.batch_stride_a
+                                               + (A_KMAJOR ? (long long)args.M * a_ld : (long long)args.K * a_ld));
+        const InT* warm_end_b = scalar_pointer(static_cast<const InT*>(args.B) + (args.batches - 1) * args.batch_stride_b
+                                               + (B_KMAJOR ? (long long)args.N * b_ld : (long long)args.K * b_ld));
+        // (scalar by hand: the tile coordinates come out of vector divisions)
+        auto quarters_of = [&](const work_item& x) {
+            const unsigned int qa = warm_full ? wave : (x.col0 / BN) & 3, qb = warm_full ? wave : (x.row0 / BM) & 3;
+            return (unsigned int)__builtin_amdgcn_readfirstlane(qa | (qb << 8));
+        };
+        unsigned int stream_quarters = quarters_of(cur);
         auto advance = [&]() {
             a_src += a_step;
             b_src += b_step;
@@ -799,6 +842,7 @@ struct solo_gemm
                 stream_left        = nx.nk;
                 stream_next        = nx.next;
                 stream_ends        = nx.ends_k;
+                stream_quarters    = quarters_of(nx);
             }
         };
         // whether the tile at (a_src, b_src) is a last K tile held only in part
@@ -872,6 +916,23 @@ struct solo_gemm
                 step<1, plan_a>(c0, fa[0], fb[0], fa[1], fb[1], acc);
                 __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
                 __builtin_amdgcn_s_barrier();
+                if(warm_dist != 0 && stream_left > warm_dist)
+                {
+                    // a K tile further down the stream than the one whose loads follow, if it
+                    // is the same item's
+                    if(warm_full || wave == 0)
+                    {
+                        touch_lines(lds_sink, warm_voff_a, a_src + warm_dist * a_step, warm_end_a,
+                                    (unsigned int)__builtin_amdgcn_readfirstlane((unsigned int)(
+                                        (stream_quarters & 255) * (A_KMAJOR ? a_ld * 2 : 128))));
+                    }
+                    if(warm_full || wave == 1)
+                    {
+                        touch_lines(lds_sink, warm_voff_b, b_src + warm_dist * b_step, warm_end_b,
+                                    (unsigned int)__builtin_amdgcn_readfirstlane((unsigned int)(
+                                        (stream_quarters >> 8) * (B_KMAJOR ? b_ld * 2 : 128))));
+                    }
+                }
                 step<0, plan_b>(c1, fa[1], fb[1], fa[0], fb[0], acc);
                 a_prev     = a_src;
                 b_prev     = b_src;

@@ -156,6 +156,12 @@ class Loader:
             ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
         L.rocm_wmma_gemm_run_variant.restype = ctypes.c_int
         L.rocm_wmma_gemm_run_variant.argtypes = [ctypes.c_int] * 4 + self._ENTRY_ARGS
+        if hasattr(L, "rocm_wmma_gemm_run_variant_ex"):
+            L.rocm_wmma_gemm_run_variant_ex.restype = ctypes.c_int
+            L.rocm_wmma_gemm_run_variant_ex.argtypes = [ctypes.c_int] * 5 + self._ENTRY_ARGS
+            L.rocm_wmma_gemm_select_ex.restype = ctypes.c_int
+            L.rocm_wmma_gemm_select_ex.argtypes = [ctypes.c_size_t] * 4 + [ctypes.c_int] * 4 + [
+                ctypes.POINTER(ctypes.c_int)] * 3
         if hasattr(L, "rocm_wmma_gemm_workspace_release"):
             L.rocm_wmma_gemm_workspace_release.restype = ctypes.c_int
             L.rocm_wmma_gemm_workspace_release.argtypes = []
@@ -250,13 +256,23 @@ class Loader:
             slot, C.data_ptr(), A.data_ptr(), B.data_ptr(), M, N, K, batch_count,
             int(layout_c), int(layout_a), int(layout_b), ctypes.byref(handle))
 
+    def select_ex(self, M: int, N: int, K: int, type_idx: int, layout_c: int, layout_a: int,
+                  layout_b: int, batch_count: int = 1) -> tuple[int, int, int, int]:
+        """(variant, swizzle, split_k, touch_ahead) the dispatcher picks for this problem."""
+        swz, sk, touch = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+        v = self._lib.rocm_wmma_gemm_select_ex(
+            M, N, K, batch_count, type_idx, int(layout_c), int(layout_a), int(layout_b),
+            ctypes.byref(swz), ctypes.byref(sk), ctypes.byref(touch))
+        return v, swz.value, sk.value, touch.value
+
     def run_variant(self, variant: int, swizzle: int, split_k: int, C, A, B, M: int, N: int,
                     K: int, layout_c=row_major, layout_a=row_major, layout_b=row_major,
-                    batch_count: int = 1, stream=None) -> int:
-        """Same as gemm() with the tile variant, swizzle and split-K forced (tuner hook)."""
+                    batch_count: int = 1, stream=None, touch_ahead: int = 0) -> int:
+        """Same as gemm() with the tile variant, swizzle, split-K form and line touches forced
+        (tuner hook)."""
         self._check(C, A, B, M, N, K, batch_count)
         slot = _type_slot(C.dtype, A.dtype)
         handle = ctypes.c_void_p(self._stream_handle(stream))
-        return self._lib.rocm_wmma_gemm_run_variant(
-            slot, variant, swizzle, split_k, C.data_ptr(), A.data_ptr(), B.data_ptr(), M, N, K,
-            batch_count, int(layout_c), int(layout_a), int(layout_b), ctypes.byref(handle))
+        return self._lib.rocm_wmma_gemm_run_variant_ex(
+            slot, variant, swizzle, split_k, touch_ahead, C.data_ptr(), A.data_ptr(), B.data_ptr(),
+            M, N, K, batch_count, int(layout_c), int(layout_a), int(layout_b), ctypes.byref(handle))

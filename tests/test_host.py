@@ -180,9 +180,13 @@ def test_generator_rejects_unknown_variant_and_roundtrips(tmp_path):
     p = tmp_path / "gemm_config_gfx950_f16.json"
     p.write_text(json.dumps(doc))
     rows = G.build_table(str(p), None, variants)
-    assert rows == [(64, 64, 64, 0, 0, 1, 0, 0, 16, 1)]  # later duplicate wins
+    assert rows == [(64, 64, 64, 0, 0, 1, 0, 0, 16, 1, 0)]  # later duplicate wins
     text = G.render(rows, [str(p)])
-    assert "{64, 64, 64, 0, 0, 1, 0, {0, 16, 1}}" in text
+    assert "{64, 64, 64, 0, 0, 1, 0, {0, 16, 1, 0}}" in text
+    doc["configurations"][1]["config"]["touch_ahead"] = 1
+    doc["configurations"][1]["timed_on"] = "bf16_bf16"  # entries may say what they were timed on
+    p.write_text(json.dumps(doc))
+    assert G.build_table(str(p), None, variants) == [(64, 64, 64, 0, 0, 1, 0, 0, 16, 1, 1)]
 
 
 def test_split_fields_of_a_config_entry():
@@ -403,3 +407,153 @@ def test_tile_ring_of_the_direct_kernels_stays_deep_for_transposed_operands(tmp_
         stray = [code[n] for n in waits if not code[n + 1].startswith("s_barrier")]
         assert not stray, f"{func}: {stray}"
         assert len(waits) <= 1, func
+
+
+# ---------------------------------------------------------------- tuner (search space, GOMEA, run-time compile)
+def _tune_module():
+    sys.path.insert(0, os.path.join(ROOT, "rocm_wmma_gemm_amd", "config"))
+    import tune
+
+    return tune
+
+
+def test_tuner_constraints_accept_every_compiled_variant_and_reject_what_cannot_build():
+    T = _tune_module()
+    import rocm_wmma_gemm_amd as R
+
+    for v in R.Loader(arch="gfx950").variants():
+        t = T.Tile(v.block_m, v.block_n, v.block_k, v.warps_m, v.warps_n, v.pipeline)
+        assert T.tile_feasible(t, True, True), t  # both operands K-contiguous: every variant is built
+        if v.block_m % 128 or v.block_n % 128:
+            if v.pipeline != 0:
+                assert not T.tile_feasible(t, False, False), t
+    bad = [T.Tile(256, 256, 64, 2, 2, 6),   # ring of 4 x 64 KB
+           T.Tile(256, 256, 64, 1, 2, 1),   # 256 x 128 wave tile: 512 accumulator registers
+           T.Tile(256, 256, 64, 2, 2, 2),   # ping-pong needs 8 waves
+           T.Tile(64, 128, 64, 4, 1, 1),    # 64 rows over 4 waves: less than a 32-row MFMA block each
+           T.Tile(128, 128, 32, 2, 2, 5),   # the persistent kernel is built for BLOCK_K 64
+           T.Tile(32, 32, 32, 2, 2, 1)]     # 2 KiB per operand tile over 4 waves
+    for t in bad:
+        assert not T.tile_feasible(t, True, True), t
+    # split forms: plain split-K only with few tiles and a long K; a tail split only with a thin last wave
+    big = T.Tile(256, 256, 64, 2, 2, 5)
+    assert T.split_feasible(big, 4, 1, 4096, 4096, 4096)
+    assert not T.split_feasible(big, 4, 4, 4096, 4096, 4096)
+    assert T.split_feasible(big, 1, 16, 1024, 1024, 65536)
+    assert T.split_feasible(big, 4, -4, 4352, 4096, 8192) and not T.split_feasible(big, 4, -4, 4096, 4096, 8192)
+    assert T.split_feasible(big, 4, -1, 3072, 3072, 3072) and not T.split_feasible(T.Tile(256, 256, 64, 2, 4, 1), 4, -1, 3072, 3072, 3072)
+    assert T.kernel_space_layout(0, 1, 0) == (True, True) and T.kernel_space_layout(0, 0, 1) == (False, True)
+
+
+def test_gomea_finds_the_optimum_of_a_linked_landscape_with_a_fake_timer():
+    """The search, driven by a synthetic timer instead of the GPU (as test_race_* drive
+    race.py): a landscape over the tuner's real gene domains whose best point is a tuple the
+    library does not hold and needs genes to change together (a K step of 32 only pays with
+    eight waves, and only on one tile shape), with infeasible regions and candidates that
+    fail to run.  Seeded with the compiled variants, as the tuner seeds it, GOMEA must find
+    the optimum while timing a small part of the feasible space."""
+    import itertools
+    import random
+
+    T = _tune_module()
+    import rocm_wmma_gemm_amd as R
+
+    domains = [T.GENES[g] for g in T.GENE_ORDER]
+    calls = []
+
+    def fake_ms(genes):
+        tile, sw, sk, touch = T.decode(genes)
+        calls.append(genes)
+        if tile.pipeline == 4 and tile.block_k == 32:
+            return None  # "failed to compile"
+        t = 10.0
+        eight = (tile.warps_m, tile.warps_n) == (2, 4)
+        t -= 2.0 * (tile.block_k == 32 and eight) - 1.0 * (tile.block_k == 32 and not eight)  # linked
+        t -= 1.5 * (tile.pipeline == 1 and tile.block_m == 128 and tile.block_n == 256)
+        t -= 0.8 * (tile.pipeline == 5)  # a good basin elsewhere
+        t -= 0.01 * (tile.block_m + tile.block_n) / 32
+        t += 0.1 * abs(sw - 8) / 8 + 0.3 * (sk != 1) + 0.05 * touch
+        return t
+
+    def feasible(genes):
+        tile, sw, sk, touch = T.decode(genes)
+        return (T.tile_feasible(tile, True, True) and T.split_feasible(tile, sw, sk, 4096, 4096, 4096)
+                and T.touch_feasible(tile, touch, 4096))
+
+    feasible_points = [g for g in itertools.product(*domains) if feasible(g)]
+    truth = min((fake_ms(g), g) for g in feasible_points if fake_ms(g) is not None)
+    best_tile = T.decode(truth[1])[0]
+    assert (best_tile.block_m, best_tile.block_n, best_tile.block_k, best_tile.pipeline) == (128, 256, 32, 1)
+    seeds = [T.encode(T.Tile(v.block_m, v.block_n, v.block_k, v.warps_m, v.warps_n, v.pipeline), 4, 1)
+             for v in R.Loader(arch="gfx950").variants()]
+    seeds = [g for g in seeds if g is not None]
+    assert truth[1] not in seeds
+    calls.clear()
+    wins = 0
+    for seed in range(5):
+        best, ms, evals = T.gomea(domains, feasible, fake_ms, budget=200, rng=random.Random(seed), seeds=seeds)
+        assert evals <= 200 and best is not None and feasible(best)
+        assert ms <= min(fake_ms(g) for g in seeds if feasible(g) and fake_ms(g) is not None)
+        wins += ms == truth[0]
+    assert wins >= 4, f"optimum {truth} found in {wins} of 5 runs"
+    assert len(feasible_points) > 3 * 200, len(feasible_points)
+    assert all(feasible(g) for g in calls), "an infeasible candidate was timed"
+    # the budget is a hard limit and a landscape with nothing feasible ends at once
+    best, ms, evals = T.gomea(domains, lambda g: False, fake_ms, budget=50, rng=random.Random(0))
+    assert best is None and evals == 0
+    # a table entry round-trips through the genes
+    cfg = T.config_json(T.Tile(256, 256, 64, 2, 2, 5), 8, -4, 1)
+    assert cfg["tail_split"] == 4 and cfg["touch_ahead"] == 1
+    assert T.decode(T.encode(*T.tuple_of(cfg))) == (T.Tile(256, 256, 64, 2, 2, 5), 8, -4, 1)
+    assert T.touch_feasible(T.Tile(256, 256, 64, 2, 2, 5), 1, 16384)
+    assert not T.touch_feasible(T.Tile(256, 256, 64, 2, 4, 1), 1, 16384)
+
+
+def test_tuner_compiles_a_tuple_the_library_does_not_hold_and_registers_it(tmp_path, built_library):
+    """The open search space: a tuple outside csrc/variants.def is compiled from
+    csrc/kernel_jit.hip at tune time and added to the loaded library, where it gets the
+    next variant index (reference config/tuner.cpp:237-395 compiles one tuple with hipRTC)."""
+    T = _tune_module()
+    import rocm_wmma_gemm_amd as R
+
+    L = R.Loader(arch="gfx950")
+    compiled = L.variants()
+    tile = T.Tile(128, 256, 32, 2, 2, 1)
+    assert all((v.block_m, v.block_n, v.block_k, v.warps_m, v.warps_n, v.pipeline)
+               != (128, 256, 32, 2, 2, 1) for v in compiled)
+    jit = T.JitBuilder(L._lib, cache_dir=str(tmp_path))
+    idx = jit.variant_index(tile, 0, True, True)
+    assert idx == len(compiled)
+    again = L.variants()
+    assert len(again) == len(compiled) + 1
+    v = again[idx]
+    assert (v.block_m, v.block_n, v.block_k, v.warps_m, v.warps_n, v.pipeline) == (128, 256, 32, 2, 2, 1)
+    assert v.lds_bytes == 4 * (128 + 256) * 32 * 2 and v.threads == 256
+    # another layout pair of the same tuple joins the same index; the build is cached
+    assert jit.variant_index(tile, 0, True, False) == idx
+    assert T.JitBuilder(L._lib, cache_dir=str(tmp_path)).build(tile, 0, True, True) is not None
+    assert len(L.variants()) == len(compiled) + 1
+    # a tuple the templates refuse does not build; a compiled tuple cannot be registered
+    assert jit.variant_index(T.Tile(256, 256, 64, 2, 2, 2), 0, True, True) is None
+    c = compiled[2]
+    fake = (ctypes.c_void_p * 3)(0, 0, 0)
+    assert L._lib.rocm_wmma_gemm_register_variant(c.block_m, c.block_n, c.block_k, c.warps_m, c.warps_n,
+                                                  c.pipeline, 0, 1, 1, fake) == -1
+    assert L._lib.rocm_wmma_gemm_register_variant(100, 256, 64, 2, 2, 1, 0, 1, 1, fake) == -2
+
+
+def test_tuner_adopts_new_tuples_into_the_variant_list(tmp_path):
+    T = _tune_module()
+    src = os.path.join(ROOT, "rocm_wmma_gemm_amd", "csrc", "variants.def")
+    copy = tmp_path / "variants.def"
+    copy.write_text(open(src).read())
+    sys.path.insert(0, os.path.join(ROOT, "rocm_wmma_gemm_amd", "config"))
+    import generate_config as G
+
+    before = G.read_variants(str(copy))
+    added = T.adopt([T.Tile(128, 256, 32, 2, 2, 1), T.Tile(256, 256, 64, 2, 2, 5),
+                     T.Tile(128, 256, 32, 2, 2, 1)], path=str(copy))
+    assert added == [f"RWG_VARIANT({len(before)}, 128, 256, 32, 2, 2, 1)"]
+    after = G.read_variants(str(copy))  # still dense and parseable
+    assert len(after) == len(before) + 1 and after[-1]["block_k"] == 32
+    assert T.adopt([T.Tile(128, 256, 32, 2, 2, 1)], path=str(copy)) == []
