@@ -227,6 +227,23 @@ def main() -> int:
         out["float_bf16_8192_rcr"] = {"tflops": round(tf2, 1),
                                       "pct_of_peak": round(100 * tf2 / PEAK_TFLOPS, 2),
                                       "data": "normal(0,1) seed 1"}
+        # the HBM-bound corner of the workload set: M = 16 against N = K = 8192, A row-major,
+        # B column-major (weights stored N x K); algorithmic bytes over the time per call
+        m3, n3 = 16, 8192
+        A3 = (torch.rand(m3 * n3, device="cuda", generator=gen) * 2 - 1).to(torch.float16)
+        B3 = (torch.rand(n3 * n3, device="cuda", generator=gen) * 2 - 1).to(torch.float16)
+        C3 = torch.empty(m3 * n3, dtype=torch.float16, device="cuda")
+        run3 = lambda: loader.gemm(C3, A3, B3, m3, n3, n3, 0, 0, 1)  # noqa: E731
+        for _ in range(a.warmup):
+            run3()
+        s, _ = timed_region(torch, run3, a.steps)
+        bytes3 = (m3 * n3 + n3 * n3 + m3 * n3) * 2
+        out["skinny_16x8192x8192_rcr"] = {
+            "us_per_call_back_to_back": round(s / a.steps * 1e6, 2),
+            "tb_per_s": round(bytes3 * a.steps / s / 1e12, 3),
+            "frac_of_8_tb_per_s_hbm_roof": round(bytes3 * a.steps / s / 8e12, 3),
+            "algorithmic_bytes": bytes3}
+        del A3, B3, C3
         # vendor libraries on the same GPU and the same data (context only): rocBLAS and
         # hipBLASLt called directly through libvendor_gemm.so, and torch.matmul
         vendor_ctx = {}

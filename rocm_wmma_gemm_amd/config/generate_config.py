@@ -93,7 +93,31 @@ def build_table(f16_json: str, f32_json: str | None, variants: list[dict]) -> li
     return sorted(seen.values())
 
 
-def render(rows: list[tuple], sources: list[str]) -> str:
+def load_model(path: str) -> dict:
+    with open(path) as f:
+        m = json.load(f)
+    for key in ("compute_units", "launch_us", "reduce_us", "plane_bytes_per_us", "tile_bytes_per_us",
+                "copy_bytes_per_us", "step_us", "item_us"):
+        if key not in m:
+            raise ValueError(f"{path}: missing {key}")
+    return m
+
+
+def render_model(m: dict) -> list[str]:
+    steps = []
+    for pipe, tiles in sorted(m["step_us"].items()):
+        for tile, us in sorted(tiles.items()):
+            bm, bn = (int(x) for x in tile.split("x"))
+            steps.append(f"    {{{int(pipe)}, {bm}, {bn}, {float(us)!r}, {float(m['item_us'][pipe])!r}}},")
+    return ([f"constexpr int model_compute_units = {int(m['compute_units'])};"]
+            + [f"constexpr double model_{k} = {float(m[k])!r};" for k in
+               ("launch_us", "reduce_us", "plane_bytes_per_us", "tile_bytes_per_us", "copy_bytes_per_us")]
+            + [f"constexpr int model_step_count = {len(steps)};",
+               f"constexpr model_step model_steps[{max(len(steps), 1)}] = {{"]
+            + (steps or ["    {0, 0, 0, 0.0, 0.0},"]) + ["};"])
+
+
+def render(rows: list[tuple], sources: list[str], model: dict | None = None) -> str:
     lines = [
         "// Generated by config/generate_config.py -- do not edit.",
         "// Sources: " + ", ".join(os.path.basename(s) for s in sources),
@@ -108,7 +132,9 @@ def render(rows: list[tuple], sources: list[str]) -> str:
         lines.append("    {0, 0, 0, 0, 0, 0, 0, {0, 1, 1, 0}},")
     for m, n, k, tg, la, lb, lc, var, swz, sk, touch in rows:
         lines.append(f"    {{{m}, {n}, {k}, {tg}, {la}, {lb}, {lc}, {{{var}, {swz}, {sk}, {touch}}}}},")
-    lines += ["};", "}}} // namespace rocm_wmma_gemm::host::generated", "#endif", ""]
+    lines += ["};"]
+    lines += render_model(model if model is not None else load_model(os.path.join(HERE, "model_gfx950.json")))
+    lines += ["}}} // namespace rocm_wmma_gemm::host::generated", "#endif", ""]
     return "\n".join(lines)
 
 
@@ -118,6 +144,7 @@ def main(argv=None) -> int:
     ap.add_argument("--f16-config", default=None)
     ap.add_argument("--f32-config", default=None)
     ap.add_argument("--variants", default=os.path.join(CSRC, "variants.def"))
+    ap.add_argument("--model", default=None, help="constants of the dispatcher's time estimate (model_<arch>.json)")
     ap.add_argument("output", nargs="?", default=os.path.join(CSRC, "config_generated.hpp"))
     a = ap.parse_args(argv)
     f16 = a.f16_config or os.path.join(HERE, f"gemm_config_{a.arch}_f16.json")
@@ -127,7 +154,8 @@ def main(argv=None) -> int:
     f32 = a.f32_config or os.path.join(HERE, f"gemm_config_{a.arch}_f32.json")
     variants = read_variants(a.variants)
     rows = build_table(f16, f32, variants)
-    text = render(rows, [f16] + ([f32] if os.path.exists(f32) else []))
+    model_path = a.model or os.path.join(HERE, f"model_{a.arch}.json")
+    text = render(rows, [f16] + ([f32] if os.path.exists(f32) else []) + [model_path], load_model(model_path))
     old = open(a.output).read() if os.path.exists(a.output) else None
     if old != text:
         with open(a.output, "w") as f:

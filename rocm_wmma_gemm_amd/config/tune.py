@@ -143,6 +143,14 @@ def tile_feasible(t: Tile, a_kmajor: bool, b_kmajor: bool) -> bool:
     waves = t.warps_m * t.warps_n
     if t.block_m % (32 * t.warps_m) or t.block_n % (32 * t.warps_n):
         return False
+    if t.pipeline == 7:
+        # whole-K streaming kernel: small tiles, stages of 128, at least one operand
+        # K-contiguous, the other on a 64-wide side of the tile
+        return ((a_kmajor or b_kmajor) and (a_kmajor or t.block_m == 64) and (b_kmajor or t.block_n == 64)
+                and t.block_k == 128 and t.block_m in (32, 64) and t.block_n in (32, 64)
+                and (t.warps_m, t.warps_n) == (t.block_m // 32, t.block_n // 32))
+    if t.block_k == 128:
+        return False
     wtm, wtn = t.block_m // t.warps_m, t.block_n // t.warps_n
     if wtm * wtn // 64 > 256:  # accumulator registers per lane
         return False
@@ -180,6 +188,11 @@ def split_feasible(t: Tile, swizzle: int, split: int, rows: int, cols: int, K: i
         return False  # a tile much larger than the problem only wastes work
     if tiles <= 8 and swizzle != 1:
         return False
+    if t.pipeline == 7:
+        # one workgroup per tile over the whole K: no band height, no split; worth a try
+        # when a 256 x 256 tiling leaves most compute units without a tile
+        return swizzle == (1 if tiles <= 8 else 4) and split == 1 \
+            and -(-rows // 256) * -(-cols // 256) < CUS // 2 and K % 128 == 0
     if split == 1:
         return True
     if split > 1:

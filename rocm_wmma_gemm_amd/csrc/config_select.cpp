@@ -13,6 +13,11 @@ namespace host
 
 const tuned_entry* const tuned_table = generated::entries;
 const size_t             tuned_count = generated::entry_count;
+const model_constants    model_measured
+    = {generated::model_compute_units,      generated::model_launch_us,
+       generated::model_reduce_us,          generated::model_plane_bytes_per_us,
+       generated::model_tile_bytes_per_us,  generated::model_copy_bytes_per_us,
+       generated::model_steps,              generated::model_step_count};
 
 namespace
 {
@@ -126,27 +131,23 @@ const model_variant model_variants[] = {
 };
 #undef RWG_VARIANT
 
-// Microseconds per K tile of 64 with every CU of an MI355X at work, and per tile for
-// its stores, read off the tuner's measurements (persistent 16x16x32 kernel at 4096^3
-// to 8192^3 and 3072^3; ring-of-4 direct kernel at 2048^3 and the skinny shapes).
+// Microseconds per K tile of 64 with every compute unit at work, and per tile for its
+// stores: measured constants (model_measured), one pair per pipeline and tile.
 bool step_cost(const model_variant& v, double* step_us, double* item_us)
 {
     if(v.block_k != 64)
     {
         return false;
     }
-    const int area = v.block_m * v.block_n;
-    if(v.pipeline == 5)
+    for(int i = 0; i < model_measured.step_count; ++i)
     {
-        *step_us = area == 256 * 256 ? 1.30 : area == 256 * 192 ? 1.05 : area == 192 * 192 ? 0.90 : 0.0;
-        *item_us = 5.0;
-        return *step_us > 0.0;
-    }
-    if(v.pipeline == 6)
-    {
-        *step_us = area == 128 * 128 ? 0.60 : area == 64 * 256 ? 0.50 : 0.0;
-        *item_us = 2.0;
-        return *step_us > 0.0;
+        const model_step& s = model_measured.steps[i];
+        if(s.pipeline == v.pipeline && s.block_m == v.block_m && s.block_n == v.block_n)
+        {
+            *step_us = s.step_us;
+            *item_us = s.item_us;
+            return true;
+        }
     }
     return false;
 }
@@ -166,7 +167,8 @@ size_t ceil_div(size_t a, size_t b)
 // with the second less than half full) and ran at 0.7 of the 196 tiles of 256 x 256.
 // On the 208 tuned entries the model can serve, its pick is on average 2.7 % slower than
 // the tuner's, 25 % at worst.
-bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_plan* out, size_t batch)
+bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_plan* out, size_t batch,
+                size_t cus_of_device)
 {
     const size_t rows = lc == 0 ? m : n;
     const size_t cols = lc == 0 ? n : m;
@@ -186,15 +188,43 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
     {
         return false; // shapes every direct kernel would only take through padded copies
     }
-    constexpr size_t cus           = 256;
-    constexpr double launch_us     = 6.0;
-    constexpr double reduce_us     = 4.0;
-    constexpr double plane_bytes_per_us = 2.2e6; // partial planes: written, then read by reduce_partials
-    constexpr double tile_bytes_per_us  = 3.7e6; // partial tiles (split tail, walk by K tile)
+    // Skinny against a large K-contiguous operand (decode-like: 16..64 rows against 8192 x
+    // 8192): the whole-K streaming kernel, 32 rows or columns on the skinny side and 64 on
+    // the side that streams from HBM.  Measured at N = K = 8192, fp16, one call at a time:
+    // M = 16 / 32 / 64 in 33.9 / 33.7 / 35.2 us against 39.1 / 44.9 / 39.8 us for the best
+    // split-K plan with its reduce launch; at M = 128 the split-K plan stays ahead (43.5
+    // against 47.1 us), every workgroup reading all of the small operand from L2.
+    // The operand on the skinny side must be K-contiguous; the large one may also be
+    // contiguous along its rows of the tile (weights stored K x N), on the 64-wide side.
+    if(k % 128 == 0 && k >= 2048 && batch == 1
+       && ((rows <= 64 && cols >= 2048 && a_kmajor) || (cols <= 64 && rows >= 2048 && b_kmajor)))
+    {
+        const int want_m = rows <= 64 ? 32 : 64, want_n = rows <= 64 ? 64 : 32;
+        const int count  = static_cast<int>(sizeof(model_variants) / sizeof(model_variants[0]));
+        for(int i = 0; i < count; ++i)
+        {
+            if(model_variants[i].pipeline == 7 && model_variants[i].block_m == want_m
+               && model_variants[i].block_n == want_n)
+            {
+                out->variant = i;
+                out->swizzle = 1;
+                out->split_k = 1;
+                out->touch   = 0;
+                return true;
+            }
+        }
+    }
+    // (the constants are per compute unit at work, so the estimate carries over to a GPU
+    // or partition with another count; the tile walk still assumes 8 XCDs)
+    const size_t cus                = cus_of_device != 0 ? cus_of_device : static_cast<size_t>(model_measured.compute_units);
+    const double launch_us          = model_measured.launch_us;
+    const double reduce_us          = model_measured.reduce_us;
+    const double plane_bytes_per_us = model_measured.plane_bytes_per_us; // written, then read by reduce_partials
+    const double tile_bytes_per_us  = model_measured.tile_bytes_per_us; // split tail, walk by K tile
     // (small planes are paid for in latency, not bandwidth: past 32 MB the rest moves at
     // twice the rate; 8192x1024x8192 cut in two moves 134 MB in ~30 us)
     auto plane_traffic_us = [&](double bytes) {
-        constexpr double knee = 32.0 * 1024 * 1024;
+        const double knee = 32.0 * 1024 * 1024;
         return bytes <= knee ? bytes / plane_bytes_per_us
                              : knee / plane_bytes_per_us + (bytes - knee) / (2.0 * plane_bytes_per_us);
     };
@@ -236,7 +266,7 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
             const double elems = ((rows % bm != 0 || !k_whole ? static_cast<double>(tm * bm) * k_pad : 0.0)
                                   + (cols % bn != 0 || !k_whole ? static_cast<double>(tn * bn) * k_pad : 0.0))
                                  * static_cast<double>(batch);
-            copies_us = launch_us + elems * 2.0 * 2.0 / 3.0e6;
+            copies_us = launch_us + elems * 2.0 * 2.0 / model_measured.copy_bytes_per_us;
         }
         auto consider = [&](double t, int split) {
             t += copies_us;
@@ -322,13 +352,14 @@ launch_plan select_plan_from(const tuned_entry* table, size_t count, size_t m, s
     return heuristic_plan(m, n, k, lc);
 }
 
-launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int la, int lb, size_t batch)
+launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int la, int lb, size_t batch,
+                        size_t cus)
 {
     const int   group = type_group_of(type_idx);
     launch_plan plan;
     // the table was tuned on single GEMMs: a batch changes how many tiles there are to
     // spread, which is the model's business
-    if(batch > 1 && model_plan(m, n, k, lc, la, lb, &plan, batch))
+    if(batch > 1 && model_plan(m, n, k, lc, la, lb, &plan, batch, cus))
     {
         return plan;
     }
@@ -339,7 +370,7 @@ launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int 
         return plan;
     }
     // ... then the model for regular shapes, and the nearest tuned entry for the rest
-    if(model_plan(m, n, k, lc, la, lb, &plan, 1))
+    if(model_plan(m, n, k, lc, la, lb, &plan, 1, cus))
     {
         return plan;
     }

@@ -40,6 +40,27 @@ struct tuned_entry
     launch_plan plan;
 };
 
+// Constants of model_plan's time estimate (microseconds, bytes per microsecond), measured
+// on the GPU: config/fit_model.py fits them to a tuner log, config/model_<arch>.json keeps
+// them and config/generate_config.py copies them into the generated header.
+struct model_step
+{
+    int    pipeline, block_m, block_n;
+    double step_us; // per K tile of 64 with every compute unit at work
+    double item_us; // per tile: the stores of C and the turn to the next tile
+};
+struct model_constants
+{
+    int    compute_units; // of the GPU the constants were measured on
+    double launch_us, reduce_us;
+    double plane_bytes_per_us; // split-K partial planes: written, then read by the reduce kernel
+    double tile_bytes_per_us; // partial tiles of a split tail wave or of the walk by K tile
+    double copy_bytes_per_us; // padded operand copies
+    const model_step* steps;
+    int               step_count;
+};
+extern const model_constants model_measured;
+
 // Defined in config_select.cpp
 extern const tuned_entry* const tuned_table;
 extern const size_t             tuned_count;
@@ -52,7 +73,9 @@ bool find_closest(const tuned_entry* table, size_t count, size_t m, size_t n, si
 launch_plan heuristic_plan(size_t m, size_t n, size_t k, int lc);
 // Estimated-time choice among the compiled variants for a shape without a tuned entry;
 // false for shapes it does not cover (ragged K, odd extents).
-bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_plan* out, size_t batch = 1);
+// cus: compute units of the GPU the plan is for (0: the GPU the constants were measured on).
+bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_plan* out, size_t batch = 1,
+                size_t cus = 0);
 launch_plan select_plan_from(const tuned_entry* table, size_t count, size_t m, size_t n, size_t k,
                              int type_idx, int lc, int la, int lb);
 
@@ -61,7 +84,8 @@ inline int type_group_of(int type_idx)
     return (type_idx == 1 || type_idx == 3) ? 1 : 0;
 }
 
-launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int la, int lb, size_t batch = 1);
+launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int la, int lb, size_t batch = 1,
+                        size_t cus = 0);
 
 } // namespace host
 } // namespace rocm_wmma_gemm

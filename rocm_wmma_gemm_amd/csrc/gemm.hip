@@ -26,11 +26,23 @@ namespace host
 // pipelines keep a ring of 2 (BLOCK_K 64) or 4 (BLOCK_K 32, and pipeline 6) tile pairs.
 constexpr int ring_bytes(int bm, int bn, int bk, int pipeline)
 {
+    if(pipeline == 7)
+    {
+        // as many stages as fit 144 KB, at most 8 (device::stream_gemm::DEPTH)
+        const int stage = (bm + bn) * bk * 2, depth = 144 * 1024 / stage;
+        return (depth < 8 ? depth : 8) * stage;
+    }
     return (pipeline == 6 || (pipeline != 0 && bk == 32) ? 4 : 2) * (bm + bn) * bk * 2;
 }
 
+// (the streaming kernel always runs 4 waves: they split K, not the tile)
+constexpr int workgroup_threads(int wm, int wn, int pipeline)
+{
+    return pipeline == 7 ? 256 : 64 * wm * wn;
+}
+
 #define RWG_VARIANT(IDX, BM, BN, BK, WM, WN, PIPE) \
-    {BM, BN, BK, WM, WN, PIPE, ring_bytes(BM, BN, BK, PIPE), 64 * WM * WN},
+    {BM, BN, BK, WM, WN, PIPE, ring_bytes(BM, BN, BK, PIPE), workgroup_threads(WM, WN, PIPE)},
 const variant_desc variant_table[num_variants] = {
 #include "variants.def"
 };
@@ -383,6 +395,75 @@ bool spans_fit(const variant_desc& v, bool a_kmajor, bool b_kmajor, size_t lda, 
     return a_span < (1ull << bits) && b_span < (1ull << bits);
 }
 
+// What the whole-K streaming kernel (pipeline 7) takes: at least one operand K-contiguous
+// (the other then 64 wide in the tile, with 16-byte aligned k rows), K whole stages of 128,
+// 16-byte aligned rows, and a stage of a tile within reach of a 31-bit offset.
+bool streaming_ok(const kernel_problem& p, const variant_desc& v)
+{
+    if(!(p.K >= 128 && p.K % 128 == 0 && aligned16(p.A) && aligned16(p.B)
+         && (p.batch == 1 || (p.stride_a % 8 == 0 && p.stride_b % 8 == 0))))
+    {
+        return false;
+    }
+    if(!p.a_kmajor && !p.b_kmajor)
+    {
+        return false;
+    }
+    if((!p.a_kmajor && (v.block_m != 64 || p.M % 8 != 0)) || (!p.b_kmajor && (v.block_n != 64 || p.N % 8 != 0)))
+    {
+        return false;
+    }
+    // byte offsets inside a tile: 64 rows of K elements, or K rows of the operand's width
+    const unsigned long long span_a = p.a_kmajor ? 64ull * p.K * 2 : 1ull * p.K * p.M * 2;
+    const unsigned long long span_b = p.b_kmajor ? 64ull * p.K * 2 : 1ull * p.K * p.N * 2;
+    return span_a < (1ull << 31) && span_b < (1ull << 31);
+}
+
+template<class OutT>
+int launch_streaming(int type_idx, const launch_plan& plan, const kernel_problem& p, hipStream_t stream)
+{
+    const variant_desc& v = variant_at(plan.variant);
+    if(!streaming_ok(p, v))
+    {
+        return -1;
+    }
+    kernel_fn fn = lookup_kernel(type_idx, p.a_kmajor, p.b_kmajor, plan.variant,
+                                 static_cast<int>(device::load_mode::vec_guarded));
+    if(fn == nullptr)
+    {
+        return -1;
+    }
+    const size_t grid_m = (p.M + v.block_m - 1) / v.block_m, grid_n = (p.N + v.block_n - 1) / v.block_n;
+    if(grid_m * grid_n > 0x7fffffffull)
+    {
+        throw std::runtime_error("rocm_wmma_gemm: tile grid too large");
+    }
+    for(size_t b0 = 0; b0 < p.batch; b0 += 65535)
+    {
+        const size_t      nb = std::min<size_t>(65535, p.batch - b0);
+        device::gemm_args args{};
+        args.C              = static_cast<char*>(p.C) + b0 * p.stride_c * sizeof(OutT);
+        args.A              = static_cast<const char*>(p.A) + b0 * p.stride_a * in_bytes;
+        args.B              = static_cast<const char*>(p.B) + b0 * p.stride_b * in_bytes;
+        args.M              = static_cast<int>(p.M);
+        args.N              = static_cast<int>(p.N);
+        args.K              = static_cast<int>(p.K);
+        args.lda            = static_cast<long long>(p.a_kmajor ? p.K : p.M);
+        args.ldb            = static_cast<long long>(p.b_kmajor ? p.K : p.N);
+        args.batch_stride_a = static_cast<long long>(p.stride_a);
+        args.batch_stride_b = static_cast<long long>(p.stride_b);
+        args.batch_stride_c = static_cast<long long>(p.stride_c);
+        args.grid_m         = static_cast<int>(grid_m);
+        args.grid_n         = static_cast<int>(grid_n);
+        args.group          = 1;
+        args.k_slices       = 1;
+        args.blocks_per_batch = static_cast<int>(grid_m * grid_n);
+        args.batches          = static_cast<int>(nb);
+        fn<<<dim3(static_cast<unsigned>(grid_m * grid_n), static_cast<unsigned>(nb)), dim3(v.threads), 0, stream>>>(args);
+    }
+    return 0;
+}
+
 template<class OutT>
 int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hipStream_t stream,
            const fixed_scratch* fixed)
@@ -395,6 +476,11 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
     if(p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull)
     {
         throw std::runtime_error("rocm_wmma_gemm: M, N and K must each fit in 31 bits");
+    }
+
+    if(variant_at(plan.variant).pipeline == 7)
+    {
+        return launch_streaming<OutT>(type_idx, plan, p, stream);
     }
 
     // Operand views the kernel will see; may be replaced by padded copies below.
@@ -796,7 +882,9 @@ int run(int type_idx, const launch_plan* forced, void* C, void* A, void* B, size
     }
     const kernel_problem p = to_kernel_space(C, A, B, M, N, K, batch, layout_c, layout_a, layout_b);
     launch_plan          plan
-        = forced ? *forced : select_plan(M, N, K, type_idx, layout_c, layout_a, layout_b, batch);
+        = forced ? *forced
+                 : select_plan(M, N, K, type_idx, layout_c, layout_a, layout_b, batch,
+                               compute_units_of_current_device());
     if(variant_at(plan.variant).pipeline != 0
        && lookup_kernel(type_idx, p.a_kmajor, p.b_kmajor, plan.variant,
                         static_cast<int>(device::load_mode::vec_unguarded))
@@ -1116,7 +1204,7 @@ int rocm_wmma_gemm_register_variant(int block_m, int block_n, int block_k, int w
 {
     using namespace rocm_wmma_gemm::host;
     if(block_m <= 0 || block_n <= 0 || block_k <= 0 || warps_m <= 0 || warps_n <= 0 || pipeline < 0
-       || pipeline > 6 || block_m % (32 * warps_m) != 0 || block_n % (32 * warps_n) != 0
+       || pipeline > 7 || block_m % (32 * warps_m) != 0 || block_n % (32 * warps_n) != 0
        || 64 * warps_m * warps_n > 1024 || type_idx < 0 || type_idx >= num_types || kernels == nullptr
        || ((a_kmajor | b_kmajor) & ~1) || ring_bytes(block_m, block_n, block_k, pipeline) > 160 * 1024)
     {
@@ -1152,7 +1240,8 @@ int rocm_wmma_gemm_register_variant(int block_m, int block_n, int block_k, int w
         }
         slot                  = count;
         registered[slot].desc = {block_m, block_n, block_k, warps_m, warps_n, pipeline,
-                                 ring_bytes(block_m, block_n, block_k, pipeline), 64 * warps_m * warps_n};
+                                 ring_bytes(block_m, block_n, block_k, pipeline),
+                                 workgroup_threads(warps_m, warps_n, pipeline)};
     }
     for(int mode = 0; mode < num_modes; ++mode)
     {

@@ -1,0 +1,320 @@
+// Whole-K streaming MFMA GEMM kernel for gfx950: small output tiles (32 or 64 rows and
+// columns), one workgroup per tile, the whole K range inside the workgroup, for problems
+// that are bound by the stream of one operand from HBM (a skinny M or N against a large
+// N x K or M x K operand: decode-like shapes).
+//
+// What it is for.  A 16 x 8192 x 8192 GEMM reads 134 MB of B and does almost no arithmetic.
+// With 256 x 256 tiles it has 32 tiles for 256 compute units; the other kernels therefore
+// cut K into slices, write fp32 partial planes and add them up in a second launch, which
+// costs a quarter of the call.  Here the tiles are small enough that N / 32 of them cover
+// every compute unit without cutting K, so one launch does the whole job and the sums
+// keep one fixed order:
+//   - a workgroup streams its 32 (or 64) rows of the large operand from HBM exactly once,
+//     and its rows of the small operand from L2 (every workgroup reads all of the small
+//     operand: M x K x 2 bytes each, which is why this pays only while M is small);
+//   - the small operand must be K-contiguous (row-major activations); the large one may be
+//     K-contiguous (weights stored N x K: a row of a stage is 256 contiguous bytes, two
+//     whole cache lines) or contiguous along N (weights stored K x N), in which case its
+//     side of the tile is 64 wide, so that a k row of the tile is one whole cache line,
+//     and the fragments are transposed on the way to registers by ds_read_b64_tr_b16;
+//   - the LDS holds a ring of up to 8 stages of BK = 128 (24..64 KB of loads in flight per
+//     workgroup: what it takes to cover the latency of HBM at 20 GB/s per compute unit),
+//     filled by buffer_load ... lds, 1 KiB per instruction (4 rows x 256 bytes);
+//   - the four waves split the K range of a stage (32 each) and every wave multiplies the
+//     whole tile on v_mfma_f32_16x16x32; at the end the four partial tiles are added in
+//     wave order through LDS and the sum is converted and stored;
+//   - rows past M or N are read as zeros (the buffer descriptors end with the operand)
+//     and not stored.
+//
+// LDS layout of a stage: the A tile (BM rows), then the B tile (BN rows).  K-contiguous
+// operand: a row is 16 chunks of 16 bytes, chunk c of row r in slot c ^ (r mod 16), so
+// that the 16 rows a fragment read touches per k chunk fall on 16 different slots (all 64
+// banks once).  M/N-contiguous operand: 128 k rows of 64 elements (128 bytes), as they lie
+// in memory.
+//
+// Role with respect to the reference: as the other kernels, its gemm_impl (reference
+// rocm_wmma_gemm/include/rocm_wmma_gemm/kernel/kernel.hpp:108-556); the reference has no
+// kernel for these shapes and serves them with its nearest tuned tile (reference
+// rocm_wmma_gemm/config/generate_config.py:174-234).
+#ifndef ROCM_WMMA_GEMM_STREAM_KERNEL_HPP
+#define ROCM_WMMA_GEMM_STREAM_KERNEL_HPP
+
+#include "direct_kernel.hpp"
+
+namespace rocm_wmma_gemm
+{
+namespace device
+{
+
+template<in_kind IN, class OutT, int BM, int BN, bool A_KMAJOR = true, bool B_KMAJOR = true>
+struct stream_gemm
+{
+    using InT = typename std::conditional<IN == in_kind::f16, _Float16, __bf16>::type;
+
+    static constexpr int BK        = 128;
+    static constexpr int ROW_BYTES = BK * 2;
+    static constexpr int WAVES     = 4;
+    static constexpr int THREADS   = 64 * WAVES;
+    static constexpr int A_BYTES   = BM * ROW_BYTES;
+    static constexpr int B_BYTES   = BN * ROW_BYTES;
+    static constexpr int STAGE     = A_BYTES + B_BYTES;
+    static constexpr int DEPTH     = (144 * 1024) / STAGE < 8 ? (144 * 1024) / STAGE : 8;
+    static constexpr int LDS_BYTES = DEPTH * STAGE;
+    static constexpr int TM        = BM / 16; // MFMA tiles of a workgroup tile
+    static constexpr int TN        = BN / 16;
+    // 1 KiB loads (4 rows) of a stage per wave: load q of an operand covers rows 4q .. 4q+3
+    // and belongs to wave q mod 4
+    // (M/N-contiguous, 64 wide: load q covers k rows 8q .. 8q+7, 16 loads a stage)
+    static constexpr int LOADS_A = BM / 16;
+    static constexpr int LOADS_B = BN / 16;
+    static constexpr int PER     = LOADS_A + LOADS_B;
+    static_assert((BM == 32 || BM == 64) && (BN == 32 || BN == 64), "tiles of 32 or 64 rows and columns");
+    static_assert(A_KMAJOR || B_KMAJOR, "the small operand is K-contiguous");
+    static_assert((A_KMAJOR || BM == 64) && (B_KMAJOR || BN == 64),
+                  "a k row of an M/N-contiguous tile is one 128-byte line");
+    static_assert(DEPTH >= 3 && (DEPTH - 1) * PER < 64, "ring depth against the 6-bit vmcnt");
+    static_assert(WAVES * BM * BN * 4 <= LDS_BYTES, "the partial tiles of the waves reuse the ring");
+
+    // s_waitcnt immediate: vmcnt(n), lgkmcnt and expcnt untouched
+    static constexpr int vmcnt_imm(int n)
+    {
+        return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14);
+    }
+
+    __device__ __forceinline__ static u32x4 descriptor(const InT* origin, long long bytes)
+    {
+        const unsigned long long p = (unsigned long long)origin;
+        const unsigned int       lo = __builtin_amdgcn_readfirstlane((unsigned int)p);
+        const unsigned int       hi = __builtin_amdgcn_readfirstlane((unsigned int)(p >> 32));
+        const unsigned int       records
+            = __builtin_amdgcn_readfirstlane(bytes <= 0 ? 0u : bytes > 0x7fffffffll ? 0x7fffffffu : (unsigned int)bytes);
+        return u32x4{lo, hi & 0xffffu, records, 0x00020000u};
+    }
+
+    // One 1 KiB load: lane l's 16 bytes go to lds_block + 16 l.  (The compiler does not
+    // look for hazards around inline assembly: four wait states cover M0 and a descriptor
+    // or offset that a v_readfirstlane has just written.)
+    __device__ __forceinline__ static void load_block(unsigned int lds_block, unsigned int voff, const u32x4& rsrc,
+                                                      unsigned int soff)
+    {
+        asm volatile("s_mov_b32 m0, %[ldsb]\n\t"
+                     "s_nop 4\n\t"
+                     "buffer_load_dwordx4 %[voff], %[rsrc], %[soff] offen lds"
+                     :
+                     : [ldsb] "s"(lds_block), [voff] "v"(voff), [rsrc] "s"(rsrc), [soff] "s"(soff)
+                     : "memory");
+    }
+
+    __device__ __forceinline__ static void run(const gemm_args& args)
+    {
+        __shared__ __attribute__((aligned(1024))) char lds_raw[LDS_BYTES];
+        lds_char_ptr       lds      = (lds_char_ptr)lds_raw;
+        const unsigned int lds_addr = (unsigned int)(size_t)lds;
+
+        const int lane = threadIdx.x & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+
+        // Tile of this workgroup.  Workgroup ids that are congruent mod 8 run on the same
+        // XCD; when the tile grid has two or more tiles along its short side, the
+        // workgroups that share a panel of the large operand are given ids 8 apart, so
+        // that the panel crosses the fabric once and the others find it in that XCD's L2.
+        const int wg = blockIdx.x;
+        int       tm, tn;
+        if(args.grid_m <= args.grid_n && args.grid_n % 8 == 0)
+        {
+            const int xcd = wg & 7, j = wg >> 3;
+            tm = j % args.grid_m;
+            tn = (j / args.grid_m) * 8 + xcd;
+        }
+        else if(args.grid_n < args.grid_m && args.grid_m % 8 == 0)
+        {
+            const int xcd = wg & 7, j = wg >> 3;
+            tn = j % args.grid_n;
+            tm = (j / args.grid_n) * 8 + xcd;
+        }
+        else
+        {
+            tm = wg % args.grid_m;
+            tn = wg / args.grid_m;
+        }
+        const long long batch = blockIdx.y;
+        const int       row0 = tm * BM, col0 = tn * BN;
+        const long long lda = args.lda, ldb = args.ldb;
+        // K-contiguous: rows of the tile are rows of the operand, and the descriptor ends
+        // with the rows of this batch entry, so a tile that hangs over the edge reads zeros
+        // there.  M/N-contiguous: the tile is 64 columns of the operand's K rows, the
+        // descriptor ends with the batch entry, and columns past the edge read what lies
+        // there (the next k row): they only reach columns of C that are not stored.
+        const InT* a0 = static_cast<const InT*>(args.A) + batch * args.batch_stride_a
+                        + (A_KMAJOR ? (long long)row0 * lda : (long long)row0);
+        const InT* b0 = static_cast<const InT*>(args.B) + batch * args.batch_stride_b
+                        + (B_KMAJOR ? (long long)col0 * ldb : (long long)col0);
+        const u32x4 rsrc_a = descriptor(a0, A_KMAJOR ? (long long)(args.M - row0) * lda * 2
+                                                     : ((long long)args.K * lda - row0) * 2);
+        const u32x4 rsrc_b = descriptor(b0, B_KMAJOR ? (long long)(args.N - col0) * ldb * 2
+                                                     : ((long long)args.K * ldb - col0) * 2);
+
+        // K-contiguous: load q = wave + 4 i of an operand covers rows 4q + l/16, LDS slot
+        // l%16 of that row, so the lane fetches chunk (l%16) ^ (row mod 16), and row mod 16 =
+        // 4 wave + l/16 for every i.  M/N-contiguous: load q = wave + 4 i covers k rows
+        // 8q + l/8, 16-byte piece l%8 of the row's 128 bytes, in memory order.
+        const int          sub    = lane >> 4, slot = lane & 15;
+        const int          chunk  = slot ^ ((4 * wave + sub) & 15);
+        const unsigned int voff_a = A_KMAJOR ? (unsigned int)(((4 * wave + sub) * lda + chunk * 8) * 2)
+                                             : (unsigned int)(((8 * wave + (lane >> 3)) * lda + (lane & 7) * 8) * 2);
+        const unsigned int voff_b = B_KMAJOR ? (unsigned int)(((4 * wave + sub) * ldb + chunk * 8) * 2)
+                                             : (unsigned int)(((8 * wave + (lane >> 3)) * ldb + (lane & 7) * 8) * 2);
+        // bytes from load i to load i+1 (16 rows, or 32 k rows), and from stage to stage
+        const unsigned int step_a  = (unsigned int)((A_KMAJOR ? 16 : 32) * lda * 2);
+        const unsigned int step_b  = (unsigned int)((B_KMAJOR ? 16 : 32) * ldb * 2);
+        const unsigned int stage_a = A_KMAJOR ? (unsigned int)ROW_BYTES : (unsigned int)(BK * lda * 2);
+        const unsigned int stage_b = B_KMAJOR ? (unsigned int)ROW_BYTES : (unsigned int)(BK * ldb * 2);
+
+        const int stages = args.K / BK;
+        auto      issue  = [&](int stage, int slot_index) {
+            const unsigned int base = lds_addr + slot_index * STAGE + wave * 1024;
+#pragma unroll
+            for(int i = 0; i < LOADS_A; ++i)
+            {
+                load_block(base + i * 4096, voff_a, rsrc_a,
+                           __builtin_amdgcn_readfirstlane((unsigned int)stage * stage_a + i * step_a));
+            }
+#pragma unroll
+            for(int i = 0; i < LOADS_B; ++i)
+            {
+                load_block(base + A_BYTES + i * 4096, voff_b, rsrc_b,
+                           __builtin_amdgcn_readfirstlane((unsigned int)stage * stage_b + i * step_b));
+            }
+        };
+        // Past the last stage the loads fetch the last stage again into slots that nobody
+        // reads any more: the number of loads in flight stays what the waits assume.
+        auto clamped = [&](int stage) { return stage < stages ? stage : stages - 1; };
+
+        for(int t = 0; t < DEPTH - 1; ++t)
+        {
+            issue(clamped(t), t);
+        }
+
+        f32x4 acc[TM][TN];
+#pragma unroll
+        for(int i = 0; i < TM; ++i)
+        {
+#pragma unroll
+            for(int j = 0; j < TN; ++j)
+            {
+                acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+        }
+
+        // fragment of this wave's K step (k 32 wave .. 32 wave + 31 of the stage).
+        // K-contiguous: row l%16 of a 16-row block, k chunk 4 wave + l/16.  M/N-contiguous:
+        // two transposing reads of 4 k rows x 16 elements per 16 lanes; lane p of a group of
+        // 16 supplies the address of 4 elements of k row p/4 (ds_read_b64_tr_b16 hands lane
+        // i, element j what lane 4j + i/4 addressed, element i%4), so the group that feeds k
+        // 8 g .. 8 g + 7 reads rows 32 wave + 8 g + p/4 and the same 4 rows further on.
+        const int frag_off = slot * ROW_BYTES + (((4 * wave + sub) ^ slot) & 15) * 16;
+        const int tr_off   = (32 * wave + 8 * sub + (slot >> 2)) * 128 + (slot & 3) * 8;
+        using lds_u32x4    = __attribute__((address_space(3))) u32x4;
+        // (one statement with its own wait: the compiler does not know that these
+        // registers are filled later, and would copy them into place at once)
+        auto transposed = [](unsigned int addr) {
+            uint2 lo, hi;
+            asm volatile("ds_read_b64_tr_b16 %0, %2\n\t"
+                         "ds_read_b64_tr_b16 %1, %2 offset:512\n\t"
+                         "s_waitcnt lgkmcnt(0)"
+                         : "=&v"(lo), "=&v"(hi)
+                         : "v"(addr)
+                         : "memory");
+            return u32x4{lo.x, lo.y, hi.x, hi.y};
+        };
+
+        int slot_index = 0; // of stage t
+        for(int t = 0; t < stages; ++t)
+        {
+            // stage t has landed (the loads of the DEPTH - 2 stages after it may be in
+            // flight), in every wave: then its slot may be read, and the slot of stage
+            // t - 1, which every wave has finished reading, may be filled again
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm((DEPTH - 2) * PER));
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            issue(clamped(t + DEPTH - 1), slot_index == 0 ? DEPTH - 1 : slot_index - 1);
+
+            lds_char_ptr       sa   = lds + slot_index * STAGE + frag_off;
+            const unsigned int sa_t = lds_addr + slot_index * STAGE + tr_off;
+            u32x4              fa[TM], fb[TN];
+#pragma unroll
+            for(int i = 0; i < TM; ++i)
+            {
+                if constexpr(A_KMAJOR)
+                {
+                    fa[i] = *reinterpret_cast<lds_u32x4*>(sa + i * 16 * ROW_BYTES);
+                }
+                else
+                {
+                    fa[i] = transposed(sa_t + i * 32);
+                }
+            }
+#pragma unroll
+            for(int j = 0; j < TN; ++j)
+            {
+                if constexpr(B_KMAJOR)
+                {
+                    fb[j] = *reinterpret_cast<lds_u32x4*>(sa + A_BYTES + j * 16 * ROW_BYTES);
+                }
+                else
+                {
+                    fb[j] = transposed(sa_t + A_BYTES + j * 32);
+                }
+            }
+#pragma unroll
+            for(int i = 0; i < TM; ++i)
+            {
+#pragma unroll
+                for(int j = 0; j < TN; ++j)
+                {
+                    acc[i][j] = mfma_16x16x32<IN>(fa[i], fb[j], acc[i][j]);
+                }
+            }
+            slot_index = slot_index + 1 == DEPTH ? 0 : slot_index + 1;
+        }
+
+        // every load has landed and every wave has read its last stage: the ring becomes
+        // the four partial tiles, [wave][BM][BN] fp32
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        using lds_float = __attribute__((address_space(3))) float;
+        lds_float* part = reinterpret_cast<lds_float*>(lds);
+#pragma unroll
+        for(int i = 0; i < TM; ++i)
+        {
+#pragma unroll
+            for(int j = 0; j < TN; ++j)
+            {
+#pragma unroll
+                for(int v = 0; v < 4; ++v)
+                {
+                    // result register v of a 16 x 16 tile: row 4 (l/16) + v, column l%16
+                    part[(wave * BM + 16 * i + 4 * sub + v) * BN + 16 * j + slot] = acc[i][j][v];
+                }
+            }
+        }
+        __syncthreads();
+        OutT* C = static_cast<OutT*>(args.C) + batch * args.batch_stride_c;
+        for(int e = threadIdx.x; e < BM * BN; e += THREADS)
+        {
+            const int row = e / BN, col = e % BN;
+            // (wave order: the sum of an element is the same in every run)
+            const float s = ((part[e] + part[BM * BN + e]) + part[2 * BM * BN + e]) + part[3 * BM * BN + e];
+            if(row0 + row < args.M && col0 + col < args.N)
+            {
+                C[(long long)(row0 + row) * args.N + col0 + col] = to_out<OutT>(s);
+            }
+        }
+    }
+};
+
+} // namespace device
+} // namespace rocm_wmma_gemm
+
+#endif // ROCM_WMMA_GEMM_STREAM_KERNEL_HPP

@@ -10,6 +10,7 @@
 #include "kernel/direct_kernel.hpp"
 #include "kernel/pingpong_kernel.hpp"
 #include "kernel/solo_kernel.hpp"
+#include "kernel/stream_kernel.hpp"
 #include "kernel/gemm_kernel.hpp"
 
 namespace rocm_wmma_gemm

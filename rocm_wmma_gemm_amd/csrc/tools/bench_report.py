@@ -1,13 +1,15 @@
 #!/usr/bin/env python3
 """Markdown comparison tables (and a bar chart when matplotlib is there) from gemm_bench.
 
-Runs rocm_wmma_gemm_amd/lib/gemm_bench with --rocblas over a list of shapes and all eight
-layouts for one type pair, and writes one table per report in the layout of the
+Runs rocm_wmma_gemm_amd/lib/gemm_bench with --rocblas --hipblaslt over a list of shapes and
+all eight layouts for one type pair, and writes one table per report in the layout of the
 reference's published tables (reference docs/gfx1100_square.md: one row per shape and
 input layout pair; this library with C column-major, rocBLAS with C column-major, their
-ratio, this library with C row-major, its ratio to the same rocBLAS figure), with one
-more column: rocBLAS for C row-major, run as the transposed problem, which the
-reference's rocBLAS wrapper does not cover.
+ratio, this library with C row-major, its ratio to the same rocBLAS figure), with more
+columns: rocBLAS for C row-major, run as the transposed problem, which the reference's
+rocBLAS wrapper does not cover, and hipBLASLt (hipblasLtMatmul with the first algorithm
+its heuristic returns) for both C layouts.  The ratio is against the faster of the two
+vendor libraries.
 
     python bench_report.py --type f16_f16 --set square --out docs/gfx950_square_f16.md
     python bench_report.py --type f32_bf16 --shapes 4096,5120,5120:8192,4096,2048 --out x.md
@@ -46,8 +48,8 @@ ROW = re.compile(r"^(\S+)\s+(\d+),(\d+),(\d+)\s+([rc]{3})\s+\S+\s+\S+\s+([\d.]+)
 
 
 def run_bench(type_pair: str, shapes: str, reps: int, batch: int = 1) -> dict:
-    """{(m, n, k): {'ours'|'rocblas': {layout 'abc': TFLOP/s}}}"""
-    cmd = [BENCH, "--type", type_pair, "--shapes", shapes, "--layouts", "all", "--rocblas",
+    """{(m, n, k): {'ours'|'rocblas'|'hipblaslt': {layout 'abc': TFLOP/s}}}"""
+    cmd = [BENCH, "--type", type_pair, "--shapes", shapes, "--layouts", "all", "--rocblas", "--hipblaslt",
            "--reps", str(reps), "--batch_count", str(batch)]
     print("running:", " ".join(cmd), file=sys.stderr)
     out = subprocess.run(cmd, capture_output=True, text=True, check=True, timeout=1800).stdout
@@ -56,9 +58,9 @@ def run_bench(type_pair: str, shapes: str, reps: int, batch: int = 1) -> dict:
         m = ROW.match(line)
         if not m:
             continue
-        who = "rocblas" if m.group(1) == "rocblas" else "ours"
+        who = m.group(1) if m.group(1) in ("rocblas", "hipblaslt") else "ours"
         key = tuple(int(x) for x in m.group(2, 3, 4))
-        res.setdefault(key, {"ours": {}, "rocblas": {}})[who][m.group(5)] = float(m.group(8))
+        res.setdefault(key, {"ours": {}, "rocblas": {}, "hipblaslt": {}})[who][m.group(5)] = float(m.group(8))
     return res
 
 
@@ -76,17 +78,19 @@ def table(res: dict, type_pair: str) -> list[str]:
     name = {"r": "row", "c": "col"}
     lines = [
         f"## {TITLES[type_pair]}\n",
-        "| Matrix Size | Input Layout (A,B) | this library<br>(C=col) | rocBLAS<br>(C=col) | Ratio<br>(C=col) "
-        "| this library<br>(C=row) | rocBLAS<br>(C=row) | Ratio<br>(C=row) |",
-        "|:---|:---|---:|---:|---:|---:|---:|---:|",
+        "| Matrix Size | Input Layout (A,B) | this library<br>(C=col) | rocBLAS<br>(C=col) | hipBLASLt<br>(C=col) "
+        "| Ratio<br>(C=col) | this library<br>(C=row) | rocBLAS<br>(C=row) | hipBLASLt<br>(C=row) | Ratio<br>(C=row) |",
+        "|:---|:---|---:|---:|---:|---:|---:|---:|---:|---:|",
     ]
     for (m, n, k), r in res.items():
         for ab in ("cc", "rc", "cr", "rr"):
             cells = []
             for c in ("c", "r"):
-                ours, blas = r["ours"].get(ab + c), r["rocblas"].get(ab + c)
-                ratio = f"{ours / blas:.2f}" if ours and blas else "-"
-                cells += [f"{ours:.1f}" if ours else "-", f"{blas:.1f}" if blas else "-", ratio]
+                ours, blas, lt = r["ours"].get(ab + c), r["rocblas"].get(ab + c), r["hipblaslt"].get(ab + c)
+                vendor = max([x for x in (blas, lt) if x], default=None)
+                ratio = f"{ours / vendor:.2f}" if ours and vendor else "-"
+                cells += [f"{ours:.1f}" if ours else "-", f"{blas:.1f}" if blas else "-",
+                          f"{lt:.1f}" if lt else "-", ratio]
             lines.append(f"| {m}x{n}x{k} | {name[ab[0]]}, {name[ab[1]]} | " + " | ".join(cells) + " |")
     return lines
 
@@ -98,19 +102,21 @@ def chart(res: dict, type_pair: str, path: str) -> bool:
         import matplotlib.pyplot as plt
     except ImportError:
         return False
-    labels, ours, blas = [], [], []
+    labels, ours, blas, lt = [], [], [], []
     for (m, n, k), r in res.items():
         for lay in ("rcr", "rrr", "crr", "ccr"):
             if lay in r["ours"] and lay in r["rocblas"]:
                 labels.append(f"{m}x{n}x{k}\n{lay}")
                 ours.append(r["ours"][lay])
                 blas.append(r["rocblas"][lay])
+                lt.append(r["hipblaslt"].get(lay, 0.0))
     if not labels:
         return False
     fig, ax = plt.subplots(figsize=(max(8, 0.45 * len(labels)), 5))
     x = range(len(labels))
-    ax.bar([i - 0.2 for i in x], ours, 0.4, label="this library")
-    ax.bar([i + 0.2 for i in x], blas, 0.4, label="rocBLAS")
+    ax.bar([i - 0.27 for i in x], ours, 0.27, label="this library")
+    ax.bar([i for i in x], blas, 0.27, label="rocBLAS")
+    ax.bar([i + 0.27 for i in x], lt, 0.27, label="hipBLASLt")
     ax.set_xticks(list(x))
     ax.set_xticklabels(labels, fontsize=6, rotation=90)
     ax.set_ylabel("TFLOP/s")
@@ -141,7 +147,7 @@ def main(argv=None) -> int:
              "projection": "Transformer projection shapes",
              "batched": f"Strided batches of {batch} small problems"}.get(a.set, "Selected shapes")
     flops = "2·M·N·K" if batch == 1 else f"{batch}·2·M·N·K"
-    lines = [f"# {title}: this library and rocBLAS on one MI355X\n",
+    lines = [f"# {title}: this library, rocBLAS and hipBLASLt on one MI355X\n",
              f"TFLOP/s = {flops} / median of {a.reps} event-timed launches, seeded random operands; "
              f"{device_line()}.",
              "Produced by `rocm_wmma_gemm_amd/csrc/tools/bench_report.py` "

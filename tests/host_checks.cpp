@@ -1,6 +1,7 @@
 // Host-only checks of the pieces of the library that need no GPU: the tile map
 // (compiled here for the CPU) and the config selection functions.
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <set>
 #include <utility>
@@ -154,6 +155,20 @@ static int check_select()
         return fail("model: 304 x 4096 x 4096 wants a split");
     if(!model_plan(1024, 1024, 65536, 0, 0, 1, &p) || p.split_k == 1)
         return fail("model: long K wants a split");
+    // decode-like shapes with both operands K-contiguous: the whole-K streaming kernel, 64
+    // rows of the large operand per workgroup, also when a column-major C swaps the operands
+    if(!model_plan(32, 8192, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline != 7 || tiles[p.variant].bm != 32
+       || tiles[p.variant].bn != 64 || p.split_k != 1)
+        return fail("model: skinny M streams");
+    if(!model_plan(32, 8192, 8192, 1, 0, 1, &p) || tiles[p.variant].pipeline != 7 || tiles[p.variant].bm != 64
+       || tiles[p.variant].bn != 32)
+        return fail("model: skinny M under a column-major C streams as skinny N");
+    if(!model_plan(32, 8192, 8192, 0, 0, 0, &p) || tiles[p.variant].pipeline != 7 || tiles[p.variant].bn != 64)
+        return fail("model: weights stored K x N stream on the 64-wide side");
+    if(!model_plan(32, 8192, 8192, 0, 1, 1, &p) || tiles[p.variant].pipeline == 7)
+        return fail("model: the streaming kernel needs the small operand K-contiguous");
+    if(!model_plan(128, 8192, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline == 7)
+        return fail("model: 128 rows stay with split-K");
     // 272 tiles of 256 x 256: the last wave of 16 tiles split
     if(!model_plan(4352, 4096, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline != 5 || p.split_k >= -1)
         return fail("model: tail split");
@@ -172,6 +187,16 @@ static int check_select()
     // ... but an odd K is fine when no operand is K-contiguous (A column-major, B row-major)
     if(!model_plan(4096, 4096, 1001, 0, 1, 0, &p) || tiles[p.variant].pipeline != 5)
         return fail("model: odd K, no K-contiguous operand");
+    // another compute-unit count (a partitioned GPU): what fills 256 units in one pass takes
+    // passes on fewer, and a shape with too few tiles for 256 has enough for 64
+    if(!model_plan(4096, 4096, 4096, 0, 0, 1, &p, 1, 64) || tiles[p.variant].pipeline != 5 || p.split_k != 1)
+        return fail("model: 4096^3 on 64 compute units is four whole passes");
+    if(!model_plan(2048, 2048, 8192, 0, 0, 1, &p, 1, 256) || tiles[p.variant].bm != 128 || tiles[p.variant].bn != 128)
+        return fail("model: 2048 x 2048 on 256 compute units takes the tile that gives 256 tiles");
+    if(!model_plan(2048, 2048, 8192, 0, 0, 1, &p, 1, 32) || tiles[p.variant].bm != 256 || p.split_k != 1)
+        return fail("model: 2048 x 2048 on 32 compute units takes the large tile, two whole passes");
+    if(model_measured.compute_units != 256 || model_measured.step_count < 4)
+        return fail("model constants of the generated header");
     std::printf("select ok\n");
     return 0;
 }
@@ -225,10 +250,42 @@ static int check_workspace()
     return 0;
 }
 
+// The model's plan for one problem, for tests that compare it with measurements:
+//   host_checks model M N K lc la lb [batch [compute units]]
+// prints "variant swizzle split touch block_m block_n block_k waves_m waves_n pipeline", or "none".
+static int print_model(int argc, char** argv)
+{
+    if(argc < 8)
+        return 2;
+    struct tile { int bm, bn, bk, wm, wn, pipeline; };
+#define RWG_VARIANT(IDX, BM, BN, BK, WM, WN, PIPE) {BM, BN, BK, WM, WN, PIPE},
+    const tile tiles[] = {
+#include "variants.def"
+    };
+#undef RWG_VARIANT
+    const size_t m = std::strtoull(argv[2], nullptr, 10), n = std::strtoull(argv[3], nullptr, 10),
+                 k = std::strtoull(argv[4], nullptr, 10);
+    const int    lc = std::atoi(argv[5]), la = std::atoi(argv[6]), lb = std::atoi(argv[7]);
+    const size_t batch = argc > 8 ? std::strtoull(argv[8], nullptr, 10) : 1;
+    const size_t cus   = argc > 9 ? std::strtoull(argv[9], nullptr, 10) : 0;
+    launch_plan  p;
+    if(!model_plan(m, n, k, lc, la, lb, &p, batch, cus))
+    {
+        std::printf("none\n");
+        return 0;
+    }
+    const tile& t = tiles[p.variant];
+    std::printf("%d %d %d %d %d %d %d %d %d %d\n", p.variant, p.swizzle, p.split_k, p.touch, t.bm, t.bn, t.bk, t.wm,
+                t.wn, t.pipeline);
+    return 0;
+}
+
 int main(int argc, char** argv)
 {
     if(argc < 2)
         return 2;
+    if(!std::strcmp(argv[1], "model"))
+        return print_model(argc, argv);
     if(!std::strcmp(argv[1], "tilemap"))
         return check_tilemap();
     if(!std::strcmp(argv[1], "xcd"))

@@ -287,7 +287,7 @@ def test_every_variant_and_split_k_agree_with_oracle(loader):
                     for tname in ("f16_f16", "f32_bf16"):
                         din, dout = TYPE_PAIRS[tname]
                         A, B = make_inputs(M, N, K, la, lb, din, seed_a=7, seed_b=8)
-                        if not built_for(v, lc, la, lb):
+                        if not built_for(v, lc, la, lb, K, M, N):
                             dA, dB = to_device(A, din), to_device(B, din)
                             dC = to_device(np.zeros(M * N, dtype=A.dtype if dout != O.F32 else np.float32), dout)
                             assert loader.run_variant(v.index, 4, split_k, dC, dA, dB, M, N, K,
@@ -301,6 +301,63 @@ def test_every_variant_and_split_k_agree_with_oracle(loader):
                             raise AssertionError(
                                 f"variant {v.index} split_k {split_k} {M}x{N}x{K} layouts "
                                 f"C{lc} A{la} B{lb} {tname}: {e}") from None
+
+
+def test_whole_k_streaming_kernel_agrees_with_oracle(loader):
+    """The kernel for skinny shapes (pipeline 7: tiles of 32 or 64, one workgroup per tile
+    over the whole K, ring of up to 8 stages): every tile, skinny M and skinny N (a
+    column-major C runs as the transposed problem), the large operand K-contiguous or
+    contiguous along N, ragged M and N (rows past the edge are read as zeros and not
+    stored), one stage and many, a strided batch, all type pairs, and -1 for what it does
+    not take (two operands that are not K-contiguous, one on a 32-wide side of the tile,
+    K no multiple of 128)."""
+    import torch
+
+    stream = [v for v in loader.variants() if v.pipeline == 7]
+    assert {(v.block_m, v.block_n) for v in stream} == {(32, 32), (64, 32), (32, 64), (64, 64)}
+    shapes = [(16, 2048, 1024), (100, 1000, 384), (128, 512, 128), (33, 65, 2048), (2048, 24, 512)]
+    ran = set()
+    for v in stream:
+        for (M, N, K) in shapes:
+            # both operands K-contiguous, then the large operand contiguous along N (weights
+            # stored K x N), each with C row- and column-major
+            for (lc, la, lb) in [(0, 0, 1), (1, 0, 1), (0, 0, 0), (1, 0, 0), (0, 1, 1)]:
+                for tname in TYPE_PAIRS:
+                    din, dout = TYPE_PAIRS[tname]
+                    A, B = make_inputs(M, N, K, la, lb, din, seed_a=3, seed_b=4)
+                    if not built_for(v, lc, la, lb, K, M, N):
+                        dA, dB = to_device(A, din), to_device(B, din)
+                        dC = torch.zeros(M * N, dtype=torch_dtype(dout), device="cuda")
+                        assert loader.run_variant(v.index, 1, 1, dC, dA, dB, M, N, K, lc, la, lb) == -1, (
+                            v.index, M, N, K, lc, la, lb)
+                        continue
+                    ran.add((v.block_m, v.block_n, lc, la, lb))
+                    gpu = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout, variant=(v.index, 1, 1))
+                    try:
+                        check_against_oracle(gpu, A, B, M, N, K, lc, la, lb, din, dout)
+                    except AssertionError as e:
+                        raise AssertionError(f"variant {v.index} {M}x{N}x{K} C{lc} A{la} B{lb} {tname}: {e}") from None
+    # every tile ran with both operands K-contiguous; the 64-wide sides also took the other layout
+    assert {(bm, bn) for (bm, bn, lc, la, lb) in ran if (la, lb) == (0, 1)} == {(32, 32), (64, 32), (32, 64), (64, 64)}
+    assert (32, 64, 0, 0, 0) in ran and (64, 32, 1, 0, 0) in ran and (64, 64, 0, 0, 0) in ran
+    assert not any((la, lb) == (1, 1) and lc == 0 and bm != 64 for (bm, bn, lc, la, lb) in ran)
+    # a strided batch, and bit-identical repeats
+    v = stream[0]
+    M, N, K, batch = 48, 320, 640, 3
+    As = [O.init_matrix(M, K, 0, O.F16, seed=1 + b) for b in range(batch)]
+    Bs = [O.init_matrix(K, N, 1, O.F16, seed=9 + b) for b in range(batch)]
+    gpu = run_gpu(loader, np.concatenate(As), np.concatenate(Bs), M, N, K, 0, 0, 1, O.F16, O.F32, batch=batch,
+                  variant=(v.index, 1, 1))
+    again = run_gpu(loader, np.concatenate(As), np.concatenate(Bs), M, N, K, 0, 0, 1, O.F16, O.F32, batch=batch,
+                    variant=(v.index, 1, 1))
+    assert np.array_equal(gpu, again)
+    for b in range(batch):
+        check_against_oracle(gpu[b * M * N:(b + 1) * M * N], As[b], Bs[b], M, N, K, 0, 0, 1, O.F16, O.F32)
+    # what it does not take
+    dA = torch.zeros(64 * 256, dtype=torch.float16, device="cuda")
+    dC = torch.zeros(64 * 64, dtype=torch.float16, device="cuda")
+    assert loader.run_variant(v.index, 1, 1, dC, dA, dA, 64, 64, 256, 0, 1, 0) == -1   # neither operand K-contiguous
+    assert loader.run_variant(v.index, 1, 1, dC, dA, dA, 64, 64, 200, 0, 0, 1) == -1   # K % 128 != 0
 
 
 def test_split_tail_wave_agrees_with_oracle(loader):
@@ -583,7 +640,7 @@ def test_two_streams_share_the_scratch_memory(loader):
     import torch
 
     cases = [  # (M, N, K, lc, la, lb): split-K (skinny, long K) and padded copies (odd K)
-        (64, 8192, 8192, 0, 0, 1),
+        (64, 8192, 8192, 0, 1, 0),
         (1024, 1024, 16384, 0, 0, 1),
         (128, 8192, 8192, 1, 0, 0),
         (1025, 1031, 2049, 0, 0, 1),
@@ -617,7 +674,7 @@ def test_two_host_threads_each_on_its_own_stream(loader):
 
     import torch
 
-    cases = [(64, 8192, 8192, 0, 0, 1), (1025, 1031, 2049, 0, 0, 1), (512, 768, 1024, 0, 0, 1)]
+    cases = [(64, 8192, 8192, 0, 1, 0), (1025, 1031, 2049, 0, 0, 1), (512, 768, 1024, 0, 0, 1)]
     dev = []
     for (M, N, K, lc, la, lb) in cases:
         A, B = make_inputs(M, N, K, la, lb, O.F16)
@@ -664,7 +721,8 @@ def test_scratch_buffer_outlives_a_graph_that_holds_its_address(loader):
     import torch
 
     assert loader.workspace_release() == 0, "run before any other test that captures a graph"
-    M, N, K, lc, la, lb = 64, 8192, 8192, 0, 0, 1
+    M, N, K, lc, la, lb = 64, 8192, 8192, 0, 1, 0  # (a split-K plan: partial planes in the buffer)
+    assert loader.select(M, N, K, 1, lc, la, lb)[2] > 1
     A, B = make_inputs(M, N, K, la, lb, O.F16)
     dA, dB = to_device(A, O.F16), to_device(B, O.F16)
     want = torch.zeros(M * N, dtype=torch.float32, device="cuda")
@@ -720,7 +778,7 @@ def test_replays_from_a_hip_graph(loader):
     the eager results on every replay, with eager work and synchronisations in between."""
     import torch
 
-    cases = [(512, 768, 1024, 0, 0, 1), (1000, 1000, 1000, 0, 1, 0), (64, 8192, 8192, 0, 0, 1)]
+    cases = [(512, 768, 1024, 0, 0, 1), (1000, 1000, 1000, 0, 1, 0), (64, 8192, 8192, 0, 1, 0)]
     ops = []
     for (M, N, K, lc, la, lb) in cases:
         A, B = make_inputs(M, N, K, la, lb, O.F16)

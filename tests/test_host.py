@@ -52,7 +52,8 @@ def test_loader_mirror_opens_named_arch_and_lists_variants(built_library):
     for v in vs:
         assert v.block_m == v.warps_m * v.warp_tile_m * 32
         assert v.block_n == v.warps_n * v.warp_tile_n * 32
-        assert v.threads == 64 * v.warps_m * v.warps_n
+        # (the whole-K streaming kernel always runs four waves, which split K)
+        assert v.threads == (256 if v.pipeline == 7 else 64 * v.warps_m * v.warps_n)
         assert v.lds_bytes <= 160 * 1024
 
 
@@ -287,7 +288,10 @@ def test_shipped_json_matches_reference_schema():
     doc = json.load(open(os.path.join(cfg_dir, "gemm_config_gfx950_f16.json")))
     assert doc["configurations"]
     for conf in doc["configurations"]:
-        assert set(conf) == {"range", "layout", "config"}
+        # the reference's three keys (its reader takes nothing else from an entry), and
+        # optionally the type pair the entry was timed on
+        assert {"range", "layout", "config"} <= set(conf) <= {"range", "layout", "config", "timed_on"}
+        assert conf.get("timed_on", "f16_f16") in ("f16_f16", "f32_f16", "bf16_bf16", "f32_bf16")
         assert set(conf["range"]) == {"M", "N", "K"}
         assert set(conf["layout"]) == {"A", "B", "C"}
         assert all(v in ("row_major", "col_major") for v in conf["layout"].values())
@@ -557,3 +561,71 @@ def test_tuner_adopts_new_tuples_into_the_variant_list(tmp_path):
     after = G.read_variants(str(copy))  # still dense and parseable
     assert len(after) == len(before) + 1 and after[-1]["block_k"] == 32
     assert T.adopt([T.Tile(128, 256, 32, 2, 2, 1)], path=str(copy)) == []
+
+
+# ---------------------------------------------------------------- the dispatcher's model against measurements
+MODEL_LOG = os.path.join(ROOT, "tests", "golden", "tuner_log_gfx950_f16.json")
+# What the model is held to on the problems of the fixture (an exhaustive tuner sweep on an
+# MI355X, fp16, regular shapes from 2048^3 to 8192^3 and projections, three layouts each):
+MODEL_WORST_REGRET = 1.12  # its pick is never more than this factor slower than the best timing (measured: 1.07)
+MODEL_MEAN_REGRET = 1.03   # and on average within this factor (measured: 1.012)
+
+
+def _fit_module():
+    sys.path.insert(0, os.path.join(ROOT, "rocm_wmma_gemm_amd", "config"))
+    import fit_model
+
+    return fit_model
+
+
+def test_model_pick_is_within_its_stated_regret_of_the_measured_best(host_tool):
+    """Ties the dispatcher's constants to measurements: for every problem of the recorded
+    tuner sweep, the plan model_plan picks (through the same compiled code the library
+    uses) is looked up among the sweep's timings and compared with the best of them."""
+    import json
+
+    F = _fit_module()
+    table = json.load(open(MODEL_LOG))
+    regrets = {}
+    for problem, cands in table.items():
+        shape, lay, _ = problem.split(" ")
+        M, N, K = shape.split(",")
+        la, lb, lc = ("rc".index(ch) for ch in lay)
+        r = subprocess.run([host_tool, "model", M, N, K, str(lc), str(la), str(lb)], capture_output=True, text=True)
+        assert r.returncode == 0, r.stdout + r.stderr
+        if r.stdout.strip() == "none":
+            continue
+        variant, sw, sk, touch, bm, bn, bk, wm, wn, pipe = (int(x) for x in r.stdout.split())
+        # the model leaves the band height at 4; the sweep timed 4, 8, 16, -4, -8 (1 for few tiles)
+        keys = [F.candidate_key(pipe, bm, bn, bk, wm, wn, s, sk, touch) for s in (sw, 1)]
+        ms = next((cands[k] for k in keys if k in cands), None)
+        if ms is None:
+            continue  # a split the sweep's candidate rules did not include
+        regrets[problem] = ms / min(cands.values())
+    assert len(regrets) >= 30, f"only {len(regrets)} problems of the sweep could be compared"
+    worst = max(regrets, key=regrets.get)
+    mean = sum(regrets.values()) / len(regrets)
+    assert regrets[worst] <= MODEL_WORST_REGRET, (worst, regrets[worst])
+    assert mean <= MODEL_MEAN_REGRET, mean
+
+
+def test_model_constants_are_what_a_fit_of_the_recorded_sweep_gives():
+    """config/fit_model.py on the recorded sweep reproduces the shipped step costs: a retune
+    that changes kernel speed shows up here unless the constants are fitted again."""
+    import json
+
+    F = _fit_module()
+    model = json.load(open(os.path.join(ROOT, "rocm_wmma_gemm_amd", "config", "model_gfx950.json")))
+    records = F.expand(json.load(open(MODEL_LOG)))
+    assert records and F.expand(F.compact(records)) == records
+    fitted = F.fit(records, model)
+    compared = 0
+    for pipe, tiles in fitted["step_us"].items():
+        for tile, us in tiles.items():
+            if tile in model["step_us"].get(pipe, {}):
+                assert abs(us - model["step_us"][pipe][tile]) <= 0.15 * model["step_us"][pipe][tile], (pipe, tile, us)
+                compared += 1
+    assert compared >= 4
+    # the log format of tune.py --log parses
+    line = "4096,4096,4096 rcr f16_f16 p5 256x256x64 w2x2 sw4 sk1 touch0 compiled 0.0981 ms 1401.0 TFLOP/s"
+    assert F.parse([line]) == [(4096, 4096, 4096, "rcr", "f16_f16", 5, 256, 256, 64, 2, 2, 4, 1, 0, 0.0981)]

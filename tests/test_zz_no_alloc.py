@@ -44,7 +44,7 @@ def test_noalloc_entry_point_matches_the_ordinary_one_on_calls_in_a_row(loader):
 
     cases = [  # the first is the largest user of the scratch array, the rest are smaller
         (128, 8192, 8192, 0, 0, 1, "f32_f16", 1),    # split-K: fp32 partial planes
-        (64, 4096, 4096, 1, 0, 0, "f16_f16", 1),     # split-K, fewer and smaller planes
+        (64, 4096, 4096, 1, 1, 0, "f16_f16", 1),     # split-K, fewer and smaller planes
         (1025, 1031, 2049, 0, 0, 1, "bf16_bf16", 1),  # ragged: padded copies (and partial tiles)
         (16, 2048, 1024, 0, 1, 1, "f32_bf16", 3),    # small batched split
         (512, 768, 1024, 0, 0, 1, "f16_f16", 1),     # whole tiles: no scratch memory at all
@@ -79,5 +79,5 @@ def test_noalloc_entry_point_rejects_what_its_scratch_array_cannot_hold(loader):
     assert loader._lib.rocm_wmma_gemm_noalloc(7, 0, 0, 0, 16, 16, 16, 1, 0, 0, 0, None) == RL.ERR_ARGUMENT
     assert loader._lib.rocm_wmma_gemm_noalloc(0, 0, 0, 0, 16, 16, 16, 1, 0, 2, 0, None) == RL.ERR_ARGUMENT
     # and the array still serves the next call
-    rc, want, got, _, _ = _both_ways(loader, 64, 8192, 8192, 0, 0, 1, "f32_f16")
+    rc, want, got, _, _ = _both_ways(loader, 64, 8192, 8192, 0, 1, 0, "f32_f16")
     assert rc == RL.OK and torch.equal(got, want)
