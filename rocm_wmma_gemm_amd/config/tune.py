@@ -176,7 +176,7 @@ def tile_feasible(t: Tile, a_kmajor: bool, b_kmajor: bool) -> bool:
     if t.pipeline in (3, 6):
         return t.block_k == 64
     if t.pipeline == 5:
-        return (t.warps_m, t.warps_n) == (2, 2) and t.block_k == 64 and t.block_m in (192, 256) \
+        return (t.warps_m, t.warps_n) == (2, 2) and t.block_k in (32, 64) and t.block_m in (192, 256) \
             and t.block_n in (192, 256)
     return True
 

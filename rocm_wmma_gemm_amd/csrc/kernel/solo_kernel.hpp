@@ -24,6 +24,17 @@
 // about 70 in the wait and the barrier, where issuing a tile's loads back to back
 // had cost 1700-1900 cycles for the second step.
 //
+// The same kernel with BLOCK_K 32 keeps a ring of 4 tiles of one MFMA K step each (the
+// same 128 KB of LDS): a barrier per K step, and the loads of tile t+4 go out under tile
+// t, so a load has two to three tile times to land instead of a quarter to one.  Built to
+// see whether the fall of the rate for K-contiguous operands that no longer fit the 256 MB
+// memory-side cache (8192 x 8192 x 28672: 1250 TFLOP/s against 1540 at K = 8192) is a
+// matter of load latency.  It is not: the ring of 4 runs 1236 there, and 5..13 % below the
+// ring of 2 where the operands stay in that cache (the second barrier, and the 64-byte
+// half lines a K-contiguous row of 32 fetches).  What the counters show instead for those
+// shapes is the texture addresser stalled by the L1 four times as often as in the vendor's
+// kernel of the same tile, and L2 misses that take 850 cycles against 620.
+//
 // A launch has one workgroup per CU; each works through its tiles (or K slices, or a
 // range of K tiles: see walk) with one load stream running through all of them, and
 // stores C through per-wave LDS strips as 16-byte buffer stores.  Loads and stores go
@@ -37,6 +48,20 @@
 #include <utility>
 
 #include "direct_kernel.hpp"
+
+// Schedule constants of the K loop, as macros so that the tuner's run-time compile
+// (kernel_jit.hip) can try others: a fragment read after every RWG_SOLO_FRAG_GAP-th MFMA;
+// RWG_SOLO_LATE_LOADS_16THS sixteenths of a tile's loads issued in the first step of the next
+// tile (one every RWG_SOLO_LATE_GAP MFMAs), the rest under the second step of this one.
+#ifndef RWG_SOLO_FRAG_GAP
+#define RWG_SOLO_FRAG_GAP 2
+#endif
+#ifndef RWG_SOLO_LATE_LOADS_16THS
+#define RWG_SOLO_LATE_LOADS_16THS 4
+#endif
+#ifndef RWG_SOLO_LATE_GAP
+#define RWG_SOLO_LATE_GAP 4
+#endif
 
 namespace rocm_wmma_gemm
 {
@@ -84,8 +109,8 @@ struct solo_gemm
     static constexpr int B_BYTES   = BN * BK * 2;
     static constexpr int STAGE     = A_BYTES + B_BYTES;
     static constexpr int LDS_BYTES = STAGES * STAGE;
-    static_assert(BK == 64 && STAGES == 2, "ring of 2 tiles of BLOCK_K 64");
-    
+    static_assert((BK == 64 && STAGES == 2) || (BK == 32 && STAGES == 4),
+                  "ring of 2 tiles of BLOCK_K 64, or of 4 tiles of BLOCK_K 32");
 
     using op_a = direct_operand<A_KMAJOR, BM, BK, WTM, WAVES, MI>;
     using op_b = direct_operand<B_KMAJOR, BN, BK, WTN, WAVES, MI>;
@@ -96,7 +121,7 @@ struct solo_gemm
     static constexpr int KK    = BK / 32; // MFMA K steps per tile
     static constexpr int FRAGS = TM + TN;
     // Fragment u (A fragments first, then B) is read after MFMA u * FRAG_GAP.
-    static constexpr int FRAG_GAP = 2;
+    static constexpr int FRAG_GAP = RWG_SOLO_FRAG_GAP;
     static_assert(FRAGS * FRAG_GAP <= MFMAS, "fragment reads must fit under the MFMAs of a step");
 
     // s_waitcnt immediate: lgkmcnt(0), expcnt untouched, vmcnt(n)
@@ -116,12 +141,14 @@ struct solo_gemm
     // sits in the buffer descriptor (scalar registers, advanced once per tile), the
     // part that depends on i is a scalar offset i * stride, and the lane's own part is
     // a vector offset that is the same for every i (K-contiguous: the swizzle of row
-    // 8*(wave + 4i) + lane/8 does not depend on i) or alternates between two values
+    // RPL*(wave + 4i) + lane/CH does not depend on i) or alternates between two values
     // with the parity of i (M/N-contiguous: the swizzle term 2*((kg/2)%2) does).
     template<bool KMAJOR, int ROWS>
     struct load_addr
     {
-        static_assert(WAVES == 4 && BK == 64 && (KMAJOR || ROWS == 256), "derived for this tile and wave count");
+        static_assert(WAVES == 4 && (KMAJOR || ROWS == 256), "derived for this tile and wave count");
+        static constexpr int CH  = BK / 8; // 16-byte chunks of a K-contiguous row
+        static constexpr int RPL = 64 / CH; // rows of it that one load fills
         unsigned int voff[KMAJOR ? 1 : 2]; // bytes
         unsigned int stride; // bytes between load i and load i+1
 
@@ -129,11 +156,10 @@ struct solo_gemm
         {
             if constexpr(KMAJOR)
             {
-                constexpr int CH   = BK / 8;
-                const int     r    = 8 * wave + lane / CH; // row of load 0; load i adds 32 rows
-                const int     c    = (lane % CH) ^ swizzle_of_row<CH, MI>(r);
-                voff[0]            = (unsigned int)((r * ld + c * 8) * 2);
-                stride             = (unsigned int)(32 * ld * 2);
+                const int r = RPL * wave + lane / CH; // row of load 0; load i adds WAVES * RPL rows
+                const int c = (lane % CH) ^ swizzle_of_row<CH, MI>(r);
+                voff[0]     = (unsigned int)((r * ld + c * 8) * 2);
+                stride      = (unsigned int)(WAVES * RPL * ld * 2);
             }
             else
             {
@@ -166,10 +192,9 @@ struct solo_gemm
             load_addr t = *this;
             if constexpr(KMAJOR)
             {
-                constexpr int CH = BK / 8;
-                const int     r  = 8 * wave + lane / CH;
-                const int     c  = (lane % CH) ^ swizzle_of_row<CH, MI>(r);
-                t.voff[0]        = c * 8 < kt ? voff[0] : RANGE_MAX;
+                const int r = RPL * wave + lane / CH;
+                const int c = (lane % CH) ^ swizzle_of_row<CH, MI>(r);
+                t.voff[0]   = c * 8 < kt ? voff[0] : RANGE_MAX;
             }
             return t;
         }
@@ -848,20 +873,106 @@ struct solo_gemm
         // whether the tile at (a_src, b_src) is a last K tile held only in part
         auto partial_tile = [&]() { return k_ragged && stream_ends && stream_left == 1; };
 
+        const unsigned int lds_addr   = (unsigned int)(size_t)lds;
+        const unsigned int wave_block = lds_addr + wave * 1024; // this wave's block 0, stage 0
+        lds_char_ptr       strip      = lds + LDS_BYTES + wave * STRIP_BYTES;
+        u32x4 fa[2][TM], fb[2][TN];
+
+        if constexpr(STAGES == 4)
+        {
+            // Ring of 4 tiles of one K step each.  The fragments of tile t+1 are read under
+            // the MFMAs of tile t, so tile t's stage is free when all waves have arrived at
+            // the barrier in front of tile t, and the loads of tile t+4 go out under tile t:
+            // a load has between two and three tiles' time to land (one quarter to one with
+            // the ring of 2), at the price of a barrier per K step instead of one per two.
+            using plan = load_plan<2, (MFMAS - 2) / VM_LOADS, 0, VM_LOADS>;
+            constexpr unsigned int RING = STAGES * STAGE;
+#pragma unroll
+            for(int s = 0; s < STAGES; ++s)
+            {
+                const bool part = partial_tile();
+                issue_loads(std::make_integer_sequence<int, VM_LOADS>{}, la.or_else(part, la_tail),
+                            lb.or_else(part, lb_tail), wave_block + s * STAGE, descriptor(a_src, a_end),
+                            descriptor(b_src, b_end));
+                advance();
+            }
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(3 * VM_LOADS));
+            __builtin_amdgcn_s_barrier();
+            read_first(std::make_integer_sequence<int, TM>{}, std::make_integer_sequence<int, TN>{},
+                       oa, ob, lds_addr, fa[0], fb[0]);
+
+            unsigned int here = 0; // stage (byte offset) of the tile the MFMAs are on
+            // One tile: wait for the own loads of the next tile (the loads of the two tiles
+            // behind it stay in flight) and the own fragment reads of this one, barrier, then
+            // the MFMAs with the next tile's fragment reads and the loads of the tile four on.
+            auto tile_step = [&](const u32x4 (&ca)[TM], const u32x4 (&cb)[TN], u32x4 (&na)[TM], u32x4 (&nb)[TN],
+                                 f32x4 (&acc)[TM][TN]) {
+                const unsigned int there = here + STAGE == RING ? 0 : here + STAGE;
+                const bool         part  = partial_tile();
+                const addr_a       la1   = la.or_else(part, la_tail);
+                const addr_b       lb1   = lb.or_else(part, lb_tail);
+                const step_ctx     c{oa, ob, la1, lb1, lds_addr + there, wave_block + here,
+                                     descriptor(a_src, a_end), descriptor(b_src, b_end)};
+                __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * VM_LOADS));
+                __builtin_amdgcn_s_barrier();
+                step<0, plan>(c, ca, cb, na, nb, acc);
+                advance();
+                here = there;
+            };
+            for(;;)
+            {
+                f32x4 acc[TM][TN];
+#pragma unroll
+                for(int i = 0; i < TM; ++i)
+                {
+#pragma unroll
+                    for(int j = 0; j < TN; ++j)
+                    {
+                        acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                    }
+                }
+#pragma unroll
+                for(int i = 0; i < TM; ++i)
+                {
+                    settle_row(acc[i]);
+                }
+                for(int it = 0;;)
+                {
+                    tile_step(fa[0], fb[0], fa[1], fb[1], acc);
+                    if(++it == cur.nk)
+                    {
+                        break;
+                    }
+                    tile_step(fa[1], fb[1], fa[0], fb[0], acc);
+                    if(++it == cur.nk)
+                    {
+                        break;
+                    }
+                }
+                // (the fragments read under the last step belong to the next item; they are
+                // read again behind the stores, which need the registers)
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+                write_item(args, cur, acc, wave_m * WTM, wave_n * WTN, lane, strip);
+                if(cur.next >= wk.end)
+                {
+                    break;
+                }
+                cur = decode(args, wk, cur.next);
+                read_first(std::make_integer_sequence<int, TM>{}, std::make_integer_sequence<int, TN>{},
+                           oa, ob, lds_addr + here, fa[0], fb[0]);
+            }
+        }
+        else
+        {
         // Ring of 2 tiles, two K steps per tile.  Tile t: first step on K step 0 with
         // the reads of K step 1; then wait for the own loads of tile t+1 and the own
         // reads of tile t, barrier; second step on K step 1 with the reads of tile
         // t+1's K step 0.  Tile t's stage is free from that barrier on: the loads of
         // tile t+2 go out under the second step (three quarters of them) and the
         // first quarter of tile t+1's first step.
-        constexpr int LOADS_A = VM_LOADS / 4, LOADS_B = VM_LOADS - LOADS_A;
+        constexpr int LOADS_A = VM_LOADS * RWG_SOLO_LATE_LOADS_16THS / 16, LOADS_B = VM_LOADS - LOADS_A;
         using plan_b = load_plan<2, (MFMAS - 2) / LOADS_B, 0, LOADS_B>;
-        using plan_a = load_plan<1, 4, LOADS_B, LOADS_A>;
-        const unsigned int lds_addr   = (unsigned int)(size_t)lds;
-        const unsigned int wave_block = lds_addr + wave * 1024; // this wave's block 0, stage 0
-        lds_char_ptr       strip      = lds + LDS_BYTES + wave * STRIP_BYTES;
-
-        u32x4 fa[2][TM], fb[2][TN];
+        using plan_a = load_plan<1, RWG_SOLO_LATE_GAP, LOADS_B, LOADS_A>;
         // prologue: tile 0 and the first part of tile 1 on their way, tile 0 landed
         {
             const bool part = partial_tile();
@@ -957,6 +1068,7 @@ struct solo_gemm
             // more live the compiler spilled accumulators to scratch memory).
             read_first(std::make_integer_sequence<int, TM>{}, std::make_integer_sequence<int, TN>{},
                        oa, ob, lds_addr + here, fa[0], fb[0]);
+        }
         }
         // the wrapped tail loads are still in flight
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
