@@ -16,6 +16,10 @@ constants of the file (launch, reduce, bytes per microsecond of partial sums and
 are kept.  compact() turns a log into the small per-problem table that the regret test of
 tests/test_host.py holds as a fixture.
 
+With --stream the log is the file written by config/sweep_stream.py, and what is fitted are
+the constants of the estimate for the plans of the whole-K streaming kernel
+(stream_estimate below, the same arithmetic as csrc/config_select.cpp: stream_plan).
+
 No counterpart in the reference, whose dispatcher has no model: it takes the nearest tuned
 shape (reference rocm_wmma_gemm/config/generate_config.py:174-234).
 """
@@ -106,13 +110,119 @@ def fit(records, model: dict) -> dict:
     return out
 
 
+STREAM_TILES = ("32x32", "64x32", "32x64", "64x64")
+
+
+def stream_estimate(c: dict, rows: int, cols: int, K: int, a_kmajor: bool, b_kmajor: bool, bm: int, bn: int,
+                    slices: int, batch: int = 1, cus: int = 256) -> float:
+    """Microseconds of one plan of the whole-K streaming kernel: launch, then per pass over
+    the compute units the fill of the ring and the workgroup's stages, each at the slower of
+    what a compute unit pulls with its ring of loads in flight and its share of the stream
+    of the large operand from memory; plus the exchange of partial tiles when several
+    workgroups share a tile.  c = the "stream" object of the model file."""
+    tiles = -(-rows // bm) * -(-cols // bn)
+    groups = tiles * slices * batch
+    passes = -(-groups // cus)
+    active = min(groups, cus)
+    stages = (K // 128) // slices
+    wide = cols >= rows  # the large operand is B
+    large_kmajor = b_kmajor if wide else a_kmajor
+    large_bytes = (bn if wide else bm) * 256
+    sharing = -(-rows // bm) if wide else -(-cols // bn)  # workgroups that read the same panel of it
+    other = (0 if a_kmajor else 1) + (0 if b_kmajor else 1)
+    per_cu = c["stage_us"][f"{bm}x{bn}"] * (1.0 + c["transposed_operand"] * other)
+    small_bytes = (bm if wide else bn) * 256  # every workgroup reads its rows of the small operand, from L2
+    from_memory = (large_bytes * (active / sharing) / (c["bytes_per_us_kmajor" if large_kmajor else "bytes_per_us_other"])
+                   + small_bytes * active / c["bytes_per_us_l2"])
+    return (c["launch_us"] + passes * (c["fill_us"] + stages * max(per_cu, from_memory))
+            + (c["exchange_us"] if slices > 1 else 0.0))
+
+
+def stream_plans(rec: dict):
+    """(tile, slices, measured us) of a sweep record."""
+    for name, us in rec["t"].items():
+        tile, slices = name.split("s")
+        yield tile, int(slices), us
+
+
+def fit_stream(records: list, start: dict) -> dict:
+    """Least squares on log(estimate / measured) over every timing of the sweep."""
+    import math
+
+    from scipy.optimize import least_squares
+
+    keys = ["launch_us", "fill_us", "exchange_us", "bytes_per_us_kmajor", "bytes_per_us_other", "bytes_per_us_l2",
+            "transposed_operand"]
+
+    def unpack(p):
+        c = {k: float(v) for k, v in zip(keys, p)}
+        c["stage_us"] = {t: float(v) for t, v in zip(STREAM_TILES, p[len(keys):])}
+        return c
+
+    rows = []
+    for r in records:
+        for tile, slices, us in stream_plans(r):
+            bm, bn = (int(x) for x in tile.split("x"))
+            rows.append((r["M"], r["N"], r["K"], r["lay"][0] == "r", r["lay"][1] == "c", bm, bn, slices, us))
+
+    def residuals(p):
+        c = unpack(p)
+        return [math.log(stream_estimate(c, *row[:8]) / row[8]) for row in rows]
+
+    p0 = [start[k] for k in keys] + [start["stage_us"][t] for t in STREAM_TILES]
+    res = least_squares(residuals, p0, bounds=([0.0] * len(p0), [20, 10, 30, 2e7, 2e7, 2e8, 3] + [2.0] * len(STREAM_TILES)))
+    c = unpack(res.x)
+    for k in ("launch_us", "fill_us", "exchange_us"):
+        c[k] = round(c[k], 2)
+    for k in ("bytes_per_us_kmajor", "bytes_per_us_other", "bytes_per_us_l2"):
+        c[k] = round(c[k], -4)
+    c["transposed_operand"] = round(c["transposed_operand"], 3)
+    c["stage_us"] = {t: round(v, 4) for t, v in c["stage_us"].items()}
+    return c
+
+
+def stream_regret(records: list, c: dict):
+    """(geometric mean, worst) of measured time of the plan the estimate picks over the
+    best measured plan, per problem of the sweep."""
+    import math
+
+    logs, worst = [], 1.0
+    for r in records:
+        plans = list(stream_plans(r))
+        if not plans:
+            continue
+        a_k, b_k = r["lay"][0] == "r", r["lay"][1] == "c"
+        pick = min(plans, key=lambda p: stream_estimate(c, r["M"], r["N"], r["K"], a_k, b_k,
+                                                        *(int(x) for x in p[0].split("x")), p[1]))
+        ratio = pick[2] / min(p[2] for p in plans)
+        logs.append(math.log(ratio))
+        worst = max(worst, ratio)
+    return math.exp(sum(logs) / len(logs)), worst
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__.splitlines()[0])
     ap.add_argument("log")
     ap.add_argument("--model", default=os.path.join(HERE, "model_gfx950.json"))
     ap.add_argument("--write", action="store_true", help="write the fitted values into --model")
     ap.add_argument("--compact", default=None, help="also write the log as a per-problem table (JSON)")
+    ap.add_argument("--stream", action="store_true",
+                    help="the log is a sweep_stream.py file: fit the streaming kernel's constants")
     a = ap.parse_args(argv)
+    if a.stream:
+        model = json.load(open(a.model))
+        records = json.load(open(a.log))
+        new = fit_stream(records, model["stream"])
+        mean, worst = stream_regret(records, new)
+        print(json.dumps(new, indent=1))
+        print(f"regret of the estimate's pick over {len(records)} problems: mean {mean:.3f}, worst {worst:.2f}")
+        if a.write:
+            new["fitted_from"] = f"{os.path.basename(a.log)}: {sum(len(r['t']) for r in records)} timings"
+            model["stream"] = new
+            with open(a.model, "w") as f:
+                json.dump(model, f, indent=4)
+                f.write("\n")
+        return 0
     records = parse(open(a.log))
     model = json.load(open(a.model))
     new = fit(records, model)

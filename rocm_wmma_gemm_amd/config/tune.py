@@ -144,9 +144,9 @@ def tile_feasible(t: Tile, a_kmajor: bool, b_kmajor: bool) -> bool:
     if t.block_m % (32 * t.warps_m) or t.block_n % (32 * t.warps_n):
         return False
     if t.pipeline == 7:
-        # whole-K streaming kernel: small tiles, stages of 128, at least one operand
-        # K-contiguous, the other on a 64-wide side of the tile
-        return ((a_kmajor or b_kmajor) and (a_kmajor or t.block_m == 64) and (b_kmajor or t.block_n == 64)
+        # whole-K streaming kernel: small tiles, stages of 128, an operand that is not
+        # K-contiguous on a 64-wide side of the tile
+        return ((a_kmajor or t.block_m == 64) and (b_kmajor or t.block_n == 64)
                 and t.block_k == 128 and t.block_m in (32, 64) and t.block_n in (32, 64)
                 and (t.warps_m, t.warps_n) == (t.block_m // 32, t.block_n // 32))
     if t.block_k == 128:
@@ -189,10 +189,15 @@ def split_feasible(t: Tile, swizzle: int, split: int, rows: int, cols: int, K: i
     if tiles <= 8 and swizzle != 1:
         return False
     if t.pipeline == 7:
-        # one workgroup per tile over the whole K: no band height, no split; worth a try
-        # when a 256 x 256 tiling leaves most compute units without a tile
-        return swizzle == (1 if tiles <= 8 else 4) and split == 1 \
-            and -(-rows // 256) * -(-cols // 256) < CUS // 2 and K % 128 == 0
+        # a workgroup per tile over the whole K, or 2, 4 or 8 that share a tile and add their
+        # parts up inside the launch (whole stages each, at least two; a counter per tile):
+        # no band height; worth a try when a 256 x 256 tiling leaves most compute units
+        # without a tile
+        stages = K // 128
+        return swizzle == (1 if tiles <= 8 else 4) and K % 128 == 0 \
+            and -(-rows // 256) * -(-cols // 256) < CUS // 2 \
+            and (split == 1 or (split in (2, 4, 8) and stages % split == 0 and stages // split >= 2
+                                and tiles <= 4096 and tiles * split <= 4 * CUS))
     if split == 1:
         return True
     if split > 1:

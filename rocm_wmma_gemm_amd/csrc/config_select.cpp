@@ -1,6 +1,8 @@
 // Implementation of the shape -> launch plan lookup (plain C++, no device code).
 #include "config_select.hpp"
 
+#include <algorithm>
+
 #include <initializer_list>
 #include <limits>
 
@@ -17,7 +19,8 @@ const model_constants    model_measured
     = {generated::model_compute_units,      generated::model_launch_us,
        generated::model_reduce_us,          generated::model_plane_bytes_per_us,
        generated::model_tile_bytes_per_us,  generated::model_copy_bytes_per_us,
-       generated::model_steps,              generated::model_step_count};
+       generated::model_steps,              generated::model_step_count,
+       generated::model_stream_constants};
 
 namespace
 {
@@ -183,36 +186,21 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
     // K need not be whole K tiles: the persistent kernel cuts a partial last tile off
     // itself, as long as the rows of a K-contiguous operand stay 16-byte aligned
     const bool k_whole = k % 64 == 0;
+    // Skinny against a large operand (decode-like: a few rows against 4096 x 4096 .. 28672
+    // x 8192): the plans of the whole-K streaming kernel compete with the others by their
+    // estimates, and stand alone for the shapes the others would only take through copies.
+    launch_plan stream_best{};
+    double      stream_us   = 0.0;
+    const bool  have_stream = stream_plan(rows, cols, k, a_kmajor, b_kmajor, batch, cus_of_device, &stream_best, &stream_us);
     if(k < 64 || rows % 8 != 0 || cols % 8 != 0 || rows < 16 || cols < 16
        || (!k_whole && (a_kmajor || b_kmajor) && k % 8 != 0))
     {
-        return false; // shapes every direct kernel would only take through padded copies
-    }
-    // Skinny against a large K-contiguous operand (decode-like: 16..64 rows against 8192 x
-    // 8192): the whole-K streaming kernel, 32 rows or columns on the skinny side and 64 on
-    // the side that streams from HBM.  Measured at N = K = 8192, fp16, one call at a time:
-    // M = 16 / 32 / 64 in 33.9 / 33.7 / 35.2 us against 39.1 / 44.9 / 39.8 us for the best
-    // split-K plan with its reduce launch; at M = 128 the split-K plan stays ahead (43.5
-    // against 47.1 us), every workgroup reading all of the small operand from L2.
-    // The operand on the skinny side must be K-contiguous; the large one may also be
-    // contiguous along its rows of the tile (weights stored K x N), on the 64-wide side.
-    if(k % 128 == 0 && k >= 2048 && batch == 1
-       && ((rows <= 64 && cols >= 2048 && a_kmajor) || (cols <= 64 && rows >= 2048 && b_kmajor)))
-    {
-        const int want_m = rows <= 64 ? 32 : 64, want_n = rows <= 64 ? 64 : 32;
-        const int count  = static_cast<int>(sizeof(model_variants) / sizeof(model_variants[0]));
-        for(int i = 0; i < count; ++i)
+        // shapes every direct kernel would only take through padded copies
+        if(have_stream)
         {
-            if(model_variants[i].pipeline == 7 && model_variants[i].block_m == want_m
-               && model_variants[i].block_n == want_n)
-            {
-                out->variant = i;
-                out->swizzle = 1;
-                out->split_k = 1;
-                out->touch   = 0;
-                return true;
-            }
+            *out = stream_best;
         }
+        return have_stream;
     }
     // (the constants are per compute unit at work, so the estimate carries over to a GPU
     // or partition with another count; the tile walk still assumes 8 XCDs)
@@ -323,6 +311,74 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
             consider(launch_us + ceil_div(tiles * kt, groups) * step + item + reduce_us
                          + groups * 1.25 * tile_bytes * 2.0 / tile_bytes_per_us,
                      -1);
+        }
+    }
+    // (between 65 and 128 rows the two families are within 20 % of each other and the two
+    // estimates are not that good: the tiled kernels keep those when they take the shape)
+    if(have_stream && (!found || (stream_us < best && std::min(rows, cols) <= 64)))
+    {
+        *out  = stream_best;
+        found = true;
+    }
+    return found;
+}
+
+bool stream_plan(size_t rows, size_t cols, size_t k, bool a_kmajor, bool b_kmajor, size_t batch, size_t cus_of_device,
+                 launch_plan* out, double* microseconds)
+{
+    if(k % 128 != 0 || k < 256 || rows == 0 || cols == 0 || (rows > 128 && cols > 128))
+    {
+        return false;
+    }
+    const model_stream& c      = model_measured.stream;
+    const size_t        cus    = cus_of_device != 0 ? cus_of_device : static_cast<size_t>(model_measured.compute_units);
+    const size_t        stages = k / 128;
+    const bool          wide   = cols >= rows; // the large operand is B
+    const int           count  = static_cast<int>(sizeof(model_variants) / sizeof(model_variants[0]));
+    bool                found  = false;
+    for(int i = 0; i < count; ++i)
+    {
+        const model_variant& v = model_variants[i];
+        if(v.pipeline != 7)
+        {
+            continue;
+        }
+        const size_t bm = v.block_m, bn = v.block_n;
+        // an operand that is not K-contiguous: 64 wide in the tile, rows of 16-byte pieces
+        if((!a_kmajor && (bm != 64 || rows % 8 != 0)) || (!b_kmajor && (bn != 64 || cols % 8 != 0)))
+        {
+            continue;
+        }
+        const int    slot    = (bm == 64 ? 1 : 0) + (bn == 64 ? 2 : 0);
+        const size_t tm      = ceil_div(rows, bm), tn = ceil_div(cols, bn), tiles = tm * tn;
+        const double other   = (a_kmajor ? 0.0 : 1.0) + (b_kmajor ? 0.0 : 1.0);
+        const double per_cu  = c.stage_us[slot] * (1.0 + c.transposed_operand * other);
+        const double large   = static_cast<double>(wide ? bn : bm) * 256.0;
+        const double small   = static_cast<double>(wide ? bm : bn) * 256.0;
+        const double sharing = static_cast<double>(wide ? tm : tn);
+        const double rate    = (wide ? b_kmajor : a_kmajor) ? c.bytes_per_us_kmajor : c.bytes_per_us_other;
+        for(size_t s = 1; s <= 8; s *= 2)
+        {
+            // (the counters of the tiles that several workgroups share: 4096 a launch)
+            if(stages % s != 0 || stages / s < 2 || (s > 1 && tiles * batch > 4096))
+            {
+                continue;
+            }
+            const size_t groups = tiles * s * batch;
+            const double active = static_cast<double>(groups < cus ? groups : cus);
+            const double stage  = std::max(per_cu, large * (active / sharing) / rate + small * active / c.bytes_per_us_l2);
+            const double t      = c.launch_us
+                             + static_cast<double>(ceil_div(groups, cus)) * (c.fill_us + static_cast<double>(stages / s) * stage)
+                             + (s > 1 ? c.exchange_us : 0.0);
+            if(!found || t < *microseconds)
+            {
+                found         = true;
+                *microseconds = t;
+                out->variant  = i;
+                out->swizzle  = 1;
+                out->split_k  = static_cast<int>(s);
+                out->touch    = 0;
+            }
         }
     }
     return found;

@@ -49,6 +49,17 @@ struct model_step
     double step_us; // per K tile of 64 with every compute unit at work
     double item_us; // per tile: the stores of C and the turn to the next tile
 };
+// Constants of the estimate for the plans of the whole-K streaming kernel (pipeline 7),
+// fitted by config/fit_model.py --stream to a sweep of config/sweep_stream.py.
+struct model_stream
+{
+    double launch_us, fill_us; // per launch; per pass over the compute units (the ring fills)
+    double exchange_us; // several workgroups per tile: the partial tiles through memory
+    double bytes_per_us_kmajor, bytes_per_us_other; // stream of the large operand from memory
+    double bytes_per_us_l2; // the small operand, which every workgroup reads from L2
+    double transposed_operand; // relative cost of a stage per operand that is not K-contiguous
+    double stage_us[4]; // per stage of 128 of one compute unit: tiles 32x32, 64x32, 32x64, 64x64
+};
 struct model_constants
 {
     int    compute_units; // of the GPU the constants were measured on
@@ -58,6 +69,7 @@ struct model_constants
     double copy_bytes_per_us; // padded operand copies
     const model_step* steps;
     int               step_count;
+    model_stream      stream;
 };
 extern const model_constants model_measured;
 
@@ -76,6 +88,11 @@ launch_plan heuristic_plan(size_t m, size_t n, size_t k, int lc);
 // cus: compute units of the GPU the plan is for (0: the GPU the constants were measured on).
 bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_plan* out, size_t batch = 1,
                 size_t cus = 0);
+// The streaming kernel's plans alone (skinny shapes: one extent at most 128, K whole stages
+// of 128), in kernel space (rows x cols, the operands' K-contiguity): the cheapest by
+// estimate and its microseconds; false when no compiled variant takes the problem.
+bool stream_plan(size_t rows, size_t cols, size_t k, bool a_kmajor, bool b_kmajor, size_t batch, size_t cus,
+                 launch_plan* out, double* microseconds);
 launch_plan select_plan_from(const tuned_entry* table, size_t count, size_t m, size_t n, size_t k,
                              int type_idx, int lc, int la, int lb);
 

@@ -126,6 +126,36 @@ size_t out_bytes(int type_idx)
 // grown when a call needs more (after a device-wide synchronisation, since kernels of
 // earlier calls may still be reading the old buffer), never shrunk.  What a call may do
 // with the buffer is decided by workspace_decide (workspace_policy.hpp).
+// Arrival counters of the whole-K streaming kernel's K slices (one per tile and batch entry
+// of a launch): zero when the code object is loaded, and put back to zero by the workgroup
+// that finishes a tile.  One array per GPU; launches that use it also hold the workspace
+// (their partial tiles live there), so they follow one another as its users do.
+constexpr size_t stream_arrival_slots = 4096;
+__attribute__((used)) static __device__ unsigned int stream_arrivals[stream_arrival_slots];
+std::mutex    arrivals_mutex;
+unsigned int* arrivals_address[64] = {};
+
+unsigned int* arrivals_of_current_device()
+{
+    int dev = -1;
+    if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+    {
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(arrivals_mutex);
+    if(arrivals_address[dev] == nullptr)
+    {
+        void* p = nullptr;
+        if(hipGetSymbolAddress(&p, HIP_SYMBOL(stream_arrivals)) != hipSuccess || p == nullptr)
+        {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        arrivals_address[dev] = static_cast<unsigned int*>(p);
+    }
+    return arrivals_address[dev];
+}
+
 constexpr size_t workspace_first_bytes = size_t{256} << 20;
 constexpr size_t workspace_limit_bytes = size_t{16} << 30;
 constexpr int    max_devices           = 64;
@@ -395,17 +425,13 @@ bool spans_fit(const variant_desc& v, bool a_kmajor, bool b_kmajor, size_t lda, 
     return a_span < (1ull << bits) && b_span < (1ull << bits);
 }
 
-// What the whole-K streaming kernel (pipeline 7) takes: at least one operand K-contiguous
-// (the other then 64 wide in the tile, with 16-byte aligned k rows), K whole stages of 128,
+// What the whole-K streaming kernel (pipeline 7) takes: an operand that is not K-contiguous
+// 64 wide in the tile, with 16-byte aligned k rows; K whole stages of 128,
 // 16-byte aligned rows, and a stage of a tile within reach of a 31-bit offset.
 bool streaming_ok(const kernel_problem& p, const variant_desc& v)
 {
     if(!(p.K >= 128 && p.K % 128 == 0 && aligned16(p.A) && aligned16(p.B)
          && (p.batch == 1 || (p.stride_a % 8 == 0 && p.stride_b % 8 == 0))))
-    {
-        return false;
-    }
-    if(!p.a_kmajor && !p.b_kmajor)
     {
         return false;
     }
@@ -420,7 +446,8 @@ bool streaming_ok(const kernel_problem& p, const variant_desc& v)
 }
 
 template<class OutT>
-int launch_streaming(int type_idx, const launch_plan& plan, const kernel_problem& p, hipStream_t stream)
+int launch_streaming(int type_idx, const launch_plan& plan, const kernel_problem& p, hipStream_t stream,
+                     const fixed_scratch* fixed)
 {
     const variant_desc& v = variant_at(plan.variant);
     if(!streaming_ok(p, v))
@@ -437,6 +464,39 @@ int launch_streaming(int type_idx, const launch_plan& plan, const kernel_problem
     if(grid_m * grid_n > 0x7fffffffull)
     {
         throw std::runtime_error("rocm_wmma_gemm: tile grid too large");
+    }
+    // plan.split_k = s > 1: s workgroups per tile, each with K / s, added up inside the
+    // launch by the last of them to finish.  Needs whole stages per slice, a counter per
+    // tile and batch entry, and room for the partial tiles; without them the tiles stay
+    // whole.
+    const size_t tiles       = grid_m * grid_n;
+    const size_t nb_max      = std::min<size_t>(65535, p.batch);
+    size_t       slices      = plan.split_k > 1 ? static_cast<size_t>(plan.split_k) : 1;
+    const size_t stages      = p.K / 128;
+    const size_t tile_floats = static_cast<size_t>(v.block_m) * v.block_n;
+    if(slices > 1 && (slices > 8 /* device::stream_gemm::MAX_SLICES */ || stages % slices != 0 || tiles * nb_max > stream_arrival_slots || tiles * slices > 0x7fffffffull))
+    {
+        slices = 1;
+    }
+    char*           partials = nullptr;
+    unsigned int*   arrivals = nullptr;
+    workspace_lease lease; // held until the kernel is enqueued
+    if(slices > 1)
+    {
+        const size_t bytes = tiles * nb_max * slices * tile_floats * sizeof(float);
+        arrivals           = arrivals_of_current_device();
+        if(fixed != nullptr)
+        {
+            partials = bytes <= fixed->bytes ? fixed->ptr : nullptr;
+        }
+        else
+        {
+            partials = lease.acquire(bytes, stream);
+        }
+        if(partials == nullptr || arrivals == nullptr)
+        {
+            slices = 1;
+        }
     }
     for(size_t b0 = 0; b0 < p.batch; b0 += 65535)
     {
@@ -456,10 +516,12 @@ int launch_streaming(int type_idx, const launch_plan& plan, const kernel_problem
         args.grid_m         = static_cast<int>(grid_m);
         args.grid_n         = static_cast<int>(grid_n);
         args.group          = 1;
-        args.k_slices       = 1;
-        args.blocks_per_batch = static_cast<int>(grid_m * grid_n);
+        args.k_slices       = static_cast<int>(slices);
+        args.partials       = reinterpret_cast<float*>(partials);
+        args.arrivals       = arrivals;
+        args.blocks_per_batch = static_cast<int>(tiles);
         args.batches          = static_cast<int>(nb);
-        fn<<<dim3(static_cast<unsigned>(grid_m * grid_n), static_cast<unsigned>(nb)), dim3(v.threads), 0, stream>>>(args);
+        fn<<<dim3(static_cast<unsigned>(tiles * slices), static_cast<unsigned>(nb)), dim3(v.threads), 0, stream>>>(args);
     }
     return 0;
 }
@@ -480,7 +542,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
 
     if(variant_at(plan.variant).pipeline == 7)
     {
-        return launch_streaming<OutT>(type_idx, plan, p, stream);
+        return launch_streaming<OutT>(type_idx, plan, p, stream, fixed);
     }
 
     // Operand views the kernel will see; may be replaced by padded copies below.

@@ -86,6 +86,9 @@ struct gemm_args
                             // after it (one dword per line), so that the line is on its way into
                             // the XCD's L2 a tile time before the loads that need it; the
                             // workgroups that share an operand panel touch different quarters
+    unsigned int* arrivals; // whole-K streaming kernel with k_slices > 1 only: one counter per
+                            // tile and batch entry, zero before the launch and zero again after
+                            // it; partials then holds [batch][tile][slice][BM][BN]
 };
 
 // What one workgroup works on.  blockIdx.x enumerates the whole tiles first, then

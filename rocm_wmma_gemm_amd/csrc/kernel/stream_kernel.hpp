@@ -12,11 +12,10 @@
 //   - a workgroup streams its 32 (or 64) rows of the large operand from HBM exactly once,
 //     and its rows of the small operand from L2 (every workgroup reads all of the small
 //     operand: M x K x 2 bytes each, which is why this pays only while M is small);
-//   - the small operand must be K-contiguous (row-major activations); the large one may be
-//     K-contiguous (weights stored N x K: a row of a stage is 256 contiguous bytes, two
-//     whole cache lines) or contiguous along N (weights stored K x N), in which case its
-//     side of the tile is 64 wide, so that a k row of the tile is one whole cache line,
-//     and the fragments are transposed on the way to registers by ds_read_b64_tr_b16;
+//   - an operand may be K-contiguous (a row of a stage is 256 contiguous bytes, two whole
+//     cache lines) or contiguous along M or N, in which case its side of the tile is 64
+//     wide, so that a k row of the tile is one whole cache line, and the fragments are
+//     transposed on the way to registers by ds_read_b64_tr_b16;
 //   - the LDS holds a ring of up to 8 stages of BK = 128 (24..64 KB of loads in flight per
 //     workgroup: what it takes to cover the latency of HBM at 20 GB/s per compute unit),
 //     filled by buffer_load ... lds, 1 KiB per instruction (4 rows x 256 bytes);
@@ -24,7 +23,13 @@
 //     whole tile on v_mfma_f32_16x16x32; at the end the four partial tiles are added in
 //     wave order through LDS and the sum is converted and stored;
 //   - rows past M or N are read as zeros (the buffer descriptors end with the operand)
-//     and not stored.
+//     and not stored;
+//   - where the tiles are too few for the compute units (a 64-wide side on N = 8192 gives
+//     128 of them), args.k_slices workgroups share a tile, each with a run of the stages:
+//     every one writes its fp32 tile to args.partials, counts itself in at the tile's
+//     counter, and the one that finds itself last adds the tiles up in slice order (so the
+//     sum of an element is the same in every run, whoever is last), stores C and puts the
+//     counter back to zero.  One launch still, and nobody waits for anybody.
 //
 // LDS layout of a stage: the A tile (BM rows), then the B tile (BN rows).  K-contiguous
 // operand: a row is 16 chunks of 16 bytes, chunk c of row r in slot c ^ (r mod 16), so
@@ -68,8 +73,8 @@ struct stream_gemm
     static constexpr int LOADS_A = BM / 16;
     static constexpr int LOADS_B = BN / 16;
     static constexpr int PER     = LOADS_A + LOADS_B;
+    static constexpr int MAX_SLICES = 8; // workgroups that may share a tile (args.k_slices)
     static_assert((BM == 32 || BM == 64) && (BN == 32 || BN == 64), "tiles of 32 or 64 rows and columns");
-    static_assert(A_KMAJOR || B_KMAJOR, "the small operand is K-contiguous");
     static_assert((A_KMAJOR || BM == 64) && (B_KMAJOR || BN == 64),
                   "a k row of an M/N-contiguous tile is one 128-byte line");
     static_assert(DEPTH >= 3 && (DEPTH - 1) * PER < 64, "ring depth against the 6-bit vmcnt");
@@ -118,7 +123,9 @@ struct stream_gemm
         // XCD; when the tile grid has two or more tiles along its short side, the
         // workgroups that share a panel of the large operand are given ids 8 apart, so
         // that the panel crosses the fabric once and the others find it in that XCD's L2.
-        const int wg = blockIdx.x;
+        const int tiles = args.grid_m * args.grid_n;
+        const int slice = blockIdx.x / tiles; // (slices outermost: the tile's place on its XCD stays)
+        const int wg    = blockIdx.x - slice * tiles;
         int       tm, tn;
         if(args.grid_m <= args.grid_n && args.grid_n % 8 == 0)
         {
@@ -170,20 +177,23 @@ struct stream_gemm
         const unsigned int stage_a = A_KMAJOR ? (unsigned int)ROW_BYTES : (unsigned int)(BK * lda * 2);
         const unsigned int stage_b = B_KMAJOR ? (unsigned int)ROW_BYTES : (unsigned int)(BK * ldb * 2);
 
-        const int stages = args.K / BK;
-        auto      issue  = [&](int stage, int slot_index) {
+        // this workgroup's run of the K / BK stages
+        const int stages_all = args.K / BK, stages_per = (stages_all + args.k_slices - 1) / args.k_slices;
+        const int first      = slice * stages_per;
+        const int stages     = stages_all - first < stages_per ? stages_all - first : stages_per; // >= 1 (host)
+        auto      issue      = [&](int stage, int slot_index) {
             const unsigned int base = lds_addr + slot_index * STAGE + wave * 1024;
 #pragma unroll
             for(int i = 0; i < LOADS_A; ++i)
             {
                 load_block(base + i * 4096, voff_a, rsrc_a,
-                           __builtin_amdgcn_readfirstlane((unsigned int)stage * stage_a + i * step_a));
+                           __builtin_amdgcn_readfirstlane((unsigned int)(first + stage) * stage_a + i * step_a));
             }
 #pragma unroll
             for(int i = 0; i < LOADS_B; ++i)
             {
                 load_block(base + A_BYTES + i * 4096, voff_b, rsrc_b,
-                           __builtin_amdgcn_readfirstlane((unsigned int)stage * stage_b + i * step_b));
+                           __builtin_amdgcn_readfirstlane((unsigned int)(first + stage) * stage_b + i * step_b));
             }
         };
         // Past the last stage the loads fetch the last stage again into slots that nobody
@@ -215,17 +225,27 @@ struct stream_gemm
         const int frag_off = slot * ROW_BYTES + (((4 * wave + sub) ^ slot) & 15) * 16;
         const int tr_off   = (32 * wave + 8 * sub + (slot >> 2)) * 128 + (slot & 3) * 8;
         using lds_u32x4    = __attribute__((address_space(3))) u32x4;
-        // (one statement with its own wait: the compiler does not know that these
-        // registers are filled later, and would copy them into place at once)
-        auto transposed = [](unsigned int addr) {
-            uint2 lo, hi;
-            asm volatile("ds_read_b64_tr_b16 %0, %2\n\t"
-                         "ds_read_b64_tr_b16 %1, %2 offset:512\n\t"
+        // (one statement for the four fragments of a 64-wide side, with its own wait: the
+        // compiler does not know that these registers are filled later, and would copy them
+        // into place at once; four separate statements would be four trips to LDS in a row)
+        auto transposed = [](unsigned int addr, u32x4 (&f)[4]) {
+            uint2 l0, h0, l1, h1, l2, h2, l3, h3;
+            asm volatile("ds_read_b64_tr_b16 %0, %8\n\t"
+                         "ds_read_b64_tr_b16 %1, %8 offset:512\n\t"
+                         "ds_read_b64_tr_b16 %2, %8 offset:32\n\t"
+                         "ds_read_b64_tr_b16 %3, %8 offset:544\n\t"
+                         "ds_read_b64_tr_b16 %4, %8 offset:64\n\t"
+                         "ds_read_b64_tr_b16 %5, %8 offset:576\n\t"
+                         "ds_read_b64_tr_b16 %6, %8 offset:96\n\t"
+                         "ds_read_b64_tr_b16 %7, %8 offset:608\n\t"
                          "s_waitcnt lgkmcnt(0)"
-                         : "=&v"(lo), "=&v"(hi)
+                         : "=&v"(l0), "=&v"(h0), "=&v"(l1), "=&v"(h1), "=&v"(l2), "=&v"(h2), "=&v"(l3), "=&v"(h3)
                          : "v"(addr)
                          : "memory");
-            return u32x4{lo.x, lo.y, hi.x, hi.y};
+            f[0] = u32x4{l0.x, l0.y, h0.x, h0.y};
+            f[1] = u32x4{l1.x, l1.y, h1.x, h1.y};
+            f[2] = u32x4{l2.x, l2.y, h2.x, h2.y};
+            f[3] = u32x4{l3.x, l3.y, h3.x, h3.y};
         };
 
         int slot_index = 0; // of stage t
@@ -242,29 +262,29 @@ struct stream_gemm
             lds_char_ptr       sa   = lds + slot_index * STAGE + frag_off;
             const unsigned int sa_t = lds_addr + slot_index * STAGE + tr_off;
             u32x4              fa[TM], fb[TN];
-#pragma unroll
-            for(int i = 0; i < TM; ++i)
+            if constexpr(A_KMAJOR)
             {
-                if constexpr(A_KMAJOR)
+#pragma unroll
+                for(int i = 0; i < TM; ++i)
                 {
                     fa[i] = *reinterpret_cast<lds_u32x4*>(sa + i * 16 * ROW_BYTES);
                 }
-                else
-                {
-                    fa[i] = transposed(sa_t + i * 32);
-                }
             }
-#pragma unroll
-            for(int j = 0; j < TN; ++j)
+            else
             {
-                if constexpr(B_KMAJOR)
+                transposed(sa_t, fa);
+            }
+            if constexpr(B_KMAJOR)
+            {
+#pragma unroll
+                for(int j = 0; j < TN; ++j)
                 {
                     fb[j] = *reinterpret_cast<lds_u32x4*>(sa + A_BYTES + j * 16 * ROW_BYTES);
                 }
-                else
-                {
-                    fb[j] = transposed(sa_t + A_BYTES + j * 32);
-                }
+            }
+            else
+            {
+                transposed(sa_t + A_BYTES, fb);
             }
 #pragma unroll
             for(int i = 0; i < TM; ++i)
@@ -301,15 +321,76 @@ struct stream_gemm
         }
         __syncthreads();
         OutT* C = static_cast<OutT*>(args.C) + batch * args.batch_stride_c;
-        for(int e = threadIdx.x; e < BM * BN; e += THREADS)
-        {
+        // (wave order: the sum of an element is the same in every run)
+        auto tile_sum = [&](int e) {
+            return ((part[e] + part[BM * BN + e]) + part[2 * BM * BN + e]) + part[3 * BM * BN + e];
+        };
+        auto store = [&](int e, float s) {
             const int row = e / BN, col = e % BN;
-            // (wave order: the sum of an element is the same in every run)
-            const float s = ((part[e] + part[BM * BN + e]) + part[2 * BM * BN + e]) + part[3 * BM * BN + e];
             if(row0 + row < args.M && col0 + col < args.N)
             {
                 C[(long long)(row0 + row) * args.N + col0 + col] = to_out<OutT>(s);
             }
+        };
+        if(args.k_slices == 1)
+        {
+            for(int e = threadIdx.x; e < BM * BN; e += THREADS)
+            {
+                store(e, tile_sum(e));
+            }
+            return;
+        }
+        // Several workgroups per tile.  The tiles they exchange travel through memory that
+        // every XCD sees the same way: device-scope atomic stores and loads, which pass by
+        // the XCD's own L2; a workgroup counts itself in when its stores have been
+        // acknowledged, and reads the others' tiles only after it has seen all of them
+        // counted.
+        const long long tile_lin = batch * tiles + wg;
+        float*          mine     = args.partials + (tile_lin * args.k_slices + slice) * (long long)(BM * BN);
+        for(int e = threadIdx.x; e < BM * BN; e += THREADS)
+        {
+            __hip_atomic_store(mine + e, tile_sum(e), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        // (the stores above write through to memory and are acknowledged from there; a
+        // release fence at device scope would write the whole L2 back instead, which costs
+        // more than the GEMM)
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        __syncthreads();
+        __shared__ unsigned int arrived_before;
+        if(threadIdx.x == 0)
+        {
+            arrived_before = __hip_atomic_fetch_add(args.arrivals + tile_lin, 1u, __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if(arrived_before != (unsigned int)(args.k_slices - 1))
+        {
+            return; // the last one to arrive finishes the tile
+        }
+        const float* all = args.partials + tile_lin * args.k_slices * (long long)(BM * BN);
+        // (all slices' loads of an element go out before the first is used: a loop over the
+        // slices would pay a trip to memory per slice; the host keeps k_slices <= MAX_SLICES)
+        for(int e = threadIdx.x; e < BM * BN; e += THREADS)
+        {
+            float v[MAX_SLICES];
+#pragma unroll
+            for(int q = 0; q < MAX_SLICES; ++q)
+            {
+                v[q] = q < args.k_slices ? __hip_atomic_load(all + (long long)q * (BM * BN) + e, __ATOMIC_RELAXED,
+                                                             __HIP_MEMORY_SCOPE_AGENT)
+                                         : 0.0f;
+            }
+            float s = v[0];
+#pragma unroll
+            for(int q = 1; q < MAX_SLICES; ++q)
+            {
+                s = q < args.k_slices ? s + v[q] : s;
+            }
+            store(e, s);
+        }
+        if(threadIdx.x == 0)
+        {
+            __hip_atomic_store(args.arrivals + tile_lin, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 };

@@ -155,8 +155,8 @@ static int check_select()
         return fail("model: 304 x 4096 x 4096 wants a split");
     if(!model_plan(1024, 1024, 65536, 0, 0, 1, &p) || p.split_k == 1)
         return fail("model: long K wants a split");
-    // decode-like shapes with both operands K-contiguous: the whole-K streaming kernel, 64
-    // rows of the large operand per workgroup, also when a column-major C swaps the operands
+    // decode-like shapes: the whole-K streaming kernel, 64 rows of the large operand per
+    // workgroup when it has 8192 of them, also when a column-major C swaps the operands
     if(!model_plan(32, 8192, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline != 7 || tiles[p.variant].bm != 32
        || tiles[p.variant].bn != 64 || p.split_k != 1)
         return fail("model: skinny M streams");
@@ -165,10 +165,23 @@ static int check_select()
         return fail("model: skinny M under a column-major C streams as skinny N");
     if(!model_plan(32, 8192, 8192, 0, 0, 0, &p) || tiles[p.variant].pipeline != 7 || tiles[p.variant].bn != 64)
         return fail("model: weights stored K x N stream on the 64-wide side");
-    if(!model_plan(32, 8192, 8192, 0, 1, 1, &p) || tiles[p.variant].pipeline == 7)
-        return fail("model: the streaming kernel needs the small operand K-contiguous");
-    if(!model_plan(128, 8192, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline == 7)
-        return fail("model: 128 rows stay with split-K");
+    // an operand that is not K-contiguous sits on a 64-wide side of the tile
+    if(!model_plan(32, 8192, 8192, 0, 1, 1, &p) || tiles[p.variant].pipeline != 7 || tiles[p.variant].bm != 64)
+        return fail("model: activations stored K x M stream on a 64-wide side");
+    // few tiles and a long K: several workgroups per tile
+    if(!model_plan(16, 1024, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline != 7 || p.split_k < 2)
+        return fail("model: 32 tiles of a skinny shape are shared between workgroups");
+    // fewer than 16 rows, or rows that are no multiple of 8: the streaming kernel alone
+    if(!model_plan(8, 4096, 4096, 0, 0, 1, &p) || tiles[p.variant].pipeline != 7)
+        return fail("model: 8 rows stream");
+    if(!model_plan(3, 4096, 4096, 0, 0, 1, &p) || tiles[p.variant].pipeline != 7)
+        return fail("model: 3 rows stream");
+    if(model_plan(3, 4096, 4096, 0, 1, 1, &p))
+        return fail("model: 3 rows that are not K-contiguous are nobody's");
+    if(!model_plan(128, 28672, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline == 7)
+        return fail("model: 128 rows against a very large operand stay with the tiled kernels");
+    if(!model_plan(256, 8192, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline == 7)
+        return fail("model: 256 rows are not skinny");
     // 272 tiles of 256 x 256: the last wave of 16 tiles split
     if(!model_plan(4352, 4096, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline != 5 || p.split_k >= -1)
         return fail("model: tail split");
@@ -280,12 +293,39 @@ static int print_model(int argc, char** argv)
     return 0;
 }
 
+// "stream rows cols k a_kmajor b_kmajor": the streaming kernel's cheapest plan by estimate,
+// as "block_m block_n workgroups_per_tile microseconds", or "none".
+static int print_stream(int argc, char** argv)
+{
+    if(argc < 7)
+        return 2;
+    struct tile { int bm, bn, bk, wm, wn, pipeline; };
+#define RWG_VARIANT(IDX, BM, BN, BK, WM, WN, PIPE) {BM, BN, BK, WM, WN, PIPE},
+    const tile tiles[] = {
+#include "variants.def"
+    };
+#undef RWG_VARIANT
+    const size_t rows = std::strtoull(argv[2], nullptr, 10), cols = std::strtoull(argv[3], nullptr, 10),
+                 k = std::strtoull(argv[4], nullptr, 10);
+    launch_plan p;
+    double      us = 0.0;
+    if(!stream_plan(rows, cols, k, std::atoi(argv[5]) != 0, std::atoi(argv[6]) != 0, 1, 0, &p, &us))
+    {
+        std::printf("none\n");
+        return 0;
+    }
+    std::printf("%d %d %d %.6f\n", tiles[p.variant].bm, tiles[p.variant].bn, p.split_k, us);
+    return 0;
+}
+
 int main(int argc, char** argv)
 {
     if(argc < 2)
         return 2;
     if(!std::strcmp(argv[1], "model"))
         return print_model(argc, argv);
+    if(!std::strcmp(argv[1], "stream"))
+        return print_stream(argc, argv);
     if(!std::strcmp(argv[1], "tilemap"))
         return check_tilemap();
     if(!std::strcmp(argv[1], "xcd"))

@@ -309,8 +309,8 @@ def test_whole_k_streaming_kernel_agrees_with_oracle(loader):
     column-major C runs as the transposed problem), the large operand K-contiguous or
     contiguous along N, ragged M and N (rows past the edge are read as zeros and not
     stored), one stage and many, a strided batch, all type pairs, and -1 for what it does
-    not take (two operands that are not K-contiguous, one on a 32-wide side of the tile,
-    K no multiple of 128)."""
+    not take (an operand that is not K-contiguous on a 32-wide side of the tile, K no
+    multiple of 128)."""
     import torch
 
     stream = [v for v in loader.variants() if v.pipeline == 7]
@@ -321,7 +321,7 @@ def test_whole_k_streaming_kernel_agrees_with_oracle(loader):
         for (M, N, K) in shapes:
             # both operands K-contiguous, then the large operand contiguous along N (weights
             # stored K x N), each with C row- and column-major
-            for (lc, la, lb) in [(0, 0, 1), (1, 0, 1), (0, 0, 0), (1, 0, 0), (0, 1, 1)]:
+            for (lc, la, lb) in [(0, 0, 1), (1, 0, 1), (0, 0, 0), (1, 0, 0), (0, 1, 1), (0, 1, 0), (1, 1, 0)]:
                 for tname in TYPE_PAIRS:
                     din, dout = TYPE_PAIRS[tname]
                     A, B = make_inputs(M, N, K, la, lb, din, seed_a=3, seed_b=4)
@@ -341,6 +341,8 @@ def test_whole_k_streaming_kernel_agrees_with_oracle(loader):
     assert {(bm, bn) for (bm, bn, lc, la, lb) in ran if (la, lb) == (0, 1)} == {(32, 32), (64, 32), (32, 64), (64, 64)}
     assert (32, 64, 0, 0, 0) in ran and (64, 32, 1, 0, 0) in ran and (64, 64, 0, 0, 0) in ran
     assert not any((la, lb) == (1, 1) and lc == 0 and bm != 64 for (bm, bn, lc, la, lb) in ran)
+    # neither operand K-contiguous: the 64 x 64 tile alone
+    assert {(bm, bn) for (bm, bn, lc, la, lb) in ran if (la, lb) == (1, 0)} == {(64, 64)}
     # a strided batch, and bit-identical repeats
     v = stream[0]
     M, N, K, batch = 48, 320, 640, 3
@@ -356,8 +358,66 @@ def test_whole_k_streaming_kernel_agrees_with_oracle(loader):
     # what it does not take
     dA = torch.zeros(64 * 256, dtype=torch.float16, device="cuda")
     dC = torch.zeros(64 * 64, dtype=torch.float16, device="cuda")
-    assert loader.run_variant(v.index, 1, 1, dC, dA, dA, 64, 64, 256, 0, 1, 0) == -1   # neither operand K-contiguous
+    assert loader.run_variant(v.index, 1, 1, dC, dA, dA, 64, 64, 256, 0, 1, 0) == -1   # 32-wide sides, neither operand K-contiguous
     assert loader.run_variant(v.index, 1, 1, dC, dA, dA, 64, 64, 200, 0, 0, 1) == -1   # K % 128 != 0
+
+
+def test_workgroups_that_share_a_tile_of_the_streaming_kernel(loader):
+    """Split field s > 1 on pipeline 7: s workgroups per tile, each with K / s, exchange
+    their fp32 tiles through the scratch memory inside the one launch; whichever finishes
+    last adds them up in slice order.  Against the oracle, and bit-identical from run to
+    run (the order of the sum does not depend on who is last); every tile, 2, 4 and 8 workgroups
+    per tile, ragged M and N, a strided batch, launches back to back (the counters are back
+    at zero after each), the entry point that allocates nothing, and a split that does not
+    divide the stages (the tile then stays whole)."""
+    import torch
+
+    stream = [v for v in loader.variants() if v.pipeline == 7]
+    shapes = [(16, 1024, 2048), (40, 200, 1024), (128, 256, 4096), (1000, 24, 2048)]
+    for v in stream:
+        for split in (2, 4, 8):
+            for (M, N, K) in shapes:
+                for (lc, la, lb) in [(0, 0, 1), (0, 0, 0), (1, 0, 0), (0, 1, 0)]:
+                    if not built_for(v, lc, la, lb, K, M, N):
+                        continue
+                    tname = "f16_f16" if (M + split) % 3 else "f32_bf16"
+                    din, dout = TYPE_PAIRS[tname]
+                    A, B = make_inputs(M, N, K, la, lb, din, seed_a=5, seed_b=6)
+                    runs = [run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout, variant=(v.index, 1, split))
+                            for _ in range(3)]
+                    try:
+                        check_against_oracle(runs[0], A, B, M, N, K, lc, la, lb, din, dout)
+                    except AssertionError as e:
+                        raise AssertionError(
+                            f"variant {v.index} split {split} {M}x{N}x{K} C{lc} A{la} B{lb} {tname}: {e}") from None
+                    assert all(np.array_equal(r.view(np.uint8), runs[0].view(np.uint8)) for r in runs[1:]), (
+                        v.index, split, M, N, K, lc, la, lb)
+    # a strided batch (a counter per tile and batch entry)
+    v = next(x for x in stream if (x.block_m, x.block_n) == (32, 64))
+    M, N, K, batch = 48, 320, 1024, 3
+    As = [O.init_matrix(M, K, 0, O.F16, seed=1 + b) for b in range(batch)]
+    Bs = [O.init_matrix(K, N, 1, O.F16, seed=9 + b) for b in range(batch)]
+    gpu = run_gpu(loader, np.concatenate(As), np.concatenate(Bs), M, N, K, 0, 0, 1, O.F16, O.F32, batch=batch,
+                  variant=(v.index, 1, 4))
+    for b in range(batch):
+        check_against_oracle(gpu[b * M * N:(b + 1) * M * N], As[b], Bs[b], M, N, K, 0, 0, 1, O.F16, O.F32)
+    # a split that does not divide the 10 stages: runs, as whole tiles
+    A, B = make_inputs(32, 256, 1280, 0, 1, O.F16, seed_a=2, seed_b=3)
+    check_against_oracle(run_gpu(loader, A, B, 32, 256, 1280, 0, 0, 1, O.F16, O.F16, variant=(v.index, 1, 4)),
+                         A, B, 32, 256, 1280, 0, 0, 1, O.F16, O.F16)
+    # the default dispatch shares tiles where they are few and K is long, and the entry
+    # point that allocates nothing gives the same bits
+    M, N, K = 16, 1024, 8192
+    variant, _, split = loader.select(M, N, K, 0, 0, 0, 1)
+    assert loader.variants()[variant].pipeline == 7 and split > 1, (variant, split)
+    A, B = make_inputs(M, N, K, 0, 1, O.F16, seed_a=7, seed_b=8)
+    ordinary = run_gpu(loader, A, B, M, N, K, 0, 0, 1, O.F16, O.F16)
+    check_against_oracle(ordinary, A, B, M, N, K, 0, 0, 1, O.F16, O.F16)
+    dA, dB = to_device(A, O.F16), to_device(B, O.F16)
+    dC = torch.full((M * N,), float("nan"), dtype=torch.float16, device="cuda")
+    assert loader.gemm_noalloc(dC, dA, dB, M, N, K, 0, 0, 1) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host(dC, O.F16).view(np.uint8), ordinary.view(np.uint8))
 
 
 def test_split_tail_wave_agrees_with_oracle(loader):
