@@ -430,6 +430,13 @@ launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int 
     {
         return plan;
     }
+    // A skinny shape that neither has an entry nor suits the model (K no multiple of 128,
+    // odd extents): the nearest tuned entry would be a large square's plan, 256 x 256 tiles
+    // for a handful of rows; the shape heuristic cuts K over the compute units instead.
+    if(std::min(m, n) <= 64 && std::max(m, n) >= 512)
+    {
+        return heuristic_plan(m, n, k, lc);
+    }
     return select_plan_from(tuned_table, tuned_count, m, n, k, type_idx, lc, la, lb);
 }
 

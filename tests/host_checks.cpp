@@ -182,6 +182,13 @@ static int check_select()
         return fail("model: 128 rows against a very large operand stay with the tiled kernels");
     if(!model_plan(256, 8192, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline == 7)
         return fail("model: 256 rows are not skinny");
+    // a skinny shape the model does not take (K no multiple of 128) and the table does not
+    // hold: the shape heuristic's split, not the nearest large square's plan
+    {
+        const launch_plan q = select_plan(8, 4096, 4000, 0, 0, 0, 1);
+        if(tiles[q.variant].pipeline != 0 || q.split_k < 2)
+            return fail("select: skinny shape with K = 4000");
+    }
     // 272 tiles of 256 x 256: the last wave of 16 tiles split
     if(!model_plan(4352, 4096, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline != 5 || p.split_k >= -1)
         return fail("model: tail split");
