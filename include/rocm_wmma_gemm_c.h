@@ -85,7 +85,9 @@ int rocm_wmma_gemm_variant_info_get(int variant, rocm_wmma_gemm_variant_info* in
  * gemm_config_gfx950_*.json, then shape heuristics).  type_idx as above.
  * Also reports the swizzle (band height of the tile walk: g > 0 bands of g tile rows,
  * g < 0 bands of -g tile columns) and the split field: s > 1 = every
- * tile's K range is cut into s slices; -s < -1 = only the tiles of the last, partial
+ * tile's K range is cut into s slices (added up by a second kernel; on the whole-K streaming
+ * kernel, pipeline 7, s = 2, 4 or 8 workgroups share a tile and the last of them to finish
+ * adds the parts up inside the one launch); -s < -1 = only the tiles of the last, partial
  * wave over the compute units are cut into s slices; -1 = the persistent kernel's
  * workgroups each take the same number of K tiles of the sequence of all K tiles of the
  * launch, wherever the tile borders fall, and the cut tiles are added up afterwards (other

@@ -947,6 +947,13 @@ int run(int type_idx, const launch_plan* forced, void* C, void* A, void* B, size
         = forced ? *forced
                  : select_plan(M, N, K, type_idx, layout_c, layout_a, layout_b, batch,
                                compute_units_of_current_device());
+    if(!forced && variant_at(plan.variant).pipeline == 7 && !streaming_ok(p, variant_at(plan.variant)))
+    {
+        // the dispatcher prices shapes, not pointers: operands that the streaming kernel
+        // cannot take (base pointers or batch strides that are not 16-byte aligned) go
+        // to the general kernel with the shape heuristic's split
+        plan = heuristic_plan(M, N, K, layout_c);
+    }
     if(variant_at(plan.variant).pipeline != 0
        && lookup_kernel(type_idx, p.a_kmajor, p.b_kmajor, plan.variant,
                         static_cast<int>(device::load_mode::vec_unguarded))
