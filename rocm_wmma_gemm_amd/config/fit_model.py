@@ -116,14 +116,15 @@ STREAM_TILES = ("32x32", "64x32", "32x64", "64x64")
 def stream_estimate(c: dict, rows: int, cols: int, K: int, a_kmajor: bool, b_kmajor: bool, bm: int, bn: int,
                     slices: int, batch: int = 1, cus: int = 256) -> float:
     """Microseconds of one plan of the whole-K streaming kernel: launch, then per pass over
-    the compute units the fill of the ring and the workgroup's stages, each at the slower of
-    what a compute unit pulls with its ring of loads in flight and its share of the stream
-    of the large operand from memory; plus the exchange of partial tiles when several
+    the compute units (two workgroups to a unit, one for the 64 x 64 tile) the fill of the
+    ring and the workgroup's stages, each at the slower of what a workgroup pulls with its
+    ring of loads in flight and its share of the stream of the large operand from memory; plus the exchange of partial tiles when several
     workgroups share a tile.  c = the "stream" object of the model file."""
     tiles = -(-rows // bm) * -(-cols // bn)
     groups = tiles * slices * batch
-    passes = -(-groups // cus)
-    active = min(groups, cus)
+    resident = cus * (1 if (bm, bn) == (64, 64) else 2)  # workgroups that the LDS lets run at once
+    passes = -(-groups // resident)
+    active = min(groups, resident)
     stages = (K // 128) // slices
     wide = cols >= rows  # the large operand is B
     large_kmajor = b_kmajor if wide else a_kmajor
@@ -132,6 +133,8 @@ def stream_estimate(c: dict, rows: int, cols: int, K: int, a_kmajor: bool, b_kma
     other = (0 if a_kmajor else 1) + (0 if b_kmajor else 1)
     per_cu = c["stage_us"][f"{bm}x{bn}"] * (1.0 + c["transposed_operand"] * other)
     small_bytes = (bm if wide else bn) * 256  # every workgroup reads its rows of the small operand, from L2
+    # (the workgroups that read the same panel find only part of it in L2)
+    sharing = 1.0 + (sharing - 1.0) * c["panel_sharing"]
     from_memory = (large_bytes * (active / sharing) / (c["bytes_per_us_kmajor" if large_kmajor else "bytes_per_us_other"])
                    + small_bytes * active / c["bytes_per_us_l2"])
     return (c["launch_us"] + passes * (c["fill_us"] + stages * max(per_cu, from_memory))
@@ -152,7 +155,7 @@ def fit_stream(records: list, start: dict) -> dict:
     from scipy.optimize import least_squares
 
     keys = ["launch_us", "fill_us", "exchange_us", "bytes_per_us_kmajor", "bytes_per_us_other", "bytes_per_us_l2",
-            "transposed_operand"]
+            "transposed_operand", "panel_sharing"]
 
     def unpack(p):
         c = {k: float(v) for k, v in zip(keys, p)}
@@ -170,13 +173,14 @@ def fit_stream(records: list, start: dict) -> dict:
         return [math.log(stream_estimate(c, *row[:8]) / row[8]) for row in rows]
 
     p0 = [start[k] for k in keys] + [start["stage_us"][t] for t in STREAM_TILES]
-    res = least_squares(residuals, p0, bounds=([0.0] * len(p0), [20, 10, 30, 2e7, 2e7, 2e8, 3] + [2.0] * len(STREAM_TILES)))
+    res = least_squares(residuals, p0, bounds=([0.0] * len(p0), [20, 10, 30, 2e7, 2e7, 2e8, 3, 1] + [2.0] * len(STREAM_TILES)))
     c = unpack(res.x)
     for k in ("launch_us", "fill_us", "exchange_us"):
         c[k] = round(c[k], 2)
     for k in ("bytes_per_us_kmajor", "bytes_per_us_other", "bytes_per_us_l2"):
         c[k] = round(c[k], -4)
     c["transposed_operand"] = round(c["transposed_operand"], 3)
+    c["panel_sharing"] = round(c["panel_sharing"], 3)
     c["stage_us"] = {t: round(v, 4) for t, v in c["stage_us"].items()}
     return c
 

@@ -355,7 +355,7 @@ bool stream_plan(size_t rows, size_t cols, size_t k, bool a_kmajor, bool b_kmajo
         const double per_cu  = c.stage_us[slot] * (1.0 + c.transposed_operand * other);
         const double large   = static_cast<double>(wide ? bn : bm) * 256.0;
         const double small   = static_cast<double>(wide ? bm : bn) * 256.0;
-        const double sharing = static_cast<double>(wide ? tm : tn);
+        const double sharing = 1.0 + (static_cast<double>(wide ? tm : tn) - 1.0) * c.panel_sharing;
         const double rate    = (wide ? b_kmajor : a_kmajor) ? c.bytes_per_us_kmajor : c.bytes_per_us_other;
         for(size_t s = 1; s <= 8; s *= 2)
         {
@@ -364,11 +364,13 @@ bool stream_plan(size_t rows, size_t cols, size_t k, bool a_kmajor, bool b_kmajo
             {
                 continue;
             }
-            const size_t groups = tiles * s * batch;
-            const double active = static_cast<double>(groups < cus ? groups : cus);
+            // (the LDS lets two workgroups run on a compute unit at once, one of the 64 x 64 tile)
+            const size_t groups   = tiles * s * batch;
+            const size_t resident = cus * ((bm == 64 && bn == 64) ? 1 : 2);
+            const double active   = static_cast<double>(groups < resident ? groups : resident);
             const double stage  = std::max(per_cu, large * (active / sharing) / rate + small * active / c.bytes_per_us_l2);
             const double t      = c.launch_us
-                             + static_cast<double>(ceil_div(groups, cus)) * (c.fill_us + static_cast<double>(stages / s) * stage)
+                             + static_cast<double>(ceil_div(groups, resident)) * (c.fill_us + static_cast<double>(stages / s) * stage)
                              + (s > 1 ? c.exchange_us : 0.0);
             if(!found || t < *microseconds)
             {

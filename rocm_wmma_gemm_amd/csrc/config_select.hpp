@@ -58,6 +58,8 @@ struct model_stream
     double bytes_per_us_kmajor, bytes_per_us_other; // stream of the large operand from memory
     double bytes_per_us_l2; // the small operand, which every workgroup reads from L2
     double transposed_operand; // relative cost of a stage per operand that is not K-contiguous
+    double panel_sharing; // how much of a panel of the large operand that g workgroups read
+                          // is fetched once for all: it counts as fetched g / (1 + (g - 1) x this) times
     double stage_us[4]; // per stage of 128 of one compute unit: tiles 32x32, 64x32, 32x64, 64x64
 };
 struct model_constants

@@ -28,8 +28,8 @@ constexpr int ring_bytes(int bm, int bn, int bk, int pipeline)
 {
     if(pipeline == 7)
     {
-        // as many stages as fit 144 KB, at most 8 (device::stream_gemm::DEPTH)
-        const int stage = (bm + bn) * bk * 2, depth = 144 * 1024 / stage;
+        // as many stages as fit 76 KB, at least 3 and at most 8 (device::stream_gemm::DEPTH)
+        const int stage = (bm + bn) * bk * 2, fit = 76 * 1024 / stage, depth = fit < 3 ? 3 : fit;
         return (depth < 8 ? depth : 8) * stage;
     }
     return (pipeline == 6 || (pipeline != 0 && bk == 32) ? 4 : 2) * (bm + bn) * bk * 2;

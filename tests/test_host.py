@@ -636,8 +636,8 @@ STREAM_SWEEP = os.path.join(ROOT, "tests", "golden", "stream_sweep_gfx950_f16.js
 # What the estimate for the streaming kernel's plans is held to on the recorded sweep (135
 # decode-like problems on an MI355X, fp16: M = 8..128 against N x K from 1024 to 28672, three
 # layout triples, every tile with 1, 2, 4 and 8 workgroups per tile):
-STREAM_WORST_REGRET = 1.40  # measured 1.33
-STREAM_MEAN_REGRET = 1.04   # measured 1.027 (geometric mean)
+STREAM_WORST_REGRET = 1.45  # measured 1.36
+STREAM_MEAN_REGRET = 1.05   # measured 1.034 (geometric mean)
 
 
 def test_stream_plan_pick_is_within_its_stated_regret_of_the_measured_best(host_tool):
@@ -676,7 +676,7 @@ def test_stream_constants_are_what_a_fit_of_the_recorded_sweep_gives():
     shipped = json.load(open(os.path.join(ROOT, "rocm_wmma_gemm_amd", "config", "model_gfx950.json")))["stream"]
     fitted = F.fit_stream(json.load(open(STREAM_SWEEP)), shipped)
     for key in ("launch_us", "fill_us", "exchange_us", "bytes_per_us_kmajor", "bytes_per_us_other", "bytes_per_us_l2",
-                "transposed_operand"):
+                "transposed_operand", "panel_sharing"):
         assert abs(fitted[key] - shipped[key]) <= 0.1 * shipped[key] + 0.05, (key, fitted[key], shipped[key])
     for tile, us in shipped["stage_us"].items():
         assert abs(fitted["stage_us"][tile] - us) <= 0.1 * us, (tile, fitted["stage_us"][tile], us)
