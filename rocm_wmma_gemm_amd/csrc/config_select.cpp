@@ -314,8 +314,12 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
         }
     }
     // (between 65 and 128 rows the two families are within 20 % of each other and the two
-    // estimates are not that good: the tiled kernels keep those when they take the shape)
-    if(have_stream && (!found || (stream_us < best && std::min(rows, cols) <= 64)))
+    // estimates are not that good: the tiled kernels keep those when they take the shape,
+    // except against a small large operand with both K-contiguous, where the streaming
+    // kernel measured 1.1 to 1.5 times faster: 128 x 4096 x 4096 14.1 against 19.2 us)
+    const size_t skinny = std::min(rows, cols), other = std::max(rows, cols);
+    const bool   compete = skinny <= 64 || (a_kmajor && b_kmajor && other * k <= (size_t{1} << 24));
+    if(have_stream && (!found || (stream_us < best && compete)))
     {
         *out  = stream_best;
         found = true;

@@ -182,6 +182,11 @@ static int check_select()
         return fail("model: 128 rows against a very large operand stay with the tiled kernels");
     if(!model_plan(256, 8192, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline == 7)
         return fail("model: 256 rows are not skinny");
+    // 65 to 128 rows: only against a small large operand, both K-contiguous
+    if(!model_plan(128, 4096, 4096, 0, 0, 1, &p) || tiles[p.variant].pipeline != 7)
+        return fail("model: 128 rows against 4096 x 4096, both K-contiguous, stream");
+    if(!model_plan(128, 4096, 4096, 0, 0, 0, &p) || tiles[p.variant].pipeline == 7)
+        return fail("model: 128 rows against 4096 x 4096 stored K x N stay with the tiled kernels");
     // a skinny shape the model does not take (K no multiple of 128) and the table does not
     // hold: the shape heuristic's split, not the nearest large square's plan
     {
