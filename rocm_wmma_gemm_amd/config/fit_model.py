@@ -135,7 +135,12 @@ def stream_estimate(c: dict, rows: int, cols: int, K: int, a_kmajor: bool, b_kma
     small_bytes = (bm if wide else bn) * 256  # every workgroup reads its rows of the small operand, from L2
     # (the workgroups that read the same panel find only part of it in L2)
     sharing = 1.0 + (sharing - 1.0) * c["panel_sharing"]
-    from_memory = (large_bytes * (active / sharing) / (c["bytes_per_us_kmajor" if large_kmajor else "bytes_per_us_other"])
+    rate = c["bytes_per_us_kmajor" if large_kmajor else "bytes_per_us_other"]
+    if max(rows, cols) * K * 2 > 256 << 20:
+        # the large operand does not fit the memory-side cache, which serves part of a
+        # repeated call on a smaller one (not fitted: left free it soaks up other effects)
+        rate *= c["beyond_cache"]
+    from_memory = (large_bytes * (active / sharing) / rate
                    + small_bytes * active / c["bytes_per_us_l2"])
     return (c["launch_us"] + passes * (c["fill_us"] + stages * max(per_cu, from_memory))
             + (c["exchange_us"] if slices > 1 else 0.0))
@@ -159,6 +164,7 @@ def fit_stream(records: list, start: dict) -> dict:
 
     def unpack(p):
         c = {k: float(v) for k, v in zip(keys, p)}
+        c["beyond_cache"] = start["beyond_cache"]
         c["stage_us"] = {t: float(v) for t, v in zip(STREAM_TILES, p[len(keys):])}
         return c
 

@@ -113,7 +113,7 @@ def render_model(m: dict) -> list[str]:
     stream = ["constexpr model_stream model_stream_constants = {"
               + ", ".join(repr(float(st[k])) for k in ("launch_us", "fill_us", "exchange_us", "bytes_per_us_kmajor",
                                                         "bytes_per_us_other", "bytes_per_us_l2",
-                                                        "transposed_operand", "panel_sharing"))
+                                                        "transposed_operand", "panel_sharing", "beyond_cache"))
               + ", {" + ", ".join(repr(float(st["stage_us"][t])) for t in ("32x32", "64x32", "32x64", "64x64")) + "}};"]
     return ([f"constexpr int model_compute_units = {int(m['compute_units'])};"]
             + [f"constexpr double model_{k} = {float(m[k])!r};" for k in

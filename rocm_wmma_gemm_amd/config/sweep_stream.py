@@ -25,6 +25,11 @@ sys.path.insert(0, os.path.normpath(os.path.join(HERE, "..", "..")))
 SHAPES = [(M, N, K) for M in (8, 16, 32, 64, 128)
           for (N, K) in ((1024, 8192), (2048, 2048), (4096, 4096), (4096, 14336), (8192, 8192), (14336, 4096),
                          (28672, 8192), (8192, 1024), (2048, 8192))]
+# small problems, where a 256 x 256 tiling leaves most compute units idle and a workgroup per
+# 32- or 64-wide tile over the whole K is a contender too (--small)
+SMALL_SHAPES = [(256, 256, 1024), (512, 512, 512), (512, 512, 4096), (768, 768, 768), (1024, 1024, 1024),
+                (1024, 1024, 4096), (1536, 1536, 1536), (2048, 2048, 2048), (2048, 1024, 1024), (512, 2048, 2048),
+                (1024, 4096, 1024), (2048, 2048, 512), (256, 4096, 2048), (384, 1536, 1536), (3072, 1024, 1024)]
 LAYOUTS = ("rcr", "rrr", "crr")  # A, B, C: r row-major, c column-major
 
 
@@ -39,6 +44,7 @@ def main(argv=None) -> int:
     ap.add_argument("--out", required=True)
     ap.add_argument("--type", default="f16_f16", choices=["f16_f16", "bf16_bf16"])
     ap.add_argument("--reps", type=int, default=15)
+    ap.add_argument("--small", action="store_true", help="the small square and rectangular shapes instead")
     a = ap.parse_args(argv)
 
     import torch
@@ -68,7 +74,7 @@ def main(argv=None) -> int:
     gen = torch.Generator(device="cuda")
     gen.manual_seed(1)
     out = []
-    for (M, N, K) in SHAPES:
+    for (M, N, K) in (SMALL_SHAPES if a.small else SHAPES):
         A = torch.randn(M * K, device="cuda", generator=gen).to(dtype)
         B = torch.randn(K * N, device="cuda", generator=gen).to(dtype)
         C = torch.empty(M * N, dtype=dtype, device="cuda")

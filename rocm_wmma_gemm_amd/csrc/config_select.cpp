@@ -317,8 +317,11 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
     // estimates are not that good: the tiled kernels keep those when they take the shape,
     // except against a small large operand with both K-contiguous, where the streaming
     // kernel measured 1.1 to 1.5 times faster: 128 x 4096 x 4096 14.1 against 19.2 us)
+    // and small problems (at most 2^20 elements of C, K up to 4096: 512 x 2048 x 2048 12.7
+    // against 17.9 us, 256 x 256 x 1024 9.3 against 13.7) unless neither operand is K-contiguous
     const size_t skinny = std::min(rows, cols), other = std::max(rows, cols);
-    const bool   compete = skinny <= 64 || (a_kmajor && b_kmajor && other * k <= (size_t{1} << 24));
+    const bool   compete = skinny <= 64 || (a_kmajor && b_kmajor && other * k <= (size_t{1} << 24))
+                         || (rows * cols <= (size_t{1} << 20) && k <= 4096 && (a_kmajor || b_kmajor));
     if(have_stream && (!found || (stream_us < best && compete)))
     {
         *out  = stream_best;
@@ -330,7 +333,8 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
 bool stream_plan(size_t rows, size_t cols, size_t k, bool a_kmajor, bool b_kmajor, size_t batch, size_t cus_of_device,
                  launch_plan* out, double* microseconds)
 {
-    if(k % 128 != 0 || k < 256 || rows == 0 || cols == 0 || (rows > 128 && cols > 128))
+    // skinny, or so small that tiles of 64 x 64 do not outnumber the compute units of an MI355X
+    if(k % 128 != 0 || k < 256 || rows == 0 || cols == 0 || (rows > 128 && cols > 128 && rows * cols > (size_t{1} << 20)))
     {
         return false;
     }
@@ -360,7 +364,8 @@ bool stream_plan(size_t rows, size_t cols, size_t k, bool a_kmajor, bool b_kmajo
         const double large   = static_cast<double>(wide ? bn : bm) * 256.0;
         const double small   = static_cast<double>(wide ? bm : bn) * 256.0;
         const double sharing = 1.0 + (static_cast<double>(wide ? tm : tn) - 1.0) * c.panel_sharing;
-        const double rate    = (wide ? b_kmajor : a_kmajor) ? c.bytes_per_us_kmajor : c.bytes_per_us_other;
+        const double rate    = ((wide ? b_kmajor : a_kmajor) ? c.bytes_per_us_kmajor : c.bytes_per_us_other)
+                            * (std::max(rows, cols) * k * 2 > (size_t{256} << 20) ? c.beyond_cache : 1.0);
         for(size_t s = 1; s <= 8; s *= 2)
         {
             // (the counters of the tiles that several workgroups share: 4096 a launch)

@@ -60,6 +60,8 @@ struct model_stream
     double transposed_operand; // relative cost of a stage per operand that is not K-contiguous
     double panel_sharing; // how much of a panel of the large operand that g workgroups read
                           // is fetched once for all: it counts as fetched g / (1 + (g - 1) x this) times
+    double beyond_cache; // factor on the two rates from memory for a large operand over 256 MB
+                         // (set by hand, not fitted)
     double stage_us[4]; // per stage of 128 of one compute unit: tiles 32x32, 64x32, 32x64, 64x64
 };
 struct model_constants
@@ -90,8 +92,8 @@ launch_plan heuristic_plan(size_t m, size_t n, size_t k, int lc);
 // cus: compute units of the GPU the plan is for (0: the GPU the constants were measured on).
 bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_plan* out, size_t batch = 1,
                 size_t cus = 0);
-// The streaming kernel's plans alone (skinny shapes: one extent at most 128, K whole stages
-// of 128), in kernel space (rows x cols, the operands' K-contiguity): the cheapest by
+// The streaming kernel's plans alone (skinny shapes: one extent at most 128, or small ones:
+// at most 2^20 elements of C; K whole stages of 128), in kernel space (rows x cols, the operands' K-contiguity): the cheapest by
 // estimate and its microseconds; false when no compiled variant takes the problem.
 bool stream_plan(size_t rows, size_t cols, size_t k, bool a_kmajor, bool b_kmajor, size_t batch, size_t cus,
                  launch_plan* out, double* microseconds);

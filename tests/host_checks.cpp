@@ -185,8 +185,13 @@ static int check_select()
     // 65 to 128 rows: only against a small large operand, both K-contiguous
     if(!model_plan(128, 4096, 4096, 0, 0, 1, &p) || tiles[p.variant].pipeline != 7)
         return fail("model: 128 rows against 4096 x 4096, both K-contiguous, stream");
-    if(!model_plan(128, 4096, 4096, 0, 0, 0, &p) || tiles[p.variant].pipeline == 7)
-        return fail("model: 128 rows against 4096 x 4096 stored K x N stay with the tiled kernels");
+    if(!model_plan(128, 4096, 4096, 0, 1, 0, &p) || tiles[p.variant].pipeline == 7)
+        return fail("model: 128 rows against 4096 x 4096, neither K-contiguous, stay with the tiled kernels");
+    // small problems: at most 2^20 elements of C, an operand K-contiguous
+    if(!model_plan(512, 2048, 2048, 0, 0, 0, &p) || tiles[p.variant].pipeline != 7)
+        return fail("model: 512 x 2048 x 2048 streams");
+    if(!model_plan(2048, 1024, 1024, 0, 0, 1, &p) || tiles[p.variant].pipeline == 7)
+        return fail("model: 2048 x 1024 x 1024 is too large for a workgroup per small tile");
     // a skinny shape the model does not take (K no multiple of 128) and the table does not
     // hold: the shape heuristic's split, not the nearest large square's plan
     {

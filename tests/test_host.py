@@ -632,12 +632,14 @@ def test_model_constants_are_what_a_fit_of_the_recorded_sweep_gives():
     assert F.parse([line]) == [(4096, 4096, 4096, "rcr", "f16_f16", 5, 256, 256, 64, 2, 2, 4, 1, 0, 0.0981)]
 
 
-STREAM_SWEEP = os.path.join(ROOT, "tests", "golden", "stream_sweep_gfx950_f16.json")
-# What the estimate for the streaming kernel's plans is held to on the recorded sweep (135
-# decode-like problems on an MI355X, fp16: M = 8..128 against N x K from 1024 to 28672, three
-# layout triples, every tile with 1, 2, 4 and 8 workgroups per tile):
-STREAM_WORST_REGRET = 1.45  # measured 1.36
-STREAM_MEAN_REGRET = 1.05   # measured 1.034 (geometric mean)
+STREAM_SWEEP = os.path.join(ROOT, "tests", "golden", "stream_sweep_gfx950_f16.json")  # what the constants are fitted to
+STREAM_SMALL_SWEEP = os.path.join(ROOT, "tests", "golden", "stream_small_sweep_gfx950_f16.json")  # held out
+# What the estimate for the streaming kernel's plans is held to on the recorded sweeps (on an
+# MI355X, fp16, three layout triples, every tile with 1, 2, 4 and 8 workgroups per tile): the
+# 135 decode-like problems its constants are fitted to (M = 8..128 against N x K from 1024 to
+# 28672) and 45 small ones that the fit has not seen (256 x 256 x 1024 to 2048^3):
+STREAM_WORST_REGRET = 1.45  # measured 1.36 (fitted problems), 1.11 (held out)
+STREAM_MEAN_REGRET = 1.05   # measured 1.030 and 1.013 (geometric mean)
 
 
 def test_stream_plan_pick_is_within_its_stated_regret_of_the_measured_best(host_tool):
@@ -648,14 +650,25 @@ def test_stream_plan_pick_is_within_its_stated_regret_of_the_measured_best(host_
     import math
 
     F = _fit_module()
-    records = json.load(open(STREAM_SWEEP))
     constants = json.load(open(os.path.join(ROOT, "rocm_wmma_gemm_amd", "config", "model_gfx950.json")))["stream"]
-    logs, worst = [], (1.0, None)
+    for sweep, at_least in ((STREAM_SWEEP, 130), (STREAM_SMALL_SWEEP, 20)):
+        _stream_regret_of(host_tool, F, json.load(open(sweep)), constants, at_least)
+
+
+def _stream_regret_of(host_tool, F, records, constants, at_least):
+    import math
+
+    logs, worst = [], (1.0, ())
     for r in records:
         a_k, b_k = r["lay"][0] == "r", r["lay"][1] == "c"  # C row-major in the sweep
         out = subprocess.run([host_tool, "stream", str(r["M"]), str(r["N"]), str(r["K"]), str(int(a_k)), str(int(b_k))],
                              capture_output=True, text=True)
-        assert out.returncode == 0 and out.stdout.strip() != "none", (r["M"], r["N"], r["K"], r["lay"], out.stdout)
+        assert out.returncode == 0, (r["M"], r["N"], r["K"], r["lay"], out.stdout)
+        if out.stdout.strip() == "none":
+            # neither skinny nor small: not the streaming kernel's (the sweep holds a few such
+            # shapes to show where it stops paying)
+            assert min(r["M"], r["N"]) > 128 and r["M"] * r["N"] > 1 << 20
+            continue
         bm, bn, slices, us = out.stdout.split()
         name = f"{bm}x{bn}s{slices}"
         assert name in r["t"], (name, sorted(r["t"]))
@@ -664,7 +677,7 @@ def test_stream_plan_pick_is_within_its_stated_regret_of_the_measured_best(host_
         ratio = r["t"][name] / min(r["t"].values())
         logs.append(math.log(ratio))
         worst = max(worst, (ratio, (r["M"], r["N"], r["K"], r["lay"], name)))
-    assert len(logs) >= 100
+    assert len(logs) >= at_least
     assert worst[0] <= STREAM_WORST_REGRET, worst
     assert math.exp(sum(logs) / len(logs)) <= STREAM_MEAN_REGRET
 
