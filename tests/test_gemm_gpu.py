@@ -702,12 +702,16 @@ def test_two_streams_share_the_scratch_memory(loader):
     result must equal, bit for bit, what the same call gives when nothing else runs."""
     import torch
 
-    cases = [  # (M, N, K, lc, la, lb): split-K (skinny, long K) and padded copies (odd K)
+    cases = [  # (M, N, K, lc, la, lb): split-K (skinny, long K), padded copies (odd K), and the
+        # streaming kernel's shared tiles (partial tiles in the buffer, one set of counters)
         (64, 8192, 8192, 0, 1, 0),
         (1024, 1024, 16384, 0, 0, 1),
         (128, 8192, 8192, 1, 0, 0),
         (1025, 1031, 2049, 0, 0, 1),
+        (16, 1024, 8192, 0, 0, 1),
+        (32, 2048, 8192, 0, 0, 0),
     ]
+    assert loader.select(16, 1024, 8192, 0, 0, 0, 1)[2] > 1 and loader.select(32, 2048, 8192, 0, 0, 0, 0)[2] > 1
     dev = []
     for (M, N, K, lc, la, lb) in cases:
         A, B = make_inputs(M, N, K, la, lb, O.F16)
