@@ -121,15 +121,10 @@ size_t out_bytes(int type_idx)
     return (type_idx == 1 || type_idx == 3) ? 4 : 2;
 }
 
-// Library-owned scratch memory, one buffer per device: fp32 partial planes of split-K
-// and zero-padded copies of ragged or misaligned operands.  Allocated on first use,
-// grown when a call needs more (after a device-wide synchronisation, since kernels of
-// earlier calls may still be reading the old buffer), never shrunk.  What a call may do
-// with the buffer is decided by workspace_decide (workspace_policy.hpp).
 // Arrival counters of the whole-K streaming kernel's K slices (one per tile and batch entry
 // of a launch): zero when the code object is loaded, and put back to zero by the workgroup
-// that finishes a tile.  One array per GPU; launches that use it also hold the workspace
-// (their partial tiles live there), so they follow one another as its users do.
+// that finishes a tile.  One array per GPU; launches that use it also hold the scratch
+// buffer below (their partial tiles live there), so they follow one another as its users do.
 constexpr size_t stream_arrival_slots = 4096;
 __attribute__((used)) static __device__ unsigned int stream_arrivals[stream_arrival_slots];
 std::mutex    arrivals_mutex;
@@ -156,6 +151,11 @@ unsigned int* arrivals_of_current_device()
     return arrivals_address[dev];
 }
 
+// Library-owned scratch memory, one buffer per device: fp32 partial planes of split-K
+// and zero-padded copies of ragged or misaligned operands.  Allocated on first use,
+// grown when a call needs more (after a device-wide synchronisation, since kernels of
+// earlier calls may still be reading the old buffer), never shrunk.  What a call may do
+// with the buffer is decided by workspace_decide (workspace_policy.hpp).
 constexpr size_t workspace_first_bytes = size_t{256} << 20;
 constexpr size_t workspace_limit_bytes = size_t{16} << 30;
 constexpr int    max_devices           = 64;
