@@ -448,7 +448,26 @@ launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int 
     {
         return heuristic_plan(m, n, k, lc);
     }
-    return select_plan_from(tuned_table, tuned_count, m, n, k, type_idx, lc, la, lb);
+    plan = select_plan_from(tuned_table, tuned_count, m, n, k, type_idx, lc, la, lb);
+    // The nearest entry may be a small problem's, tuned onto the streaming kernel, which
+    // takes only whole stages of K and wants an operand that is not K-contiguous on a 64-wide
+    // side: a shape that does not fit takes the shape heuristic's plan instead.
+    const model_variant& v = model_variants[plan.variant];
+    if(v.pipeline == 7)
+    {
+        const size_t rows = lc == 0 ? m : n, cols = lc == 0 ? n : m;
+        bool         a_kmajor = la == 0, b_kmajor = lb == 1;
+        if(lc != 0)
+        {
+            std::swap(a_kmajor, b_kmajor);
+        }
+        if(k % 128 != 0 || (!a_kmajor && (v.block_m != 64 || rows % 8 != 0))
+           || (!b_kmajor && (v.block_n != 64 || cols % 8 != 0)))
+        {
+            return heuristic_plan(m, n, k, lc);
+        }
+    }
+    return plan;
 }
 
 } // namespace host

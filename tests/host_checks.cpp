@@ -199,6 +199,13 @@ static int check_select()
         if(tiles[q.variant].pipeline != 0 || q.split_k < 2)
             return fail("select: skinny shape with K = 4000");
     }
+    // next to 1024^3, whose entries run on the streaming kernel: a K that is no multiple of
+    // 128 must not inherit that plan
+    {
+        const launch_plan q = select_plan(81, 1132, 1274, 0, 0, 0, 1);
+        if(tiles[q.variant].pipeline == 7)
+            return fail("select: the streaming kernel's plan for a K it cannot take");
+    }
     // 272 tiles of 256 x 256: the last wave of 16 tiles split
     if(!model_plan(4352, 4096, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline != 5 || p.split_k >= -1)
         return fail("model: tail split");
