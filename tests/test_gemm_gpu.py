@@ -153,6 +153,42 @@ def test_seeded_random_shapes_through_the_default_dispatch(loader, chunk):
             check_against_oracle(gpu[b * M * N:(b + 1) * M * N], As[b], Bs[b], M, N, K, lc, la, lb, din, dout)
 
 
+def test_seeded_random_skinny_and_small_shapes_through_the_default_dispatch(loader):
+    """60 seeded problems of the kinds that the dispatcher's estimate sends to the whole-K
+    streaming kernel or prices against it: a few rows or columns (1 to 128, any value) against
+    a larger operand, and small problems, K in whole stages of 128; all layouts and type
+    pairs, some as strided batches.  Most run on the streaming kernel (several with shared
+    tiles), the rest on what beat it; each element against the oracle."""
+    rng = np.random.RandomState(4711)
+    names = list(TYPE_PAIRS)
+    pipelines = {}
+    for n in range(60):
+        kind = n % 3
+        if kind == 0:
+            M = [1, 2, 3, 5, 8, 13, 16, 24, 31, 32, 33, 48, 64, 65, 100, 128][rng.randint(16)]
+            N = [256, 520, 1000, 1024, 2048, 3000, 4096][rng.randint(7)]
+        elif kind == 1:
+            N = [1, 4, 8, 16, 30, 64, 96, 128][rng.randint(8)]
+            M = [256, 777, 1024, 2048, 4096][rng.randint(5)]
+        else:
+            M = [130, 256, 300, 512, 768, 1000, 1024][rng.randint(7)]
+            N = [130, 256, 384, 512, 1024, 2000][rng.randint(6)]
+        K = 128 * rng.randint(2, 33)
+        lc, la, lb = LAYOUTS8[rng.randint(8)]
+        tname = names[rng.randint(4)]
+        batch = [1, 1, 1, 2, 3][rng.randint(5)]
+        din, dout = TYPE_PAIRS[tname]
+        variant = loader.select(M, N, K, names.index(tname), lc, la, lb, batch)[0]
+        pipelines[loader.variants()[variant].pipeline] = pipelines.get(loader.variants()[variant].pipeline, 0) + 1
+        print(f"random problem {M}x{N}x{K} layouts(C,A,B)=({lc},{la},{lb}) {tname} batch {batch}", flush=True)
+        As = [O.init_matrix(M, K, la, din, seed=300 + n + b) for b in range(batch)]
+        Bs = [O.init_matrix(K, N, lb, din, seed=900 + n + b) for b in range(batch)]
+        gpu = run_gpu(loader, np.concatenate(As), np.concatenate(Bs), M, N, K, lc, la, lb, din, dout, batch=batch)
+        for b in range(batch):
+            check_against_oracle(gpu[b * M * N:(b + 1) * M * N], As[b], Bs[b], M, N, K, lc, la, lb, din, dout)
+    assert pipelines.get(7, 0) >= 25, pipelines  # the streaming kernel is what most of these run on
+
+
 def test_seeded_random_large_shapes_through_the_default_dispatch(loader):
     """The same for 10 problems of many tiles (extents 1500..5200, K 500..4200, all
     alignment classes): every element through the row/column checksums, a 32-row band in
