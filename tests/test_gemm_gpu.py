@@ -877,11 +877,14 @@ def test_scratch_buffer_outlives_a_graph_that_holds_its_address(loader):
 
 def test_replays_from_a_hip_graph(loader):
     """GEMM calls recorded into a HIP graph (whole tiles on the persistent kernel, a ragged
-    shape, and a split-K call whose scratch memory was sized by an eager call before) give
-    the eager results on every replay, with eager work and synchronisations in between."""
+    shape, a split-K call whose scratch memory was sized by an eager call before, and a skinny
+    call whose workgroups share tiles through that memory and the arrival counters) give the
+    eager results on every replay, with eager work and synchronisations in between."""
     import torch
 
-    cases = [(512, 768, 1024, 0, 0, 1), (1000, 1000, 1000, 0, 1, 0), (64, 8192, 8192, 0, 1, 0)]
+    cases = [(512, 768, 1024, 0, 0, 1), (1000, 1000, 1000, 0, 1, 0), (64, 8192, 8192, 0, 1, 0),
+             (16, 1024, 8192, 0, 0, 1)]
+    assert loader.select(16, 1024, 8192, 0, 0, 0, 1)[2] > 1
     ops = []
     for (M, N, K, lc, la, lb) in cases:
         A, B = make_inputs(M, N, K, la, lb, O.F16)
