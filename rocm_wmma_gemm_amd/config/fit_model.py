@@ -125,7 +125,7 @@ def stream_estimate(c: dict, rows: int, cols: int, K: int, a_kmajor: bool, b_kma
     resident = cus * (1 if (bm, bn) == (64, 64) else 2)  # workgroups that the LDS lets run at once
     passes = -(-groups // resident)
     active = min(groups, resident)
-    stages = (K // 128) // slices
+    stages = -(-K // 128) // slices
     wide = cols >= rows  # the large operand is B
     large_kmajor = b_kmajor if wide else a_kmajor
     large_bytes = (bn if wide else bm) * 256

@@ -35,7 +35,7 @@ LAYOUTS = ("rcr", "rrr", "crr")  # A, B, C: r row-major, c column-major
 
 def takes(v, a_kmajor: bool, b_kmajor: bool, M: int, N: int, K: int) -> bool:
     """What csrc/gemm.hip: streaming_ok asks of a problem, for C row-major."""
-    return (K % 128 == 0 and (a_kmajor or (v.block_m == 64 and M % 8 == 0))
+    return (K >= 128 and (K % 8 == 0 or not (a_kmajor or b_kmajor)) and (a_kmajor or (v.block_m == 64 and M % 8 == 0))
             and (b_kmajor or (v.block_n == 64 and N % 8 == 0)))
 
 
@@ -88,7 +88,7 @@ def main(argv=None) -> int:
                 if not takes(v, la == 0, lb == 1, M, N, K):
                     continue
                 for slices in (1, 2, 4, 8):
-                    if (K // 128) % slices or (K // 128) // slices < 2:
+                    if -(-K // 128) % slices or -(-K // 128) // slices < 2:
                         continue
                     rec["t"][f"{v.block_m}x{v.block_n}s{slices}"] = round(timed(
                         lambda: L.run_variant(v.index, 1, slices, C, A, B, M, N, K, lc, la, lb)), 2)

@@ -190,11 +190,12 @@ def split_feasible(t: Tile, swizzle: int, split: int, rows: int, cols: int, K: i
         return False
     if t.pipeline == 7:
         # a workgroup per tile over the whole K, or 2, 4 or 8 that share a tile and add their
-        # parts up inside the launch (whole stages each, at least two; a counter per tile):
+        # parts up inside the launch (whole stages of 128 each, at least two, the last of K may
+        # be cut short; a counter per tile):
         # no band height; worth a try when a 256 x 256 tiling leaves most compute units
         # without a tile
-        stages = K // 128
-        return swizzle == (1 if tiles <= 8 else 4) and K % 128 == 0 \
+        stages = -(-K // 128)
+        return swizzle == (1 if tiles <= 8 else 4) and K >= 128 and K % 8 == 0 \
             and -(-rows // 256) * -(-cols // 256) < CUS // 2 \
             and (split == 1 or (split in (2, 4, 8) and stages % split == 0 and stages // split >= 2
                                 and tiles <= 4096 and tiles * split <= 4 * CUS))

@@ -334,13 +334,16 @@ bool stream_plan(size_t rows, size_t cols, size_t k, bool a_kmajor, bool b_kmajo
                  launch_plan* out, double* microseconds)
 {
     // skinny, or so small that tiles of 64 x 64 do not outnumber the compute units of an MI355X
-    if(k % 128 != 0 || k < 256 || rows == 0 || cols == 0 || (rows > 128 && cols > 128 && rows * cols > (size_t{1} << 20)))
+    // (K in stages of 128, the last of which may be cut short; rows of a K-contiguous operand
+    // must stay 16-byte aligned)
+    if(k < 256 || ((a_kmajor || b_kmajor) && k % 8 != 0) || rows == 0 || cols == 0
+       || (rows > 128 && cols > 128 && rows * cols > (size_t{1} << 20)))
     {
         return false;
     }
     const model_stream& c      = model_measured.stream;
     const size_t        cus    = cus_of_device != 0 ? cus_of_device : static_cast<size_t>(model_measured.compute_units);
-    const size_t        stages = k / 128;
+    const size_t        stages = (k + 127) / 128;
     const bool          wide   = cols >= rows; // the large operand is B
     const int           count  = static_cast<int>(sizeof(model_variants) / sizeof(model_variants[0]));
     bool                found  = false;
@@ -441,8 +444,8 @@ launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int 
     {
         return plan;
     }
-    // A skinny shape that neither has an entry nor suits the model (K no multiple of 128,
-    // odd extents): the nearest tuned entry would be a large square's plan, 256 x 256 tiles
+    // A skinny shape that neither has an entry nor suits the model (rows that are not 16-byte
+    // aligned): the nearest tuned entry would be a large square's plan, 256 x 256 tiles
     // for a handful of rows; the shape heuristic cuts K over the compute units instead.
     if(std::min(m, n) <= 64 && std::max(m, n) >= 512)
     {
@@ -450,8 +453,8 @@ launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int 
     }
     plan = select_plan_from(tuned_table, tuned_count, m, n, k, type_idx, lc, la, lb);
     // The nearest entry may be a small problem's, tuned onto the streaming kernel, which
-    // takes only whole stages of K and wants an operand that is not K-contiguous on a 64-wide
-    // side: a shape that does not fit takes the shape heuristic's plan instead.
+    // wants 16-byte aligned rows and an operand that is not K-contiguous on a 64-wide side: a
+    // shape that does not fit takes the shape heuristic's plan instead.
     const model_variant& v = model_variants[plan.variant];
     if(v.pipeline == 7)
     {
@@ -461,7 +464,7 @@ launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int 
         {
             std::swap(a_kmajor, b_kmajor);
         }
-        if(k % 128 != 0 || (!a_kmajor && (v.block_m != 64 || rows % 8 != 0))
+        if(k < 128 || ((a_kmajor || b_kmajor) && k % 8 != 0) || (!a_kmajor && (v.block_m != 64 || rows % 8 != 0))
            || (!b_kmajor && (v.block_n != 64 || cols % 8 != 0)))
         {
             return heuristic_plan(m, n, k, lc);

@@ -93,7 +93,8 @@ launch_plan heuristic_plan(size_t m, size_t n, size_t k, int lc);
 bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_plan* out, size_t batch = 1,
                 size_t cus = 0);
 // The streaming kernel's plans alone (skinny shapes: one extent at most 128, or small ones:
-// at most 2^20 elements of C; K whole stages of 128), in kernel space (rows x cols, the operands' K-contiguity): the cheapest by
+// at most 2^20 elements of C; K at least 256, a multiple of 8 where an operand is
+// K-contiguous), in kernel space (rows x cols, the operands' K-contiguity): the cheapest by
 // estimate and its microseconds; false when no compiled variant takes the problem.
 bool stream_plan(size_t rows, size_t cols, size_t k, bool a_kmajor, bool b_kmajor, size_t batch, size_t cus,
                  launch_plan* out, double* microseconds);

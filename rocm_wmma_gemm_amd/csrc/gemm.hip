@@ -426,11 +426,11 @@ bool spans_fit(const variant_desc& v, bool a_kmajor, bool b_kmajor, size_t lda, 
 }
 
 // What the whole-K streaming kernel (pipeline 7) takes: an operand that is not K-contiguous
-// 64 wide in the tile, with 16-byte aligned k rows; K whole stages of 128,
-// 16-byte aligned rows, and a stage of a tile within reach of a 31-bit offset.
+// 64 wide in the tile, with 16-byte aligned k rows; at least one stage of 128 of K (the last
+// may be cut short); 16-byte aligned rows, and a stage of a tile within reach of a 31-bit offset.
 bool streaming_ok(const kernel_problem& p, const variant_desc& v)
 {
-    if(!(p.K >= 128 && p.K % 128 == 0 && aligned16(p.A) && aligned16(p.B)
+    if(!(p.K >= 128 && ((!p.a_kmajor && !p.b_kmajor) || p.K % 8 == 0) && aligned16(p.A) && aligned16(p.B)
          && (p.batch == 1 || (p.stride_a % 8 == 0 && p.stride_b % 8 == 0))))
     {
         return false;
@@ -472,7 +472,7 @@ int launch_streaming(int type_idx, const launch_plan& plan, const kernel_problem
     const size_t tiles       = grid_m * grid_n;
     const size_t nb_max      = std::min<size_t>(65535, p.batch);
     size_t       slices      = plan.split_k > 1 ? static_cast<size_t>(plan.split_k) : 1;
-    const size_t stages      = p.K / 128;
+    const size_t stages      = (p.K + 127) / 128;
     const size_t tile_floats = static_cast<size_t>(v.block_m) * v.block_n;
     if(slices > 1 && (slices > 8 /* device::stream_gemm::MAX_SLICES */ || stages % slices != 0 || tiles * nb_max > stream_arrival_slots || tiles * slices > 0x7fffffffull))
     {

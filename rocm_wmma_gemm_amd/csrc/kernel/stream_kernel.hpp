@@ -24,7 +24,8 @@
 //     whole tile on v_mfma_f32_16x16x32; at the end the four partial tiles are added in
 //     wave order through LDS and the sum is converted and stored;
 //   - rows past M or N are read as zeros (the buffer descriptors end with the operand)
-//     and not stored;
+//     and not stored; so are the columns of a last stage past K (K a multiple of 8 where an
+//     operand is K-contiguous, so that its rows stay 16-byte aligned);
 //   - where the tiles are too few for the compute units (a 64-wide side on N = 8192 gives
 //     128 of them), args.k_slices workgroups share a tile, each with a run of the stages:
 //     every one writes its fp32 tile to args.partials, counts itself in at the tile's
@@ -186,21 +187,30 @@ struct stream_gemm
         const unsigned int stage_b = B_KMAJOR ? (unsigned int)ROW_BYTES : (unsigned int)(BK * ldb * 2);
 
         // this workgroup's run of the K / BK stages
-        const int stages_all = args.K / BK, stages_per = (stages_all + args.k_slices - 1) / args.k_slices;
+        // (K need not be whole stages: of a last stage that K cuts short, the lanes of a
+        // K-contiguous operand whose 8 columns lie past K load out of range and get zeros;
+        // the k rows of an M/N-contiguous operand past K lie past the end of its descriptor)
+        const int          k_tail     = args.K % BK;
+        const unsigned int past_range = 0x80000000u;
+        const unsigned int voff_a_tail = A_KMAJOR && k_tail != 0 && chunk * 8 >= k_tail ? past_range : voff_a;
+        const unsigned int voff_b_tail = B_KMAJOR && k_tail != 0 && chunk * 8 >= k_tail ? past_range : voff_b;
+        const int stages_all = (args.K + BK - 1) / BK, stages_per = (stages_all + args.k_slices - 1) / args.k_slices;
         const int first      = slice * stages_per;
         const int stages     = stages_all - first < stages_per ? stages_all - first : stages_per; // >= 1 (host)
         auto      issue      = [&](int stage, int slot_index) {
             const unsigned int base = lds_addr + slot_index * STAGE + wave * 1024;
+            const bool         last = first + stage == stages_all - 1; // the stage that K may cut short
+            const unsigned int va = last ? voff_a_tail : voff_a, vb = last ? voff_b_tail : voff_b;
 #pragma unroll
             for(int i = 0; i < LOADS_A; ++i)
             {
-                load_block(base + i * 4096, voff_a, rsrc_a,
+                load_block(base + i * 4096, va, rsrc_a,
                            __builtin_amdgcn_readfirstlane((unsigned int)(first + stage) * stage_a + i * step_a));
             }
 #pragma unroll
             for(int i = 0; i < LOADS_B; ++i)
             {
-                load_block(base + A_BYTES + i * 4096, voff_b, rsrc_b,
+                load_block(base + A_BYTES + i * 4096, vb, rsrc_b,
                            __builtin_amdgcn_readfirstlane((unsigned int)(first + stage) * stage_b + i * step_b));
             }
         };

@@ -192,20 +192,23 @@ static int check_select()
         return fail("model: 512 x 2048 x 2048 streams");
     if(!model_plan(2048, 1024, 1024, 0, 0, 1, &p) || tiles[p.variant].pipeline == 7)
         return fail("model: 2048 x 1024 x 1024 is too large for a workgroup per small tile");
-    // a skinny shape the model does not take (K no multiple of 128) and the table does not
-    // hold: the shape heuristic's split, not the nearest large square's plan
+    // a skinny shape the model does not take (K-contiguous rows of 4001 elements) and the
+    // table does not hold: the shape heuristic's split, not the nearest large square's plan
     {
-        const launch_plan q = select_plan(8, 4096, 4000, 0, 0, 0, 1);
+        const launch_plan q = select_plan(8, 4096, 4001, 0, 0, 0, 1);
         if(tiles[q.variant].pipeline != 0 || q.split_k < 2)
-            return fail("select: skinny shape with K = 4000");
+            return fail("select: skinny shape with K = 4001");
     }
-    // next to 1024^3, whose entries run on the streaming kernel: a K that is no multiple of
-    // 128 must not inherit that plan
+    // next to 1024^3, whose entries run on the streaming kernel: K-contiguous rows that are
+    // not 16-byte aligned must not inherit that plan
     {
         const launch_plan q = select_plan(81, 1132, 1274, 0, 0, 0, 1);
         if(tiles[q.variant].pipeline == 7)
-            return fail("select: the streaming kernel's plan for a K it cannot take");
+            return fail("select: the streaming kernel's plan for rows it cannot take");
     }
+    // K in stages of 128 of which the last is cut short
+    if(!model_plan(16, 4096, 1000, 0, 0, 1, &p) || tiles[p.variant].pipeline != 7)
+        return fail("model: a skinny shape with K = 1000 streams");
     // 272 tiles of 256 x 256: the last wave of 16 tiles split
     if(!model_plan(4352, 4096, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline != 5 || p.split_k >= -1)
         return fail("model: tail split");

@@ -347,14 +347,16 @@ def test_whole_k_streaming_kernel_agrees_with_oracle(loader):
     over the whole K, ring of up to 8 stages): every tile, skinny M and skinny N (a
     column-major C runs as the transposed problem), the large operand K-contiguous or
     contiguous along N, ragged M and N (rows past the edge are read as zeros and not
-    stored), one stage and many, a strided batch, all type pairs, and -1 for what it does
-    not take (an operand that is not K-contiguous on a 32-wide side of the tile, K no
-    multiple of 128)."""
+    stored), one stage and many, a last stage that K cuts short, a strided batch, all type
+    pairs, and -1 for what it does not take (an operand that is not K-contiguous on a 32-wide
+    side of the tile, K-contiguous rows that are not 16-byte aligned, less than a stage of K)."""
     import torch
 
     stream = [v for v in loader.variants() if v.pipeline == 7]
     assert {(v.block_m, v.block_n) for v in stream} == {(32, 32), (64, 32), (32, 64), (64, 64)}
-    shapes = [(16, 2048, 1024), (100, 1000, 384), (128, 512, 128), (33, 65, 2048), (2048, 24, 512)]
+    # (K = 200, 1000 and 1352: a last stage that K cuts short; 1001 where no operand is K-contiguous)
+    shapes = [(16, 2048, 1024), (100, 1000, 384), (128, 512, 128), (33, 65, 2048), (2048, 24, 512),
+              (40, 520, 200), (1000, 1000, 1000), (64, 128, 1352)]
     ran = set()
     for v in stream:
         for (M, N, K) in shapes:
@@ -398,7 +400,8 @@ def test_whole_k_streaming_kernel_agrees_with_oracle(loader):
     dA = torch.zeros(64 * 256, dtype=torch.float16, device="cuda")
     dC = torch.zeros(64 * 64, dtype=torch.float16, device="cuda")
     assert loader.run_variant(v.index, 1, 1, dC, dA, dA, 64, 64, 256, 0, 1, 0) == -1   # 32-wide sides, neither operand K-contiguous
-    assert loader.run_variant(v.index, 1, 1, dC, dA, dA, 64, 64, 200, 0, 0, 1) == -1   # K % 128 != 0
+    assert loader.run_variant(v.index, 1, 1, dC, dA, dA, 64, 64, 204, 0, 0, 1) == -1   # K-contiguous rows of 408 bytes
+    assert loader.run_variant(v.index, 1, 1, dC, dA, dA, 64, 64, 120, 0, 0, 1) == -1   # less than a stage of K
 
 
 def test_workgroups_that_share_a_tile_of_the_streaming_kernel(loader):
@@ -412,7 +415,7 @@ def test_workgroups_that_share_a_tile_of_the_streaming_kernel(loader):
     import torch
 
     stream = [v for v in loader.variants() if v.pipeline == 7]
-    shapes = [(16, 1024, 2048), (40, 200, 1024), (128, 256, 4096), (1000, 24, 2048)]
+    shapes = [(16, 1024, 2048), (40, 200, 1024), (128, 256, 4096), (1000, 24, 2048), (24, 512, 1000)]
     for v in stream:
         for split in (2, 4, 8):
             for (M, N, K) in shapes:
