@@ -130,20 +130,26 @@ def stream_estimate(c: dict, rows: int, cols: int, K: int, a_kmajor: bool, b_kma
     large_kmajor = b_kmajor if wide else a_kmajor
     large_bytes = (bn if wide else bm) * 256
     sharing = -(-rows // bm) if wide else -(-cols // bn)  # workgroups that read the same panel of it
-    other = (0 if a_kmajor else 1) + (0 if b_kmajor else 1)
+    # (transposing reads: by the width of the side they fill, in units of 64)
+    other = (0 if a_kmajor else bm / 64) + (0 if b_kmajor else bn / 64)
     per_cu = c["stage_us"][f"{bm}x{bn}"] * (1.0 + c["transposed_operand"] * other)
     small_bytes = (bm if wide else bn) * 256  # every workgroup reads its rows of the small operand, from L2
     # (the workgroups that read the same panel find only part of it in L2)
     sharing = 1.0 + (sharing - 1.0) * c["panel_sharing"]
     rate = c["bytes_per_us_kmajor" if large_kmajor else "bytes_per_us_other"]
+    if not large_kmajor and (bn if wide else bm) == 32:
+        rate *= c["half_line"]  # k rows of 64 bytes: half a cache line per request
     if max(rows, cols) * K * 2 > 256 << 20:
         # the large operand does not fit the memory-side cache, which serves part of a
         # repeated call on a smaller one (not fitted: left free it soaks up other effects)
         rate *= c["beyond_cache"]
+    l2_rate = c["bytes_per_us_l2"]
+    if not (a_kmajor if wide else b_kmajor) and (bm if wide else bn) == 32:
+        l2_rate *= c["half_line"]
     from_memory = (large_bytes * (active / sharing) / rate
-                   + small_bytes * active / c["bytes_per_us_l2"])
+                   + small_bytes * active / l2_rate)
     return (c["launch_us"] + passes * (c["fill_us"] + stages * max(per_cu, from_memory))
-            + (c["exchange_us"] if slices > 1 else 0.0))
+            + (c["exchange_us"] + c["exchange_us_per_kb"] * slices * bm * bn * 4 / 1024 if slices > 1 else 0.0))
 
 
 def stream_plans(rec: dict):
@@ -160,7 +166,7 @@ def fit_stream(records: list, start: dict) -> dict:
     from scipy.optimize import least_squares
 
     keys = ["launch_us", "fill_us", "exchange_us", "bytes_per_us_kmajor", "bytes_per_us_other", "bytes_per_us_l2",
-            "transposed_operand", "panel_sharing"]
+            "transposed_operand", "panel_sharing", "half_line", "exchange_us_per_kb"]
 
     def unpack(p):
         c = {k: float(v) for k, v in zip(keys, p)}
@@ -179,7 +185,7 @@ def fit_stream(records: list, start: dict) -> dict:
         return [math.log(stream_estimate(c, *row[:8]) / row[8]) for row in rows]
 
     p0 = [start[k] for k in keys] + [start["stage_us"][t] for t in STREAM_TILES]
-    res = least_squares(residuals, p0, bounds=([0.0] * len(p0), [20, 10, 30, 2e7, 2e7, 2e8, 3, 1] + [2.0] * len(STREAM_TILES)))
+    res = least_squares(residuals, p0, bounds=([0.0] * len(p0), [20, 10, 30, 2e7, 2e7, 2e8, 3, 1, 1, 1] + [2.0] * len(STREAM_TILES)))
     c = unpack(res.x)
     for k in ("launch_us", "fill_us", "exchange_us"):
         c[k] = round(c[k], 2)
@@ -187,6 +193,8 @@ def fit_stream(records: list, start: dict) -> dict:
         c[k] = round(c[k], -4)
     c["transposed_operand"] = round(c["transposed_operand"], 3)
     c["panel_sharing"] = round(c["panel_sharing"], 3)
+    c["half_line"] = round(c["half_line"], 3)
+    c["exchange_us_per_kb"] = round(c["exchange_us_per_kb"], 4)
     c["stage_us"] = {t: round(v, 4) for t, v in c["stage_us"].items()}
     return c
 
@@ -227,7 +235,7 @@ def main(argv=None) -> int:
         print(json.dumps(new, indent=1))
         print(f"regret of the estimate's pick over {len(records)} problems: mean {mean:.3f}, worst {worst:.2f}")
         if a.write:
-            new["fitted_from"] = f"{os.path.basename(a.log)}: {sum(len(r['t']) for r in records)} timings"
+            new["fitted_from"] = f"{os.path.basename(a.log)}: {sum(len(r['t']) for r in records)} timings (beyond_cache set by hand)"
             model["stream"] = new
             with open(a.model, "w") as f:
                 json.dump(model, f, indent=4)

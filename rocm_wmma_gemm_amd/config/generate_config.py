@@ -111,9 +111,10 @@ def render_model(m: dict) -> list[str]:
             steps.append(f"    {{{int(pipe)}, {bm}, {bn}, {float(us)!r}, {float(m['item_us'][pipe])!r}}},")
     st = m["stream"]
     stream = ["constexpr model_stream model_stream_constants = {"
-              + ", ".join(repr(float(st[k])) for k in ("launch_us", "fill_us", "exchange_us", "bytes_per_us_kmajor",
-                                                        "bytes_per_us_other", "bytes_per_us_l2",
-                                                        "transposed_operand", "panel_sharing", "beyond_cache"))
+              + ", ".join(repr(float(st[k])) for k in ("launch_us", "fill_us", "exchange_us", "exchange_us_per_kb",
+                                                        "bytes_per_us_kmajor", "bytes_per_us_other", "bytes_per_us_l2",
+                                                        "transposed_operand", "panel_sharing", "half_line",
+                                                        "beyond_cache"))
               + ", {" + ", ".join(repr(float(st["stage_us"][t])) for t in ("32x32", "64x32", "32x64", "64x64")) + "}};"]
     return ([f"constexpr int model_compute_units = {int(m['compute_units'])};"]
             + [f"constexpr double model_{k} = {float(m[k])!r};" for k in

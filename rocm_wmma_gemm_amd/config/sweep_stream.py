@@ -4,7 +4,7 @@
     python sweep_stream.py --out stream_sweep.json [--type f16_f16] [--reps 15]
 
 For each shape M x N x K of a grid of decode-like problems (M = 8..128 against N x K from
-1024 to 28672) and each of three layout triples (both operands K-contiguous, one, neither)
+1024 to 28672) and each of four layout triples (both operands K-contiguous, either, neither)
 it runs every compiled pipeline-7 variant that takes the layout with 1, 2, 4 and 8
 workgroups per tile through the tuner hook (rocm_wmma_gemm_run_variant) and writes, per
 problem, the time of every plan, of the default dispatch and of hipBLASLt.  fit_model.py
@@ -30,13 +30,13 @@ SHAPES = [(M, N, K) for M in (8, 16, 32, 64, 128)
 SMALL_SHAPES = [(256, 256, 1024), (512, 512, 512), (512, 512, 4096), (768, 768, 768), (1024, 1024, 1024),
                 (1024, 1024, 4096), (1536, 1536, 1536), (2048, 2048, 2048), (2048, 1024, 1024), (512, 2048, 2048),
                 (1024, 4096, 1024), (2048, 2048, 512), (256, 4096, 2048), (384, 1536, 1536), (3072, 1024, 1024)]
-LAYOUTS = ("rcr", "rrr", "crr")  # A, B, C: r row-major, c column-major
+LAYOUTS = ("rcr", "rrr", "ccr", "crr")  # A, B, C: r row-major, c column-major
 
 
 def takes(v, a_kmajor: bool, b_kmajor: bool, M: int, N: int, K: int) -> bool:
     """What csrc/gemm.hip: streaming_ok asks of a problem, for C row-major."""
-    return (K >= 128 and (K % 8 == 0 or not (a_kmajor or b_kmajor)) and (a_kmajor or (v.block_m == 64 and M % 8 == 0))
-            and (b_kmajor or (v.block_n == 64 and N % 8 == 0)))
+    return (K >= 128 and (K % 8 == 0 or not (a_kmajor or b_kmajor)) and (a_kmajor or M % 8 == 0)
+            and (b_kmajor or N % 8 == 0))
 
 
 def main(argv=None) -> int:

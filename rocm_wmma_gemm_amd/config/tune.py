@@ -144,10 +144,8 @@ def tile_feasible(t: Tile, a_kmajor: bool, b_kmajor: bool) -> bool:
     if t.block_m % (32 * t.warps_m) or t.block_n % (32 * t.warps_n):
         return False
     if t.pipeline == 7:
-        # whole-K streaming kernel: small tiles, stages of 128, an operand that is not
-        # K-contiguous on a 64-wide side of the tile
-        return ((a_kmajor or t.block_m == 64) and (b_kmajor or t.block_n == 64)
-                and t.block_k == 128 and t.block_m in (32, 64) and t.block_n in (32, 64)
+        # whole-K streaming kernel: small tiles, stages of 128, either layout of an operand
+        return (t.block_k == 128 and t.block_m in (32, 64) and t.block_n in (32, 64)
                 and (t.warps_m, t.warps_n) == (t.block_m // 32, t.block_n // 32))
     if t.block_k == 128:
         return False

@@ -355,20 +355,24 @@ bool stream_plan(size_t rows, size_t cols, size_t k, bool a_kmajor, bool b_kmajo
             continue;
         }
         const size_t bm = v.block_m, bn = v.block_n;
-        // an operand that is not K-contiguous: 64 wide in the tile, rows of 16-byte pieces
-        if((!a_kmajor && (bm != 64 || rows % 8 != 0)) || (!b_kmajor && (bn != 64 || cols % 8 != 0)))
+        // an operand that is not K-contiguous: k rows of 16-byte pieces
+        if((!a_kmajor && rows % 8 != 0) || (!b_kmajor && cols % 8 != 0))
         {
             continue;
         }
         const int    slot    = (bm == 64 ? 1 : 0) + (bn == 64 ? 2 : 0);
         const size_t tm      = ceil_div(rows, bm), tn = ceil_div(cols, bn), tiles = tm * tn;
-        const double other   = (a_kmajor ? 0.0 : 1.0) + (b_kmajor ? 0.0 : 1.0);
+        // (transposing reads: by the width of the side they fill, in units of 64)
+        const double other   = (a_kmajor ? 0.0 : static_cast<double>(bm) / 64.0) + (b_kmajor ? 0.0 : static_cast<double>(bn) / 64.0);
         const double per_cu  = c.stage_us[slot] * (1.0 + c.transposed_operand * other);
         const double large   = static_cast<double>(wide ? bn : bm) * 256.0;
         const double small   = static_cast<double>(wide ? bm : bn) * 256.0;
         const double sharing = 1.0 + (static_cast<double>(wide ? tm : tn) - 1.0) * c.panel_sharing;
-        const double rate    = ((wide ? b_kmajor : a_kmajor) ? c.bytes_per_us_kmajor : c.bytes_per_us_other)
+        const bool   large_kmajor = wide ? b_kmajor : a_kmajor, small_kmajor = wide ? a_kmajor : b_kmajor;
+        const double rate    = (large_kmajor ? c.bytes_per_us_kmajor : c.bytes_per_us_other)
+                            * (!large_kmajor && (wide ? bn : bm) == 32 ? c.half_line : 1.0)
                             * (std::max(rows, cols) * k * 2 > (size_t{256} << 20) ? c.beyond_cache : 1.0);
+        const double l2_rate = c.bytes_per_us_l2 * (!small_kmajor && (wide ? bm : bn) == 32 ? c.half_line : 1.0);
         for(size_t s = 1; s <= 8; s *= 2)
         {
             // (the counters of the tiles that several workgroups share: 4096 a launch)
@@ -380,10 +384,10 @@ bool stream_plan(size_t rows, size_t cols, size_t k, bool a_kmajor, bool b_kmajo
             const size_t groups   = tiles * s * batch;
             const size_t resident = cus * ((bm == 64 && bn == 64) ? 1 : 2);
             const double active   = static_cast<double>(groups < resident ? groups : resident);
-            const double stage  = std::max(per_cu, large * (active / sharing) / rate + small * active / c.bytes_per_us_l2);
+            const double stage  = std::max(per_cu, large * (active / sharing) / rate + small * active / l2_rate);
             const double t      = c.launch_us
                              + static_cast<double>(ceil_div(groups, resident)) * (c.fill_us + static_cast<double>(stages / s) * stage)
-                             + (s > 1 ? c.exchange_us : 0.0);
+                             + (s > 1 ? c.exchange_us + c.exchange_us_per_kb * static_cast<double>(s * bm * bn * 4) / 1024.0 : 0.0);
             if(!found || t < *microseconds)
             {
                 found         = true;
@@ -453,7 +457,7 @@ launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int 
     }
     plan = select_plan_from(tuned_table, tuned_count, m, n, k, type_idx, lc, la, lb);
     // The nearest entry may be a small problem's, tuned onto the streaming kernel, which
-    // wants 16-byte aligned rows and an operand that is not K-contiguous on a 64-wide side: a
+    // wants 16-byte aligned rows of either kind: a
     // shape that does not fit takes the shape heuristic's plan instead.
     const model_variant& v = model_variants[plan.variant];
     if(v.pipeline == 7)
@@ -464,8 +468,8 @@ launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int 
         {
             std::swap(a_kmajor, b_kmajor);
         }
-        if(k < 128 || ((a_kmajor || b_kmajor) && k % 8 != 0) || (!a_kmajor && (v.block_m != 64 || rows % 8 != 0))
-           || (!b_kmajor && (v.block_n != 64 || cols % 8 != 0)))
+        if(k < 128 || ((a_kmajor || b_kmajor) && k % 8 != 0) || (!a_kmajor && rows % 8 != 0)
+           || (!b_kmajor && cols % 8 != 0))
         {
             return heuristic_plan(m, n, k, lc);
         }

@@ -54,12 +54,15 @@ struct model_step
 struct model_stream
 {
     double launch_us, fill_us; // per launch; per pass over the compute units (the ring fills)
-    double exchange_us; // several workgroups per tile: the partial tiles through memory
+    double exchange_us; // several workgroups per tile: the partial tiles through memory ...
+    double exchange_us_per_kb; // ... and per KiB of them that the last workgroup adds up
     double bytes_per_us_kmajor, bytes_per_us_other; // stream of the large operand from memory
     double bytes_per_us_l2; // the small operand, which every workgroup reads from L2
     double transposed_operand; // relative cost of a stage per operand that is not K-contiguous
     double panel_sharing; // how much of a panel of the large operand that g workgroups read
                           // is fetched once for all: it counts as fetched g / (1 + (g - 1) x this) times
+    double half_line; // factor on a rate for an operand contiguous along M or N on a 32-wide side
+                      // of the tile: requests of 64 bytes, half a cache line
     double beyond_cache; // factor on the two rates from memory for a large operand over 256 MB
                          // (set by hand, not fitted)
     double stage_us[4]; // per stage of 128 of one compute unit: tiles 32x32, 64x32, 32x64, 64x64

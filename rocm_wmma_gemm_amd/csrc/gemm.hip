@@ -426,7 +426,7 @@ bool spans_fit(const variant_desc& v, bool a_kmajor, bool b_kmajor, size_t lda, 
 }
 
 // What the whole-K streaming kernel (pipeline 7) takes: an operand that is not K-contiguous
-// 64 wide in the tile, with 16-byte aligned k rows; at least one stage of 128 of K (the last
+// with 16-byte aligned k rows; at least one stage of 128 of K (the last
 // may be cut short); 16-byte aligned rows, and a stage of a tile within reach of a 31-bit offset.
 bool streaming_ok(const kernel_problem& p, const variant_desc& v)
 {
@@ -435,7 +435,7 @@ bool streaming_ok(const kernel_problem& p, const variant_desc& v)
     {
         return false;
     }
-    if((!p.a_kmajor && (v.block_m != 64 || p.M % 8 != 0)) || (!p.b_kmajor && (v.block_n != 64 || p.N % 8 != 0)))
+    if((!p.a_kmajor && p.M % 8 != 0) || (!p.b_kmajor && p.N % 8 != 0))
     {
         return false;
     }

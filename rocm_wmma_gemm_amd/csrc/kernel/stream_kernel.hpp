@@ -13,9 +13,10 @@
 //     and its rows of the small operand from L2 (every workgroup reads all of the small
 //     operand: M x K x 2 bytes each, which is why this pays only while M is small);
 //   - an operand may be K-contiguous (a row of a stage is 256 contiguous bytes, two whole
-//     cache lines) or contiguous along M or N, in which case its side of the tile is 64
-//     wide, so that a k row of the tile is one whole cache line, and the fragments are
-//     transposed on the way to registers by ds_read_b64_tr_b16;
+//     cache lines) or contiguous along M or N, in which case a k row of the tile is 128
+//     bytes (a 64-wide side: one whole cache line, what the large operand wants) or 64 (a
+//     32-wide side: half the waste where the small operand has 16 rows), and the fragments
+//     are transposed on the way to registers by ds_read_b64_tr_b16;
 //   - the LDS holds a ring of 3 or 4 stages of BK = 128 per workgroup, two workgroups to a
 //     compute unit (48..96 KB of loads in flight per compute unit: what it takes to cover
 //     the latency of HBM at 20..40 GB/s per compute unit), filled by buffer_load ... lds,
@@ -36,8 +37,12 @@
 // LDS layout of a stage: the A tile (BM rows), then the B tile (BN rows).  K-contiguous
 // operand: a row is 16 chunks of 16 bytes, chunk c of row r in slot c ^ (r mod 16), so
 // that the 16 rows a fragment read touches per k chunk fall on 16 different slots (all 64
-// banks once).  M/N-contiguous operand: 128 k rows of 64 elements (128 bytes), as they lie
-// in memory.
+// banks once).  M/N-contiguous operand: 128 k rows of 64 or 32 elements; the 32-byte
+// pieces of k row k are permuted within the row (mn_piece), so that the 4 k rows x 32
+// bytes that 16 lanes of a transposing read touch, and those of the next 16 lanes 8 rows
+// further on, fall on different banks (64 wide, in memory order, they are 4-way
+// conflicts: 16 x 8192 x 8192 with B row-major 29.6 us, with the pieces permuted 28.1 us;
+// B column-major, whose fragments are plain 16-byte reads, 24.3 us).
 //
 // Role with respect to the reference: as the other kernels, its gemm_impl (reference
 // rocm_wmma_gemm/include/rocm_wmma_gemm/kernel/kernel.hpp:108-556); the reference has no
@@ -69,7 +74,9 @@ struct stream_gemm
     // share a compute unit (all tiles but 64 x 64, whose three stages take 96 KB): while one
     // fills its ring or adds up and stores its tile, the other keeps the loads coming.
     // Against one workgroup per compute unit with a ring of 144 KB, same plans: +9.6 %
-    // (geometric mean over 135 skinny problems), 16 x 28672 x 8192 4.1 -> 4.6 TB/s.
+    // (geometric mean over 135 skinny problems), 16 x 28672 x 8192 4.1 -> 4.6 TB/s.  (A ring
+    // of 152 KB is no better where a compute unit has one workgroup anyway: 128 tiles of
+    // 16 x 8192 x 8192, 24.3 us with 3 stages of 32 x 64, 25.7 us with 6.)
     static constexpr int RING_KB   = 76;
     static constexpr int DEPTH_FIT = (RING_KB * 1024) / STAGE < 3 ? 3 : (RING_KB * 1024) / STAGE;
     static constexpr int DEPTH     = DEPTH_FIT < 8 ? DEPTH_FIT : 8;
@@ -78,14 +85,13 @@ struct stream_gemm
     static constexpr int TN        = BN / 16;
     // 1 KiB loads (4 rows) of a stage per wave: load q of an operand covers rows 4q .. 4q+3
     // and belongs to wave q mod 4
-    // (M/N-contiguous, 64 wide: load q covers k rows 8q .. 8q+7, 16 loads a stage)
+    // (M/N-contiguous, W wide: load q covers the 512 / W k rows from (512 / W) q on, W / 4
+    // loads a stage)
     static constexpr int LOADS_A = BM / 16;
     static constexpr int LOADS_B = BN / 16;
     static constexpr int PER     = LOADS_A + LOADS_B;
     static constexpr int MAX_SLICES = 8; // workgroups that may share a tile (args.k_slices)
     static_assert((BM == 32 || BM == 64) && (BN == 32 || BN == 64), "tiles of 32 or 64 rows and columns");
-    static_assert((A_KMAJOR || BM == 64) && (B_KMAJOR || BN == 64),
-                  "a k row of an M/N-contiguous tile is one 128-byte line");
     static_assert(DEPTH >= 3 && (DEPTH - 1) * PER < 64, "ring depth against the 6-bit vmcnt");
     static_assert(WAVES * BM * BN * 4 <= LDS_BYTES, "the partial tiles of the waves reuse the ring");
 
@@ -117,6 +123,82 @@ struct stream_gemm
                      :
                      : [ldsb] "s"(lds_block), [voff] "v"(voff), [rsrc] "s"(rsrc), [soff] "s"(soff)
                      : "memory");
+    }
+
+    // M/N-contiguous operand, W elements wide (a k row of 2 W bytes; 512 / W k rows per 1 KiB
+    // load).  Where the 32-byte pieces of k row k lie within the row: piece j in place
+    // j ^ mn_piece(k).  A transposing read touches, per 16 lanes, 32 bytes of 4 consecutive
+    // k rows, and the next 16 lanes the same 8 rows further on: W = 64, rows 128 bytes apart,
+    // rows k and k + 2 and the rows 8 further all start on the same bank; W = 32, rows k and
+    // k + 4 do (the 4 rows of a group do not meet), and the rows 8 further.
+    template<int W>
+    __device__ __forceinline__ static int mn_piece(int k)
+    {
+        return W == 64 ? ((k & 3) ^ ((k >> 3) & 1)) : ((k >> 3) & 1);
+    }
+
+    // byte offset of lane l's 16 bytes of load `wave` (+ 4 i) from the operand's stage origin
+    template<int W>
+    __device__ __forceinline__ static unsigned int mn_load_offset(int lane, int wave, long long ld)
+    {
+        constexpr int LANES_PER_ROW = W / 8, ROWS_PER_LOAD = 512 / W;
+        const int     k      = ROWS_PER_LOAD * wave + lane / LANES_PER_ROW; // (mod 16 as for every i)
+        const int     place  = (lane % LANES_PER_ROW) >> 1;
+        const int     piece  = place ^ mn_piece<W>(k);
+        return (unsigned int)((k * ld + piece * 16 + (lane & 1) * 8) * 2);
+    }
+
+    // LDS offset, within the operand's part of a stage, of what lane (sub, slot) addresses for
+    // column piece 0 of its transposing reads
+    template<int W>
+    __device__ __forceinline__ static int mn_read_offset(int wave, int sub, int slot)
+    {
+        const int k = 32 * wave + 8 * sub + (slot >> 2);
+        return k * (2 * W) + mn_piece<W>(k) * 32 + (slot & 3) * 8;
+    }
+
+    // The fragments of a 64-wide side: column piece j of this lane's rows lies at addr ^ 32 j
+    // (the stage and the rows are whole multiples of 128 bytes), the 4 rows further on 512
+    // bytes later.  (One statement for the four fragments, with its own wait: the compiler
+    // does not know that these registers are filled later, and would copy them into place at
+    // once; four separate statements would be four trips to LDS in a row.)
+    __device__ __forceinline__ static void transposed(unsigned int addr, u32x4 (&f)[4])
+    {
+        const unsigned int a1 = addr ^ 32u, a2 = addr ^ 64u, a3 = addr ^ 96u;
+        uint2              l0, h0, l1, h1, l2, h2, l3, h3;
+        asm volatile("ds_read_b64_tr_b16 %0, %8\n\t"
+                     "ds_read_b64_tr_b16 %1, %8 offset:512\n\t"
+                     "ds_read_b64_tr_b16 %2, %9\n\t"
+                     "ds_read_b64_tr_b16 %3, %9 offset:512\n\t"
+                     "ds_read_b64_tr_b16 %4, %10\n\t"
+                     "ds_read_b64_tr_b16 %5, %10 offset:512\n\t"
+                     "ds_read_b64_tr_b16 %6, %11\n\t"
+                     "ds_read_b64_tr_b16 %7, %11 offset:512\n\t"
+                     "s_waitcnt lgkmcnt(0)"
+                     : "=&v"(l0), "=&v"(h0), "=&v"(l1), "=&v"(h1), "=&v"(l2), "=&v"(h2), "=&v"(l3), "=&v"(h3)
+                     : "v"(addr), "v"(a1), "v"(a2), "v"(a3)
+                     : "memory");
+        f[0] = u32x4{l0.x, l0.y, h0.x, h0.y};
+        f[1] = u32x4{l1.x, l1.y, h1.x, h1.y};
+        f[2] = u32x4{l2.x, l2.y, h2.x, h2.y};
+        f[3] = u32x4{l3.x, l3.y, h3.x, h3.y};
+    }
+
+    // a 32-wide side: rows of 64 bytes, two column pieces
+    __device__ __forceinline__ static void transposed(unsigned int addr, u32x4 (&f)[2])
+    {
+        const unsigned int a1 = addr ^ 32u;
+        uint2              l0, h0, l1, h1;
+        asm volatile("ds_read_b64_tr_b16 %0, %4\n\t"
+                     "ds_read_b64_tr_b16 %1, %4 offset:256\n\t"
+                     "ds_read_b64_tr_b16 %2, %5\n\t"
+                     "ds_read_b64_tr_b16 %3, %5 offset:256\n\t"
+                     "s_waitcnt lgkmcnt(0)"
+                     : "=&v"(l0), "=&v"(h0), "=&v"(l1), "=&v"(h1)
+                     : "v"(addr), "v"(a1)
+                     : "memory");
+        f[0] = u32x4{l0.x, l0.y, h0.x, h0.y};
+        f[1] = u32x4{l1.x, l1.y, h1.x, h1.y};
     }
 
     __device__ __forceinline__ static void run(const gemm_args& args)
@@ -172,17 +254,20 @@ struct stream_gemm
 
         // K-contiguous: load q = wave + 4 i of an operand covers rows 4q + l/16, LDS slot
         // l%16 of that row, so the lane fetches chunk (l%16) ^ (row mod 16), and row mod 16 =
-        // 4 wave + l/16 for every i.  M/N-contiguous: load q = wave + 4 i covers k rows
-        // 8q + l/8, 16-byte piece l%8 of the row's 128 bytes, in memory order.
+        // 4 wave + l/16 for every i.  M/N-contiguous, W wide: a k row is 2 W bytes, load
+        // q = wave + 4 i covers the 512 / W k rows from (512 / W) q on, and the lane fills
+        // 16-byte slot l mod (W / 8) of its row, which holds the half l%2 of the 32-byte piece
+        // that mn_piece() puts there.
         const int          sub    = lane >> 4, slot = lane & 15;
         const int          chunk  = slot ^ ((4 * wave + sub) & 15);
         const unsigned int voff_a = A_KMAJOR ? (unsigned int)(((4 * wave + sub) * lda + chunk * 8) * 2)
-                                             : (unsigned int)(((8 * wave + (lane >> 3)) * lda + (lane & 7) * 8) * 2);
+                                             : mn_load_offset<BM>(lane, wave, lda);
         const unsigned int voff_b = B_KMAJOR ? (unsigned int)(((4 * wave + sub) * ldb + chunk * 8) * 2)
-                                             : (unsigned int)(((8 * wave + (lane >> 3)) * ldb + (lane & 7) * 8) * 2);
-        // bytes from load i to load i+1 (16 rows, or 32 k rows), and from stage to stage
-        const unsigned int step_a  = (unsigned int)((A_KMAJOR ? 16 : 32) * lda * 2);
-        const unsigned int step_b  = (unsigned int)((B_KMAJOR ? 16 : 32) * ldb * 2);
+                                             : mn_load_offset<BN>(lane, wave, ldb);
+        // bytes from load i to load i+1 (16 rows, or 4 loads' worth of k rows), and from stage
+        // to stage
+        const unsigned int step_a  = (unsigned int)((A_KMAJOR ? 16 : 4 * (512 / BM)) * lda * 2);
+        const unsigned int step_b  = (unsigned int)((B_KMAJOR ? 16 : 4 * (512 / BN)) * ldb * 2);
         const unsigned int stage_a = A_KMAJOR ? (unsigned int)ROW_BYTES : (unsigned int)(BK * lda * 2);
         const unsigned int stage_b = B_KMAJOR ? (unsigned int)ROW_BYTES : (unsigned int)(BK * ldb * 2);
 
@@ -241,30 +326,9 @@ struct stream_gemm
         // i, element j what lane 4j + i/4 addressed, element i%4), so the group that feeds k
         // 8 g .. 8 g + 7 reads rows 32 wave + 8 g + p/4 and the same 4 rows further on.
         const int frag_off = slot * ROW_BYTES + (((4 * wave + sub) ^ slot) & 15) * 16;
-        const int tr_off   = (32 * wave + 8 * sub + (slot >> 2)) * 128 + (slot & 3) * 8;
+        const int tr_off_a = mn_read_offset<BM>(wave, sub, slot);
+        const int tr_off_b = mn_read_offset<BN>(wave, sub, slot);
         using lds_u32x4    = __attribute__((address_space(3))) u32x4;
-        // (one statement for the four fragments of a 64-wide side, with its own wait: the
-        // compiler does not know that these registers are filled later, and would copy them
-        // into place at once; four separate statements would be four trips to LDS in a row)
-        auto transposed = [](unsigned int addr, u32x4 (&f)[4]) {
-            uint2 l0, h0, l1, h1, l2, h2, l3, h3;
-            asm volatile("ds_read_b64_tr_b16 %0, %8\n\t"
-                         "ds_read_b64_tr_b16 %1, %8 offset:512\n\t"
-                         "ds_read_b64_tr_b16 %2, %8 offset:32\n\t"
-                         "ds_read_b64_tr_b16 %3, %8 offset:544\n\t"
-                         "ds_read_b64_tr_b16 %4, %8 offset:64\n\t"
-                         "ds_read_b64_tr_b16 %5, %8 offset:576\n\t"
-                         "ds_read_b64_tr_b16 %6, %8 offset:96\n\t"
-                         "ds_read_b64_tr_b16 %7, %8 offset:608\n\t"
-                         "s_waitcnt lgkmcnt(0)"
-                         : "=&v"(l0), "=&v"(h0), "=&v"(l1), "=&v"(h1), "=&v"(l2), "=&v"(h2), "=&v"(l3), "=&v"(h3)
-                         : "v"(addr)
-                         : "memory");
-            f[0] = u32x4{l0.x, l0.y, h0.x, h0.y};
-            f[1] = u32x4{l1.x, l1.y, h1.x, h1.y};
-            f[2] = u32x4{l2.x, l2.y, h2.x, h2.y};
-            f[3] = u32x4{l3.x, l3.y, h3.x, h3.y};
-        };
 
         int slot_index = 0; // of stage t
         for(int t = 0; t < stages; ++t)
@@ -278,7 +342,7 @@ struct stream_gemm
             issue(clamped(t + DEPTH - 1), slot_index == 0 ? DEPTH - 1 : slot_index - 1);
 
             lds_char_ptr       sa   = lds + slot_index * STAGE + frag_off;
-            const unsigned int sa_t = lds_addr + slot_index * STAGE + tr_off;
+            const unsigned int sa_t = lds_addr + slot_index * STAGE;
             u32x4              fa[TM], fb[TN];
             if constexpr(A_KMAJOR)
             {
@@ -290,7 +354,7 @@ struct stream_gemm
             }
             else
             {
-                transposed(sa_t, fa);
+                transposed(sa_t + tr_off_a, fa);
             }
             if constexpr(B_KMAJOR)
             {
@@ -302,7 +366,7 @@ struct stream_gemm
             }
             else
             {
-                transposed(sa_t + A_BYTES, fb);
+                transposed(sa_t + A_BYTES + tr_off_b, fb);
             }
 #pragma unroll
             for(int i = 0; i < TM; ++i)

@@ -165,9 +165,13 @@ static int check_select()
         return fail("model: skinny M under a column-major C streams as skinny N");
     if(!model_plan(32, 8192, 8192, 0, 0, 0, &p) || tiles[p.variant].pipeline != 7 || tiles[p.variant].bn != 64)
         return fail("model: weights stored K x N stream on the 64-wide side");
-    // an operand that is not K-contiguous sits on a 64-wide side of the tile
-    if(!model_plan(32, 8192, 8192, 0, 1, 1, &p) || tiles[p.variant].pipeline != 7 || tiles[p.variant].bm != 64)
-        return fail("model: activations stored K x M stream on a 64-wide side");
+    // the large operand, when it is not K-contiguous, sits on a 64-wide side of the tile (whole
+    // cache lines); the small one may sit on a 32-wide side
+    if(!model_plan(32, 8192, 8192, 0, 1, 1, &p) || tiles[p.variant].pipeline != 7 || tiles[p.variant].bm != 32
+       || tiles[p.variant].bn != 64)
+        return fail("model: activations stored K x M stream on the 32-wide side");
+    if(!model_plan(32, 8192, 8192, 0, 1, 0, &p) || tiles[p.variant].pipeline != 7 || tiles[p.variant].bn != 64)
+        return fail("model: weights stored K x N next to activations stored K x M stream on the 64-wide side");
     // few tiles and a long K: several workgroups per tile
     if(!model_plan(16, 1024, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline != 7 || p.split_k < 2)
         return fail("model: 32 tiles of a skinny shape are shared between workgroups");
