@@ -148,6 +148,8 @@ def stream_estimate(c: dict, rows: int, cols: int, K: int, a_kmajor: bool, b_kma
         l2_rate *= c["half_line"]
     from_memory = (large_bytes * (active / sharing) / rate
                    + small_bytes * active / l2_rate)
+    # (workgroups that share a compute unit take turns at part of a stage)
+    per_cu *= 1.0 + (-(-active // cus) - 1) * c["taking_turns"]
     return (c["launch_us"] + passes * (c["fill_us"] + stages * max(per_cu, from_memory))
             + (c["exchange_us"] + c["exchange_us_per_kb"] * slices * bm * bn * 4 / 1024 if slices > 1 else 0.0))
 
@@ -170,7 +172,10 @@ def fit_stream(records: list, start: dict) -> dict:
 
     def unpack(p):
         c = {k: float(v) for k, v in zip(keys, p)}
+        # (set by hand: the skinny problems of the sweep are bound by memory and say nothing
+        # about turns on a compute unit; left free, beyond_cache soaks up other effects)
         c["beyond_cache"] = start["beyond_cache"]
+        c["taking_turns"] = start["taking_turns"]
         c["stage_us"] = {t: float(v) for t, v in zip(STREAM_TILES, p[len(keys):])}
         return c
 
@@ -199,6 +204,21 @@ def fit_stream(records: list, start: dict) -> dict:
     return c
 
 
+def stream_pick(c: dict, M: int, N: int, K: int, a_kmajor: bool, b_kmajor: bool, plans: list):
+    """The plan (tile, slices, ...) of `plans` that the dispatcher takes (csrc/config_select.cpp:
+    stream_plan): the lowest estimate; an operand contiguous along M or N sits on a 32-wide
+    side of the tile only while it has at most 128 rows."""
+    def allowed(p):
+        bm, bn = (int(x) for x in p[0].split("x"))
+        return not ((not a_kmajor and bm == 32 and M > 128) or (not b_kmajor and bn == 32 and N > 128))
+
+    def estimate(p):
+        bm, bn = (int(x) for x in p[0].split("x"))
+        return stream_estimate(c, M, N, K, a_kmajor, b_kmajor, bm, bn, p[1])
+
+    return min((p for p in plans if allowed(p)), key=estimate)
+
+
 def stream_regret(records: list, c: dict):
     """(geometric mean, worst) of measured time of the plan the estimate picks over the
     best measured plan, per problem of the sweep."""
@@ -210,8 +230,7 @@ def stream_regret(records: list, c: dict):
         if not plans:
             continue
         a_k, b_k = r["lay"][0] == "r", r["lay"][1] == "c"
-        pick = min(plans, key=lambda p: stream_estimate(c, r["M"], r["N"], r["K"], a_k, b_k,
-                                                        *(int(x) for x in p[0].split("x")), p[1]))
+        pick = stream_pick(c, r["M"], r["N"], r["K"], a_k, b_k, plans)
         ratio = pick[2] / min(p[2] for p in plans)
         logs.append(math.log(ratio))
         worst = max(worst, ratio)
@@ -235,7 +254,7 @@ def main(argv=None) -> int:
         print(json.dumps(new, indent=1))
         print(f"regret of the estimate's pick over {len(records)} problems: mean {mean:.3f}, worst {worst:.2f}")
         if a.write:
-            new["fitted_from"] = f"{os.path.basename(a.log)}: {sum(len(r['t']) for r in records)} timings (beyond_cache set by hand)"
+            new["fitted_from"] = f"{os.path.basename(a.log)}: {sum(len(r['t']) for r in records)} timings (beyond_cache and taking_turns set by hand)"
             model["stream"] = new
             with open(a.model, "w") as f:
                 json.dump(model, f, indent=4)

@@ -114,7 +114,7 @@ def render_model(m: dict) -> list[str]:
               + ", ".join(repr(float(st[k])) for k in ("launch_us", "fill_us", "exchange_us", "exchange_us_per_kb",
                                                         "bytes_per_us_kmajor", "bytes_per_us_other", "bytes_per_us_l2",
                                                         "transposed_operand", "panel_sharing", "half_line",
-                                                        "beyond_cache"))
+                                                        "beyond_cache", "taking_turns"))
               + ", {" + ", ".join(repr(float(st["stage_us"][t])) for t in ("32x32", "64x32", "32x64", "64x64")) + "}};"]
     return ([f"constexpr int model_compute_units = {int(m['compute_units'])};"]
             + [f"constexpr double model_{k} = {float(m[k])!r};" for k in

@@ -61,16 +61,29 @@ def main(argv=None) -> int:
     variants = [v for v in L.variants() if v.pipeline == 7]
 
     def timed(fn) -> float:
+        """Microseconds per call, back to back; a measurement lasts at least 2 ms (calls of
+        10 us timed over 0.15 ms are at the mercy of the clock governor)."""
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         for _ in range(4):
             fn()
-        start.record()
-        for _ in range(a.reps):
-            fn()
-        stop.record()
-        torch.cuda.synchronize()
-        return start.elapsed_time(stop) / a.reps * 1e3  # microseconds
+        reps = a.reps
+        while True:
+            start.record()
+            for _ in range(reps):
+                fn()
+            stop.record()
+            torch.cuda.synchronize()
+            ms = start.elapsed_time(stop)
+            if ms >= 2.0 or reps >= 1024:
+                return ms / reps * 1e3
+            reps *= 4
 
+    # (clocks up before the first measurement)
+    warm = torch.randn(4096 * 4096, device="cuda").to(dtype)
+    for _ in range(50):
+        L.gemm(warm, warm, warm, 4096, 4096, 4096, 0, 0, 1)
+    torch.cuda.synchronize()
+    del warm
     gen = torch.Generator(device="cuda")
     gen.manual_seed(1)
     out = []

@@ -65,6 +65,8 @@ struct model_stream
                       // of the tile: requests of 64 bytes, half a cache line
     double beyond_cache; // factor on the two rates from memory for a large operand over 256 MB
                          // (set by hand, not fitted)
+    double taking_turns; // two workgroups on a compute unit: a stage of each takes 1 + this of what
+                         // it takes alone, where the compute unit is the bound (set by hand)
     double stage_us[4]; // per stage of 128 of one compute unit: tiles 32x32, 64x32, 32x64, 64x64
 };
 struct model_constants

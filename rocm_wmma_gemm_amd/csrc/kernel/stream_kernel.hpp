@@ -201,6 +201,39 @@ struct stream_gemm
         f[1] = u32x4{l1.x, l1.y, h1.x, h1.y};
     }
 
+    // acc += A fragment x B fragment, in place.  (Written out: left to place the
+    // accumulators itself, the compiler moved them to other registers and back around every
+    // stage, up to 50 moves a stage in the kernels with transposing reads: 16 x 8192 x 8192
+    // with neither operand K-contiguous 26.1 - 32.9 us against 22.8 us, B row-major 28.4 against
+    // 22.9, both K-contiguous 24.5 against 23.9; the 64 x 64 tile 35.4 against 27.2.)
+    __device__ __forceinline__ static void multiply_add(f32x4& acc, const u32x4& fa, const u32x4& fb)
+    {
+        if constexpr(IN == in_kind::f16)
+        {
+            asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(fa), "v"(fb));
+        }
+        else
+        {
+            asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(fa), "v"(fb));
+        }
+    }
+
+    // The compiler does not see that multiply_add reads and writes the accumulators on the
+    // matrix pipeline: this keeps the wait states between its own writes (the zeros) and the
+    // first multiply_add, and between the last multiply_add and its own reads.
+    __device__ __forceinline__ static void settle(f32x4 (&acc)[TM][TN])
+    {
+#pragma unroll
+        for(int i = 0; i < TM; ++i)
+        {
+#pragma unroll
+            for(int j = 0; j < TN; j += 2)
+            {
+                asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" : "+a"(acc[i][j]), "+a"(acc[i][j + 1]));
+            }
+        }
+    }
+
     __device__ __forceinline__ static void run(const gemm_args& args)
     {
         __shared__ __attribute__((aligned(1024))) char lds_raw[LDS_BYTES];
@@ -318,6 +351,7 @@ struct stream_gemm
                 acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
             }
         }
+        settle(acc);
 
         // fragment of this wave's K step (k 32 wave .. 32 wave + 31 of the stage).
         // K-contiguous: row l%16 of a 16-row block, k chunk 4 wave + l/16.  M/N-contiguous:
@@ -374,7 +408,7 @@ struct stream_gemm
 #pragma unroll
                 for(int j = 0; j < TN; ++j)
                 {
-                    acc[i][j] = mfma_16x16x32<IN>(fa[i], fb[j], acc[i][j]);
+                    multiply_add(acc[i][j], fa[i], fb[j]);
                 }
             }
             slot_index = slot_index + 1 == DEPTH ? 0 : slot_index + 1;
@@ -385,6 +419,7 @@ struct stream_gemm
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
+        settle(acc);
         using lds_float = __attribute__((address_space(3))) float;
         lds_float* part = reinterpret_cast<lds_float*>(lds);
 #pragma unroll
@@ -423,15 +458,22 @@ struct stream_gemm
             return;
         }
         // Several workgroups per tile.  The tiles they exchange travel through memory that
-        // every XCD sees the same way: device-scope atomic stores and loads, which pass by
-        // the XCD's own L2; a workgroup counts itself in when its stores have been
-        // acknowledged, and reads the others' tiles only after it has seen all of them
-        // counted.
-        const long long tile_lin = batch * tiles + wg;
-        float*          mine     = args.partials + (tile_lin * args.k_slices + slice) * (long long)(BM * BN);
-        for(int e = threadIdx.x; e < BM * BN; e += THREADS)
+        // every XCD sees the same way: stores and loads at device scope (sc1), which write
+        // through, and miss in, the XCD's own L2; 16 bytes a lane.  A workgroup counts itself
+        // in when its stores have been acknowledged, and reads the others' tiles only after
+        // it has seen all of them counted, so nobody reads a piece that is half written.
+        constexpr int   DEVICE_SCOPE = 16; // cache policy operand of the buffer builtins: sc1
+        constexpr int   TILE4        = BM * BN / 4;
+        const long long tile_lin     = batch * tiles + wg;
+        const __amdgpu_buffer_rsrc_t shared = __builtin_amdgcn_make_buffer_rsrc(
+            args.partials + tile_lin * args.k_slices * (long long)(BM * BN), 0, args.k_slices * BM * BN * 4, 0x00020000);
+        using lds_f32x4 = __attribute__((address_space(3))) f32x4;
+        for(int e4 = threadIdx.x; e4 < TILE4; e4 += THREADS)
         {
-            __hip_atomic_store(mine + e, tile_sum(e), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const lds_f32x4* p4 = reinterpret_cast<const lds_f32x4*>(part) + e4;
+            const f32x4      s  = ((p4[0] + p4[TILE4]) + p4[2 * TILE4]) + p4[3 * TILE4]; // (wave order)
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, s), shared, (slice * TILE4 + e4) * 16, 0,
+                                                   DEVICE_SCOPE);
         }
         // (the stores above write through to memory and are acknowledged from there; a
         // release fence at device scope would write the whole L2 back instead, which costs
@@ -449,26 +491,30 @@ struct stream_gemm
         {
             return; // the last one to arrive finishes the tile
         }
-        const float* all = args.partials + tile_lin * args.k_slices * (long long)(BM * BN);
-        // (all slices' loads of an element go out before the first is used: a loop over the
+        // (all slices' loads of a piece go out before the first is used: a loop over the
         // slices would pay a trip to memory per slice; the host keeps k_slices <= MAX_SLICES)
-        for(int e = threadIdx.x; e < BM * BN; e += THREADS)
+        for(int e4 = threadIdx.x; e4 < TILE4; e4 += THREADS)
         {
-            float v[MAX_SLICES];
+            f32x4 v[MAX_SLICES];
 #pragma unroll
             for(int q = 0; q < MAX_SLICES; ++q)
             {
-                v[q] = q < args.k_slices ? __hip_atomic_load(all + (long long)q * (BM * BN) + e, __ATOMIC_RELAXED,
-                                                             __HIP_MEMORY_SCOPE_AGENT)
-                                         : 0.0f;
+                v[q] = q < args.k_slices
+                           ? __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(shared, (q * TILE4 + e4) * 16,
+                                                                                             0, DEVICE_SCOPE))
+                           : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
             }
-            float s = v[0];
+            f32x4 s = v[0];
 #pragma unroll
             for(int q = 1; q < MAX_SLICES; ++q)
             {
                 s = q < args.k_slices ? s + v[q] : s;
             }
-            store(e, s);
+#pragma unroll
+            for(int c = 0; c < 4; ++c)
+            {
+                store(4 * e4 + c, s[c]);
+            }
         }
         if(threadIdx.x == 0)
         {

@@ -825,7 +825,7 @@ def test_scratch_buffer_outlives_a_graph_that_holds_its_address(loader):
     import torch
 
     assert loader.workspace_release() == 0, "run before any other test that captures a graph"
-    M, N, K, lc, la, lb = 128, 8192, 8192, 0, 1, 0  # (a split-K plan: partial planes in the buffer)
+    M, N, K, lc, la, lb = 256, 8192, 8192, 0, 1, 0  # (a split-K plan: partial planes in the buffer)
     assert loader.select(M, N, K, 1, lc, la, lb)[2] > 1
     A, B = make_inputs(M, N, K, la, lb, O.F16)
     dA, dB = to_device(A, O.F16), to_device(B, O.F16)
