@@ -313,15 +313,25 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
                      -1);
         }
     }
-    // (between 65 and 128 rows the two families are within 20 % of each other and the two
-    // estimates are not that good: the tiled kernels keep those when they take the shape,
-    // except against a small large operand with both K-contiguous, where the streaming
-    // kernel measured 1.1 to 1.5 times faster: 128 x 4096 x 4096 14.1 against 19.2 us)
-    // and small problems (at most 2^20 elements of C, K up to 4096: 512 x 2048 x 2048 12.7
-    // against 17.9 us, 256 x 256 x 1024 9.3 against 13.7) unless neither operand is K-contiguous
-    const size_t skinny = std::min(rows, cols), other = std::max(rows, cols);
-    const bool   compete = skinny <= 64 || (a_kmajor && b_kmajor && other * k <= (size_t{1} << 24))
-                         || (rows * cols <= (size_t{1} << 20) && k <= 4096 && (a_kmajor || b_kmajor));
+    // The two estimates compete for skinny shapes (up to 128 rows or columns) and for small
+    // problems (at most 2^20 elements of C, K up to 4096: 512 x 2048 x 2048 12.2 against 17.8
+    // us, 256 x 256 x 1024 8.6 against 12.8), in every layout.  From 65 rows on only while
+    // the streaming plan's workgroups all run at once: the estimates are closer to each
+    // other than to the truth where they need a second pass over the compute units
+    // (128 x 14336 x 4096: 34.5 us streamed, 29.2 tiled; 128 x 8192 x 8192, one pass, 30.3
+    // against 37.4).
+    bool one_pass = false;
+    if(have_stream)
+    {
+        const model_variant& v      = model_variants[stream_best.variant];
+        const size_t         groups = ceil_div(rows, static_cast<size_t>(v.block_m))
+                              * ceil_div(cols, static_cast<size_t>(v.block_n))
+                              * static_cast<size_t>(stream_best.split_k) * batch;
+        one_pass = groups <= cus * ((v.block_m == 64 && v.block_n == 64) ? 1 : 2);
+    }
+    const size_t skinny  = std::min(rows, cols);
+    const bool   compete = skinny <= 64 || (skinny <= 128 && one_pass)
+                         || (rows * cols <= (size_t{1} << 20) && k <= 4096);
     if(have_stream && (!found || (stream_us < best && compete)))
     {
         *out  = stream_best;

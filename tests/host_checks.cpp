@@ -186,14 +186,18 @@ static int check_select()
         return fail("model: 128 rows against a very large operand stay with the tiled kernels");
     if(!model_plan(256, 8192, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline == 7)
         return fail("model: 256 rows are not skinny");
-    // 65 to 128 rows: only against a small large operand, both K-contiguous
+    // 65 to 128 rows: in every layout, while the streaming plan's workgroups all run at once
     if(!model_plan(128, 4096, 4096, 0, 0, 1, &p) || tiles[p.variant].pipeline != 7)
         return fail("model: 128 rows against 4096 x 4096, both K-contiguous, stream");
-    if(!model_plan(128, 4096, 4096, 0, 1, 0, &p) || tiles[p.variant].pipeline == 7)
-        return fail("model: 128 rows against 4096 x 4096, neither K-contiguous, stay with the tiled kernels");
-    // small problems: at most 2^20 elements of C, an operand K-contiguous
+    if(!model_plan(128, 4096, 4096, 0, 1, 0, &p) || tiles[p.variant].pipeline != 7)
+        return fail("model: 128 rows against 4096 x 4096, neither K-contiguous, stream");
+    if(!model_plan(128, 14336, 4096, 0, 0, 1, &p) || tiles[p.variant].pipeline == 7)
+        return fail("model: 128 rows against 14336 x 4096 (two passes of streaming workgroups) stay with the tiled kernels");
+    // small problems: at most 2^20 elements of C, any layout
     if(!model_plan(512, 2048, 2048, 0, 0, 0, &p) || tiles[p.variant].pipeline != 7)
         return fail("model: 512 x 2048 x 2048 streams");
+    if(!model_plan(512, 2048, 2048, 0, 1, 0, &p) || tiles[p.variant].pipeline != 7)
+        return fail("model: 512 x 2048 x 2048 with neither operand K-contiguous streams");
     if(!model_plan(2048, 1024, 1024, 0, 0, 1, &p) || tiles[p.variant].pipeline == 7)
         return fail("model: 2048 x 1024 x 1024 is too large for a workgroup per small tile");
     // a skinny shape the model does not take (K-contiguous rows of 4001 elements) and the
