@@ -527,20 +527,28 @@ def candidates(variants, M, N, K, lc):
 
 
 def time_candidate(L, torch, index, sw, sk, touch, C, A, B, M, N, K, lc, la, lb, reps, warmup):
+    """Milliseconds per call of one plan, calls back to back (what a caller's loop sees:
+    the launch of a call overlaps the call before it): the median of three runs of at least
+    `reps` calls and 2 ms each."""
     for _ in range(warmup):
         rc = L.run_variant(index, sw, sk, C, A, B, M, N, K, lc, la, lb, touch_ahead=touch)
         if rc != 0:
             return None
     torch.cuda.synchronize()
-    start = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
-    stop = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
-    for i in range(reps):
-        start[i].record()
-        L.run_variant(index, sw, sk, C, A, B, M, N, K, lc, la, lb, touch_ahead=touch)
-        stop[i].record()
-    torch.cuda.synchronize()
-    ms = sorted(s.elapsed_time(e) for s, e in zip(start, stop))
-    return ms[len(ms) // 2]
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    runs = []
+    while len(runs) < 3:
+        start.record()
+        for _ in range(reps):
+            L.run_variant(index, sw, sk, C, A, B, M, N, K, lc, la, lb, touch_ahead=touch)
+        stop.record()
+        torch.cuda.synchronize()
+        ms = start.elapsed_time(stop)
+        if ms < 2.0 and reps < 1024:
+            reps *= 4
+            continue
+        runs.append(ms / reps)
+    return sorted(runs)[1]
 
 
 def main(argv=None) -> int:
