@@ -332,9 +332,26 @@ struct stream_gemm
                            __builtin_amdgcn_readfirstlane((unsigned int)(first + stage) * stage_b + i * step_b));
             }
         };
+        // Where the tile grid is one tile high (a skinny M or N: no two workgroups read the
+        // same panel of the large operand), every panel starts its run of stages at a
+        // different place and wraps around.  Workgroups that walk K in step all ask for the
+        // same 256 bytes of their rows at the same time, rows a power of two apart, and
+        // those requests crowd onto a few memory channels: 16 x 8192 x 8192 with B
+        // column-major 24.1 -> 21.0 us, 16 x 28672 x 8192 (470 MB of B, past the memory-side
+        // cache) 100 -> 83 us.  (With two tiles to a panel, 128 x 8192 x 8192, the pair shares
+        // the panel through L2 only while it walks in step, and staggering the panels gains
+        // nothing there; staggering by XCD only is worse than not at all.)  The order of
+        // the sum of an element depends on its tile's place alone: results stay the same
+        // from run to run.
+        const bool one_high = args.grid_m == 1 || args.grid_n == 1;
+        const int  panel = args.grid_m <= args.grid_n ? tn : tm, panels = args.grid_m <= args.grid_n ? args.grid_n : args.grid_m;
+        const int  turn  = one_high ? (int)(((long long)panel * stages) / panels) : 0;
         // Past the last stage the loads fetch the last stage again into slots that nobody
         // reads any more: the number of loads in flight stays what the waits assume.
-        auto clamped = [&](int stage) { return stage < stages ? stage : stages - 1; };
+        auto clamped = [&](int stage) {
+            const int at = (stage < stages ? stage : stages - 1) + turn;
+            return at >= stages ? at - stages : at;
+        };
 
         for(int t = 0; t < DEPTH - 1; ++t)
         {
