@@ -142,7 +142,7 @@ def stream_estimate(c: dict, rows: int, cols: int, K: int, a_kmajor: bool, b_kma
     if max(rows, cols) * K * 2 > 256 << 20:
         # the large operand does not fit the memory-side cache, which serves part of a
         # repeated call on a smaller one (not fitted: left free it soaks up other effects)
-        rate *= c["beyond_cache"]
+        rate *= c["beyond_cache" if large_kmajor else "beyond_cache_other"]
     l2_rate = c["bytes_per_us_l2"]
     if not (a_kmajor if wide else b_kmajor) and (bm if wide else bn) == 32:
         l2_rate *= c["half_line"]
@@ -175,6 +175,7 @@ def fit_stream(records: list, start: dict) -> dict:
         # (set by hand: the skinny problems of the sweep are bound by memory and say nothing
         # about turns on a compute unit; left free, beyond_cache soaks up other effects)
         c["beyond_cache"] = start["beyond_cache"]
+        c["beyond_cache_other"] = start["beyond_cache_other"]
         c["taking_turns"] = start["taking_turns"]
         c["stage_us"] = {t: float(v) for t, v in zip(STREAM_TILES, p[len(keys):])}
         return c
@@ -254,7 +255,7 @@ def main(argv=None) -> int:
         print(json.dumps(new, indent=1))
         print(f"regret of the estimate's pick over {len(records)} problems: mean {mean:.3f}, worst {worst:.2f}")
         if a.write:
-            new["fitted_from"] = f"{os.path.basename(a.log)}: {sum(len(r['t']) for r in records)} timings (beyond_cache and taking_turns set by hand)"
+            new["fitted_from"] = f"{os.path.basename(a.log)}: {sum(len(r['t']) for r in records)} timings (beyond_cache, beyond_cache_other and taking_turns set by hand)"
             model["stream"] = new
             with open(a.model, "w") as f:
                 json.dump(model, f, indent=4)

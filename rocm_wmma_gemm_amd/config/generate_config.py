@@ -97,7 +97,7 @@ def load_model(path: str) -> dict:
     with open(path) as f:
         m = json.load(f)
     for key in ("compute_units", "launch_us", "reduce_us", "plane_bytes_per_us", "tile_bytes_per_us",
-                "copy_bytes_per_us", "step_us", "item_us", "stream"):
+                "copy_bytes_per_us", "operand_bytes_per_us", "step_us", "item_us", "stream"):
         if key not in m:
             raise ValueError(f"{path}: missing {key}")
     return m
@@ -114,11 +114,12 @@ def render_model(m: dict) -> list[str]:
               + ", ".join(repr(float(st[k])) for k in ("launch_us", "fill_us", "exchange_us", "exchange_us_per_kb",
                                                         "bytes_per_us_kmajor", "bytes_per_us_other", "bytes_per_us_l2",
                                                         "transposed_operand", "panel_sharing", "half_line",
-                                                        "beyond_cache", "taking_turns"))
+                                                        "beyond_cache", "beyond_cache_other", "taking_turns"))
               + ", {" + ", ".join(repr(float(st["stage_us"][t])) for t in ("32x32", "64x32", "32x64", "64x64")) + "}};"]
     return ([f"constexpr int model_compute_units = {int(m['compute_units'])};"]
             + [f"constexpr double model_{k} = {float(m[k])!r};" for k in
-               ("launch_us", "reduce_us", "plane_bytes_per_us", "tile_bytes_per_us", "copy_bytes_per_us")]
+               ("launch_us", "reduce_us", "plane_bytes_per_us", "tile_bytes_per_us", "copy_bytes_per_us",
+                "operand_bytes_per_us")]
             + [f"constexpr int model_step_count = {len(steps)};",
                f"constexpr model_step model_steps[{max(len(steps), 1)}] = {{"]
             + (steps or ["    {0, 0, 0, 0.0, 0.0},"]) + ["};"] + stream)

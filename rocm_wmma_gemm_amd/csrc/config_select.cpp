@@ -19,6 +19,7 @@ const model_constants    model_measured
     = {generated::model_compute_units,      generated::model_launch_us,
        generated::model_reduce_us,          generated::model_plane_bytes_per_us,
        generated::model_tile_bytes_per_us,  generated::model_copy_bytes_per_us,
+       generated::model_operand_bytes_per_us,
        generated::model_steps,              generated::model_step_count,
        generated::model_stream_constants};
 
@@ -216,6 +217,7 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
         return bytes <= knee ? bytes / plane_bytes_per_us
                              : knee / plane_bytes_per_us + (bytes - knee) / (2.0 * plane_bytes_per_us);
     };
+    const double operand_us = static_cast<double>((rows + cols) * k * batch) * 2.0 / model_measured.operand_bytes_per_us;
     const size_t     kt            = ceil_div(k, size_t{64});
     double           best          = 0.0;
     bool             found         = false;
@@ -332,7 +334,10 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
     const size_t skinny  = std::min(rows, cols);
     const bool   compete = skinny <= 64 || (skinny <= 128 && one_pass)
                          || (rows * cols <= (size_t{1} << 20) && k <= 4096);
-    if(have_stream && (!found || (stream_us < best && compete)))
+    // (no tiled plan moves A and B faster than operand_bytes_per_us, which is what bounds the
+    // skinny shapes; the estimates above rank the tiled plans among themselves without it)
+    const double tiled_us = std::max(best, launch_us + operand_us);
+    if(have_stream && (!found || (stream_us < tiled_us && compete)))
     {
         *out  = stream_best;
         found = true;
@@ -392,7 +397,7 @@ bool stream_plan(size_t rows, size_t cols, size_t k, bool a_kmajor, bool b_kmajo
         const bool   large_kmajor = wide ? b_kmajor : a_kmajor, small_kmajor = wide ? a_kmajor : b_kmajor;
         const double rate    = (large_kmajor ? c.bytes_per_us_kmajor : c.bytes_per_us_other)
                             * (!large_kmajor && (wide ? bn : bm) == 32 ? c.half_line : 1.0)
-                            * (std::max(rows, cols) * k * 2 > (size_t{256} << 20) ? c.beyond_cache : 1.0);
+                            * (std::max(rows, cols) * k * 2 > (size_t{256} << 20) ? (large_kmajor ? c.beyond_cache : c.beyond_cache_other) : 1.0);
         const double l2_rate = c.bytes_per_us_l2 * (!small_kmajor && (wide ? bm : bn) == 32 ? c.half_line : 1.0);
         for(size_t s = 1; s <= 8; s *= 2)
         {

@@ -63,8 +63,8 @@ struct model_stream
                           // is fetched once for all: it counts as fetched g / (1 + (g - 1) x this) times
     double half_line; // factor on a rate for an operand contiguous along M or N on a 32-wide side
                       // of the tile: requests of 64 bytes, half a cache line
-    double beyond_cache; // factor on the two rates from memory for a large operand over 256 MB
-                         // (set by hand, not fitted)
+    double beyond_cache, beyond_cache_other; // factors on the two rates from memory for a large
+                         // operand over 256 MB, K-contiguous or not (set by hand, not fitted)
     double taking_turns; // two workgroups on a compute unit: a stage of each takes 1 + this of what
                          // it takes alone, where the compute unit is the bound (set by hand)
     double stage_us[4]; // per stage of 128 of one compute unit: tiles 32x32, 64x32, 32x64, 64x64
@@ -76,6 +76,8 @@ struct model_constants
     double plane_bytes_per_us; // split-K partial planes: written, then read by the reduce kernel
     double tile_bytes_per_us; // partial tiles of a split tail wave or of the walk by K tile
     double copy_bytes_per_us; // padded operand copies
+    double operand_bytes_per_us; // what the tiled kernels reach at most streaming A and B from memory
+                                 // (skinny shapes: 134 MB in 24-27 us of split-K kernel, 470 MB in 83-96; set by hand)
     const model_step* steps;
     int               step_count;
     model_stream      stream;

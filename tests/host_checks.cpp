@@ -193,6 +193,13 @@ static int check_select()
         return fail("model: 128 rows against 4096 x 4096, neither K-contiguous, stream");
     if(!model_plan(128, 14336, 4096, 0, 0, 1, &p) || tiles[p.variant].pipeline == 7)
         return fail("model: 128 rows against 14336 x 4096 (two passes of streaming workgroups) stay with the tiled kernels");
+    // a large operand past the memory-side cache (470 MB): streamed when it is K-contiguous
+    // (the tiled kernels do not move operands faster than operand_bytes_per_us), left to the
+    // tiled kernels' split along K when it is not
+    if(!model_plan(16, 28672, 8192, 0, 0, 1, &p) || tiles[p.variant].pipeline != 7 || p.split_k != 1)
+        return fail("model: 16 rows against 28672 x 8192, K-contiguous, stream");
+    if(!model_plan(16, 28672, 8192, 0, 0, 0, &p) || tiles[p.variant].pipeline == 7)
+        return fail("model: 16 rows against 8192 x 28672 stored row-major stay with the tiled kernels");
     // small problems: at most 2^20 elements of C, any layout
     if(!model_plan(512, 2048, 2048, 0, 0, 0, &p) || tiles[p.variant].pipeline != 7)
         return fail("model: 512 x 2048 x 2048 streams");
