@@ -75,8 +75,10 @@ struct stream_gemm
     // fills its ring or adds up and stores its tile, the other keeps the loads coming.
     // Against one workgroup per compute unit with a ring of 144 KB, same plans: +9.6 %
     // (geometric mean over 135 skinny problems), 16 x 28672 x 8192 4.1 -> 4.6 TB/s.  (A ring
-    // of 152 KB is no better where a compute unit has one workgroup anyway: 128 tiles of
-    // 16 x 8192 x 8192, 24.3 us with 3 stages of 32 x 64, 25.7 us with 6.)
+    // of 112 or 152 KB is no better where a compute unit has one workgroup anyway: 128 tiles of
+    // 16 x 8192 x 8192, 21.4 us with 3 stages of 32 x 64, 21.3 and 21.7 us with 4 and 6.  Nor
+    // is reading the fragments of stage t + 1 under the MFMAs of stage t: it asks for a stage
+    // one stage earlier, 21.5 -> 26.7 us.)
     static constexpr int RING_KB   = 76;
     static constexpr int DEPTH_FIT = (RING_KB * 1024) / STAGE < 3 ? 3 : (RING_KB * 1024) / STAGE;
     static constexpr int DEPTH     = DEPTH_FIT < 8 ? DEPTH_FIT : 8;
