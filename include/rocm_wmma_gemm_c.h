@@ -68,7 +68,7 @@ typedef struct rocm_wmma_gemm_variant_info
 {
     int block_m, block_n, block_k; /* workgroup tile */
     int warps_m, warps_n;          /* wave grid inside the workgroup */
-    int warp_tile_m, warp_tile_n;  /* 32x32 MFMA tiles per wave */
+    int warp_tile_m, warp_tile_n;  /* 32x32 MFMA tiles per wave (0: a 16-wide side of the streaming kernel's tile) */
     int pipeline;                  /* 0 = register-staged general path, 1 = direct-to-LDS, 2 = direct-to-LDS ping-pong, 3, 4 = 1, 2 on the 16x16x32 MFMA, 5 = one wave per SIMD, persistent workgroups, 6 = 1 with a ring of 4 tiles at BLOCK_K 64 */
     int lds_bytes;                 /* static LDS per workgroup */
     int threads;                   /* workgroup size */

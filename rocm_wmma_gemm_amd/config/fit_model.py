@@ -110,7 +110,7 @@ def fit(records, model: dict) -> dict:
     return out
 
 
-STREAM_TILES = ("32x32", "64x32", "32x64", "64x64")
+STREAM_TILES = ("32x32", "64x32", "32x64", "64x64", "16x32", "16x64", "32x16", "64x16")
 
 
 def stream_estimate(c: dict, rows: int, cols: int, K: int, a_kmajor: bool, b_kmajor: bool, bm: int, bn: int,
@@ -205,19 +205,26 @@ def fit_stream(records: list, start: dict) -> dict:
     return c
 
 
+STREAM_TIE = 1.03  # estimates this close do not tell plans apart (csrc/config_select.cpp: stream_plan)
+
+
 def stream_pick(c: dict, M: int, N: int, K: int, a_kmajor: bool, b_kmajor: bool, plans: list):
     """The plan (tile, slices, ...) of `plans` that the dispatcher takes (csrc/config_select.cpp:
-    stream_plan): the lowest estimate; an operand contiguous along M or N sits on a 32-wide
-    side of the tile only while it has at most 128 rows."""
+    stream_plan): of those whose estimate is within STREAM_TIE of the lowest, the fewest
+    workgroups per tile, then the lowest estimate; an operand contiguous along M or N sits on a
+    32-wide side of the tile only while it has at most 128 rows, and never on a 16-wide one."""
     def allowed(p):
         bm, bn = (int(x) for x in p[0].split("x"))
-        return not ((not a_kmajor and bm == 32 and M > 128) or (not b_kmajor and bn == 32 and N > 128))
+        return not ((not a_kmajor and (bm == 16 or (bm == 32 and M > 128)))
+                    or (not b_kmajor and (bn == 16 or (bn == 32 and N > 128))))
 
     def estimate(p):
         bm, bn = (int(x) for x in p[0].split("x"))
         return stream_estimate(c, M, N, K, a_kmajor, b_kmajor, bm, bn, p[1])
 
-    return min((p for p in plans if allowed(p)), key=estimate)
+    known = [(estimate(p), p) for p in plans if allowed(p)]
+    lowest = min(us for us, _ in known)
+    return min((x for x in known if x[0] <= lowest * STREAM_TIE), key=lambda x: (x[1][1], x[0]))[1]
 
 
 def stream_regret(records: list, c: dict):

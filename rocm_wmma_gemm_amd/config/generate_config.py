@@ -49,8 +49,9 @@ def read_variants(path: str) -> list[dict]:
 
 def variant_of(cfg: dict, variants: list[dict]) -> int:
     """Index of the compiled variant a JSON "config" object names."""
-    bm = cfg["warps_m"] * cfg["warp_tile_m"] * MFMA_TILE
-    bn = cfg["warps_n"] * cfg["warp_tile_n"] * MFMA_TILE
+    # (warp_tile 0.5: a 16-wide side of the whole-K streaming kernel's tile)
+    bm = int(cfg["warps_m"] * cfg["warp_tile_m"] * MFMA_TILE)
+    bn = int(cfg["warps_n"] * cfg["warp_tile_n"] * MFMA_TILE)
     bk = cfg.get("block_k", 64)
     pipe = cfg.get("pipeline", 0)
     for v in variants:
@@ -115,7 +116,7 @@ def render_model(m: dict) -> list[str]:
                                                         "bytes_per_us_kmajor", "bytes_per_us_other", "bytes_per_us_l2",
                                                         "transposed_operand", "panel_sharing", "half_line",
                                                         "beyond_cache", "beyond_cache_other", "taking_turns"))
-              + ", {" + ", ".join(repr(float(st["stage_us"][t])) for t in ("32x32", "64x32", "32x64", "64x64")) + "}};"]
+              + ", {" + ", ".join(repr(float(st["stage_us"][t])) for t in ("32x32", "64x32", "32x64", "64x64", "16x32", "16x64", "32x16", "64x16")) + "}};"]
     return ([f"constexpr int model_compute_units = {int(m['compute_units'])};"]
             + [f"constexpr double model_{k} = {float(m[k])!r};" for k in
                ("launch_us", "reduce_us", "plane_bytes_per_us", "tile_bytes_per_us", "copy_bytes_per_us",

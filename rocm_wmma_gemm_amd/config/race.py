@@ -50,9 +50,10 @@ def hook_split(cfg: dict) -> int:
 def variant_of(cfg: dict, variants):
     """The compiled variant a JSON configuration names, or None."""
     for v in variants:
-        if (v.warps_m, v.warps_n, v.warp_tile_m, v.warp_tile_n, v.block_k, v.pipeline) == (
-                cfg["warps_m"], cfg["warps_n"], cfg["warp_tile_m"], cfg["warp_tile_n"],
-                cfg.get("block_k", 64), cfg.get("pipeline", 0)):
+        # (block extents rather than tiles per wave: a 16-wide side has warp_tile 0.5 in the file)
+        if (v.warps_m, v.warps_n, v.block_m, v.block_n, v.block_k, v.pipeline) == (
+                cfg["warps_m"], cfg["warps_n"], int(cfg["warps_m"] * cfg["warp_tile_m"] * 32),
+                int(cfg["warps_n"] * cfg["warp_tile_n"] * 32), cfg.get("block_k", 64), cfg.get("pipeline", 0)):
             return v
     return None
 

@@ -35,8 +35,8 @@ LAYOUTS = ("rcr", "rrr", "ccr", "crr")  # A, B, C: r row-major, c column-major
 
 def takes(v, a_kmajor: bool, b_kmajor: bool, M: int, N: int, K: int) -> bool:
     """What csrc/gemm.hip: streaming_ok asks of a problem, for C row-major."""
-    return (K >= 128 and (K % 8 == 0 or not (a_kmajor or b_kmajor)) and (a_kmajor or M % 8 == 0)
-            and (b_kmajor or N % 8 == 0))
+    return (K >= 128 and (K % 8 == 0 or not (a_kmajor or b_kmajor)) and (a_kmajor or (M % 8 == 0 and v.block_m != 16))
+            and (b_kmajor or (N % 8 == 0 and v.block_n != 16)))
 
 
 def main(argv=None) -> int:
@@ -61,22 +61,24 @@ def main(argv=None) -> int:
     variants = [v for v in L.variants() if v.pipeline == 7]
 
     def timed(fn) -> float:
-        """Microseconds per call, back to back; a measurement lasts at least 2 ms (calls of
-        10 us timed over 0.15 ms are at the mercy of the clock governor)."""
+        """Microseconds per call, back to back; the median of three measurements of at
+        least 2 ms each (calls of 10 us timed over 0.15 ms are at the mercy of the clock governor)."""
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         for _ in range(4):
             fn()
-        reps = a.reps
-        while True:
+        reps, runs = a.reps, []
+        while len(runs) < 3:  # (the median of three: a slow spell of the GPU lasts several measurements)
             start.record()
             for _ in range(reps):
                 fn()
             stop.record()
             torch.cuda.synchronize()
             ms = start.elapsed_time(stop)
-            if ms >= 2.0 or reps >= 1024:
-                return ms / reps * 1e3
-            reps *= 4
+            if ms < 2.0 and reps < 1024:
+                reps *= 4
+                continue
+            runs.append(ms / reps * 1e3)
+        return sorted(runs)[1]
 
     # (clocks up before the first measurement)
     warm = torch.randn(4096 * 4096, device="cuda").to(dtype)

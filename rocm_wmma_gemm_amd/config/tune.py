@@ -101,13 +101,14 @@ class Tile:
     warps_n: int
     pipeline: int
 
+    # (32 x 32 MFMA tiles per wave; 0.5 for a 16-wide side of the whole-K streaming kernel's tile)
     @property
     def warp_tile_m(self):
-        return self.block_m // self.warps_m // 32
+        return self.block_m // self.warps_m // 32 if self.block_m % (32 * self.warps_m) == 0 else 0.5
 
     @property
     def warp_tile_n(self):
-        return self.block_n // self.warps_n // 32
+        return self.block_n // self.warps_n // 32 if self.block_n % (32 * self.warps_n) == 0 else 0.5
 
 
 # Genes of the search (reference tune.py:75-82 has warps_m, warps_n, warp_tile_m, warp_tile_n,
@@ -115,8 +116,8 @@ class Tile:
 # form are genes too).
 GENES = {
     "pipeline": [0, 1, 2, 3, 4, 5, 6],
-    "block_m": [32, 64, 128, 192, 256],
-    "block_n": [32, 64, 128, 192, 256],
+    "block_m": [16, 32, 64, 128, 192, 256],
+    "block_n": [16, 32, 64, 128, 192, 256],
     "block_k": [32, 64],
     "waves": [(1, 2), (2, 1), (1, 4), (4, 1), (2, 2), (2, 4), (4, 2)],
     "swizzle": [1, 4, 8, 16, -4, -8],
@@ -141,12 +142,15 @@ def tile_feasible(t: Tile, a_kmajor: bool, b_kmajor: bool) -> bool:
     """What the kernel templates take (their static_asserts, restated so that the search
     does not spend a compile on a tuple that cannot build; reference tune.py:105-140)."""
     waves = t.warps_m * t.warps_n
+    if t.pipeline == 7:
+        # whole-K streaming kernel: small tiles, stages of 128, either layout of an operand;
+        # a 16-wide side (at most one) for a K-contiguous operand
+        return (t.block_k == 128 and t.block_m in (16, 32, 64) and t.block_n in (16, 32, 64)
+                and t.block_m + t.block_n >= 48
+                and (a_kmajor or t.block_m != 16) and (b_kmajor or t.block_n != 16)
+                and (t.warps_m, t.warps_n) == (max(1, t.block_m // 32), max(1, t.block_n // 32)))
     if t.block_m % (32 * t.warps_m) or t.block_n % (32 * t.warps_n):
         return False
-    if t.pipeline == 7:
-        # whole-K streaming kernel: small tiles, stages of 128, either layout of an operand
-        return (t.block_k == 128 and t.block_m in (32, 64) and t.block_n in (32, 64)
-                and (t.warps_m, t.warps_n) == (t.block_m // 32, t.block_n // 32))
     if t.block_k == 128:
         return False
     wtm, wtn = t.block_m // t.warps_m, t.block_n // t.warps_n
@@ -232,7 +236,7 @@ def encode(t: Tile, swizzle: int, split: int, touch: int = 0):
 
 def tuple_of(cfg: dict):
     """(tile, swizzle, split, touch) of a JSON "config" object."""
-    t = Tile(cfg["warps_m"] * cfg["warp_tile_m"] * 32, cfg["warps_n"] * cfg["warp_tile_n"] * 32,
+    t = Tile(int(cfg["warps_m"] * cfg["warp_tile_m"] * 32), int(cfg["warps_n"] * cfg["warp_tile_n"] * 32),
              cfg.get("block_k", 64), cfg["warps_m"], cfg["warps_n"], cfg.get("pipeline", 0))
     split = -1 if cfg.get("stream_k") else (-cfg["tail_split"] if cfg.get("tail_split", 0) > 1
                                             else cfg.get("split_k", 1))

@@ -67,7 +67,8 @@ struct model_stream
                          // operand over 256 MB, K-contiguous or not (set by hand, not fitted)
     double taking_turns; // two workgroups on a compute unit: a stage of each takes 1 + this of what
                          // it takes alone, where the compute unit is the bound (set by hand)
-    double stage_us[4]; // per stage of 128 of one compute unit: tiles 32x32, 64x32, 32x64, 64x64
+    double stage_us[8]; // per stage of 128 of one compute unit: tiles 32x32, 64x32, 32x64, 64x64,
+                        // 16x32, 16x64, 32x16, 64x16
 };
 struct model_constants
 {

