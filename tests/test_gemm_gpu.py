@@ -343,7 +343,7 @@ def test_every_variant_and_split_k_agree_with_oracle(loader):
 
 
 def test_whole_k_streaming_kernel_agrees_with_oracle(loader):
-    """The kernel for skinny shapes (pipeline 7: tiles of 32 or 64, one workgroup per tile
+    """The kernel for skinny shapes (pipeline 7: tiles of 16, 32 or 64, one workgroup per tile
     over the whole K, ring of up to 8 stages): every tile, skinny M and skinny N (a
     column-major C runs as the transposed problem), either operand K-contiguous or
     contiguous along M or N on a 32- or a 64-wide side, ragged M and N (rows past the edge are read as zeros and not
