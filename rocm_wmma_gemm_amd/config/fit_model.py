@@ -137,14 +137,14 @@ def stream_estimate(c: dict, rows: int, cols: int, K: int, a_kmajor: bool, b_kma
     # (the workgroups that read the same panel find only part of it in L2)
     sharing = 1.0 + (sharing - 1.0) * c["panel_sharing"]
     rate = c["bytes_per_us_kmajor" if large_kmajor else "bytes_per_us_other"]
-    if not large_kmajor and (bn if wide else bm) == 32:
+    if not large_kmajor and (bn if wide else bm) <= 32:
         rate *= c["half_line"]  # k rows of 64 bytes: half a cache line per request
     if max(rows, cols) * K * 2 > 256 << 20:
         # the large operand does not fit the memory-side cache, which serves part of a
         # repeated call on a smaller one (not fitted: left free it soaks up other effects)
         rate *= c["beyond_cache" if large_kmajor else "beyond_cache_other"]
     l2_rate = c["bytes_per_us_l2"]
-    if not (a_kmajor if wide else b_kmajor) and (bm if wide else bn) == 32:
+    if not (a_kmajor if wide else b_kmajor) and (bm if wide else bn) <= 32:
         l2_rate *= c["half_line"]
     from_memory = (large_bytes * (active / sharing) / rate
                    + small_bytes * active / l2_rate)
@@ -212,11 +212,10 @@ def stream_pick(c: dict, M: int, N: int, K: int, a_kmajor: bool, b_kmajor: bool,
     """The plan (tile, slices, ...) of `plans` that the dispatcher takes (csrc/config_select.cpp:
     stream_plan): of those whose estimate is within STREAM_TIE of the lowest, the fewest
     workgroups per tile, then the lowest estimate; an operand contiguous along M or N sits on a
-    32-wide side of the tile only while it has at most 128 rows, and never on a 16-wide one."""
+    16- or 32-wide side of the tile only while it has at most 128 rows."""
     def allowed(p):
         bm, bn = (int(x) for x in p[0].split("x"))
-        return not ((not a_kmajor and (bm == 16 or (bm == 32 and M > 128)))
-                    or (not b_kmajor and (bn == 16 or (bn == 32 and N > 128))))
+        return not ((not a_kmajor and bm <= 32 and M > 128) or (not b_kmajor and bn <= 32 and N > 128))
 
     def estimate(p):
         bm, bn = (int(x) for x in p[0].split("x"))

@@ -35,8 +35,8 @@ LAYOUTS = ("rcr", "rrr", "ccr", "crr")  # A, B, C: r row-major, c column-major
 
 def takes(v, a_kmajor: bool, b_kmajor: bool, M: int, N: int, K: int) -> bool:
     """What csrc/gemm.hip: streaming_ok asks of a problem, for C row-major."""
-    return (K >= 128 and (K % 8 == 0 or not (a_kmajor or b_kmajor)) and (a_kmajor or (M % 8 == 0 and v.block_m != 16))
-            and (b_kmajor or (N % 8 == 0 and v.block_n != 16)))
+    return (K >= 128 and (K % 8 == 0 or not (a_kmajor or b_kmajor)) and (a_kmajor or M % 8 == 0)
+            and (b_kmajor or N % 8 == 0))
 
 
 def main(argv=None) -> int:

@@ -143,11 +143,10 @@ def tile_feasible(t: Tile, a_kmajor: bool, b_kmajor: bool) -> bool:
     does not spend a compile on a tuple that cannot build; reference tune.py:105-140)."""
     waves = t.warps_m * t.warps_n
     if t.pipeline == 7:
-        # whole-K streaming kernel: small tiles, stages of 128, either layout of an operand;
-        # a 16-wide side (at most one) for a K-contiguous operand
+        # whole-K streaming kernel: small tiles (at most one side 16 wide), stages of 128,
+        # either layout of an operand
         return (t.block_k == 128 and t.block_m in (16, 32, 64) and t.block_n in (16, 32, 64)
                 and t.block_m + t.block_n >= 48
-                and (a_kmajor or t.block_m != 16) and (b_kmajor or t.block_n != 16)
                 and (t.warps_m, t.warps_n) == (max(1, t.block_m // 32), max(1, t.block_n // 32)))
     if t.block_m % (32 * t.warps_m) or t.block_n % (32 * t.warps_n):
         return False

@@ -377,17 +377,12 @@ bool stream_plan(size_t rows, size_t cols, size_t k, bool a_kmajor, bool b_kmajo
             continue;
         }
         const size_t bm = v.block_m, bn = v.block_n;
-        // a 16-wide side is for a K-contiguous operand
-        if((bm == 16 && !a_kmajor) || (bn == 16 && !b_kmajor))
-        {
-            continue;
-        }
         // an operand that is not K-contiguous: k rows of 16-byte pieces; on a 32-wide side of
         // the tile (k rows of 64 bytes, half a cache line a request) only while it is skinny
         // and stays in L2 (1024 x 1024 x 4096 with A column-major: 28.4 us on the 32 x 64
         // tile, 18.6 on 64 x 64)
-        if((!a_kmajor && (rows % 8 != 0 || (bm == 32 && rows > 128)))
-           || (!b_kmajor && (cols % 8 != 0 || (bn == 32 && cols > 128))))
+        if((!a_kmajor && (rows % 8 != 0 || (bm <= 32 && rows > 128)))
+           || (!b_kmajor && (cols % 8 != 0 || (bn <= 32 && cols > 128))))
         {
             continue;
         }
@@ -401,9 +396,9 @@ bool stream_plan(size_t rows, size_t cols, size_t k, bool a_kmajor, bool b_kmajo
         const double sharing = 1.0 + (static_cast<double>(wide ? tm : tn) - 1.0) * c.panel_sharing;
         const bool   large_kmajor = wide ? b_kmajor : a_kmajor, small_kmajor = wide ? a_kmajor : b_kmajor;
         const double rate    = (large_kmajor ? c.bytes_per_us_kmajor : c.bytes_per_us_other)
-                            * (!large_kmajor && (wide ? bn : bm) == 32 ? c.half_line : 1.0)
+                            * (!large_kmajor && (wide ? bn : bm) <= 32 ? c.half_line : 1.0)
                             * (std::max(rows, cols) * k * 2 > (size_t{256} << 20) ? (large_kmajor ? c.beyond_cache : c.beyond_cache_other) : 1.0);
-        const double l2_rate = c.bytes_per_us_l2 * (!small_kmajor && (wide ? bm : bn) == 32 ? c.half_line : 1.0);
+        const double l2_rate = c.bytes_per_us_l2 * (!small_kmajor && (wide ? bm : bn) <= 32 ? c.half_line : 1.0);
         for(size_t s = 1; s <= 8; s *= 2)
         {
             // (the counters of the tiles that several workgroups share: 4096 a launch)

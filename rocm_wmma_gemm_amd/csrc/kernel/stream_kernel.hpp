@@ -17,7 +17,7 @@
 //     bytes (a 64-wide side: one whole cache line, what the large operand wants) or 64 (a
 //     32-wide side: half the waste where the small operand has 16 rows), and the fragments
 //     are transposed on the way to registers by ds_read_b64_tr_b16;
-//   - a side may also be 16 wide, for a K-contiguous operand: a small operand of at most 16
+//   - a side may also be 16 wide: a small operand of at most 16
 //     rows then puts a quarter less through the compute unit's load path than 32 rows, half
 //     of them zeros (16 x 4096 x 14336: 22.9 -> 19.9 us), and 16 rows of the LARGE operand
 //     per workgroup make 256 tiles of N = 4096, a workgroup for every compute unit without
@@ -100,7 +100,6 @@ struct stream_gemm
     static constexpr int MAX_SLICES = 8; // workgroups that may share a tile (args.k_slices)
     static_assert((BM == 16 || BM == 32 || BM == 64) && (BN == 16 || BN == 32 || BN == 64) && BM + BN >= 48,
                   "tiles of 16, 32 or 64 rows and columns");
-    static_assert((A_KMAJOR || BM != 16) && (B_KMAJOR || BN != 16), "a 16-wide side is K-contiguous");
     static_assert(DEPTH >= 3 && (DEPTH - 1) * PER < 64, "ring depth against the 6-bit vmcnt");
     static_assert(WAVES * BM * BN * 4 <= LDS_BYTES, "the partial tiles of the waves reuse the ring");
 
@@ -146,11 +145,26 @@ struct stream_gemm
         return W == 64 ? ((k & 3) ^ ((k >> 3) & 1)) : ((k >> 3) & 1);
     }
 
+    // W = 16: k rows of 32 bytes, 32 of them per 1 KiB load.  The 4 rows that 16 lanes of a
+    // transposing read touch are 128 contiguous bytes, and the next 16 lanes' rows, 8 further
+    // on, would start 256 bytes later on the same banks: of every second run of 8 rows the
+    // two halves change places (row r of a wave's 32 lies in place r ^ 4 when r / 8 is odd),
+    // so that one group reads the low 128 bytes of its 256 and the next the high.
+    __device__ __forceinline__ static int mn_row16(int r)
+    {
+        return r ^ (((r >> 3) & 1) << 2);
+    }
+
     // byte offset of lane l's 16 bytes of load `wave` (+ 4 i) from the operand's stage origin
     template<int W>
     __device__ __forceinline__ static unsigned int mn_load_offset(int lane, int wave, long long ld)
     {
         constexpr int LANES_PER_ROW = W / 8, ROWS_PER_LOAD = 512 / W;
+        if constexpr(W == 16)
+        {
+            // a k row is one 32-byte piece: the rows change places instead (mn_row16)
+            return (unsigned int)(((32 * wave + mn_row16(lane >> 1)) * ld + (lane & 1) * 8) * 2);
+        }
         const int     k      = ROWS_PER_LOAD * wave + lane / LANES_PER_ROW; // (mod 16 as for every i)
         const int     place  = (lane % LANES_PER_ROW) >> 1;
         const int     piece  = place ^ mn_piece<W>(k);
@@ -162,6 +176,10 @@ struct stream_gemm
     template<int W>
     __device__ __forceinline__ static int mn_read_offset(int wave, int sub, int slot)
     {
+        if constexpr(W == 16)
+        {
+            return (32 * wave + mn_row16(8 * sub + (slot >> 2))) * 32 + (slot & 3) * 8;
+        }
         const int k = 32 * wave + 8 * sub + (slot >> 2);
         return k * (2 * W) + mn_piece<W>(k) * 32 + (slot & 3) * 8;
     }
@@ -208,6 +226,21 @@ struct stream_gemm
                      : "memory");
         f[0] = u32x4{l0.x, l0.y, h0.x, h0.y};
         f[1] = u32x4{l1.x, l1.y, h1.x, h1.y};
+    }
+
+    // a 16-wide side: rows of 32 bytes, one column piece; the 4 rows further on lie 128 bytes
+    // up or down (mn_row16): at addr ^ 128
+    __device__ __forceinline__ static void transposed(unsigned int addr, u32x4 (&f)[1])
+    {
+        const unsigned int a1 = addr ^ 128u;
+        uint2              l0, h0;
+        asm volatile("ds_read_b64_tr_b16 %0, %2\n\t"
+                     "ds_read_b64_tr_b16 %1, %3\n\t"
+                     "s_waitcnt lgkmcnt(0)"
+                     : "=&v"(l0), "=&v"(h0)
+                     : "v"(addr), "v"(a1)
+                     : "memory");
+        f[0] = u32x4{l0.x, l0.y, h0.x, h0.y};
     }
 
     // acc += A fragment x B fragment, in place.  (Written out: left to place the
@@ -308,6 +341,7 @@ struct stream_gemm
                                              : mn_load_offset<BN>(lane, wave, ldb);
         // bytes from load i to load i+1 (16 rows, or 4 loads' worth of k rows), and from stage
         // to stage
+        // (a 16-wide side has one load per wave and stage, and no step)
         const unsigned int step_a  = (unsigned int)((A_KMAJOR ? 16 : 4 * (512 / BM)) * lda * 2);
         const unsigned int step_b  = (unsigned int)((B_KMAJOR ? 16 : 4 * (512 / BN)) * ldb * 2);
         const unsigned int stage_a = A_KMAJOR ? (unsigned int)ROW_BYTES : (unsigned int)(BK * lda * 2);

@@ -72,8 +72,7 @@ constexpr kernel_fn entry()
         return &device::gemm_entry<device::direct_gemm<kIn, out_t, RWG_AK != 0, RWG_BK != 0, BM, BN, BK, WM, WN, 4,
                                                        MODE == device::load_mode::vec_guarded>>;
     }
-    else if constexpr(MODE != device::load_mode::scalar && PIPE == 7 && (RWG_AK != 0 || BM != 16)
-                      && (RWG_BK != 0 || BN != 16))
+    else if constexpr(MODE != device::load_mode::scalar && PIPE == 7)
     {
         // (one kernel for whole and ragged tiles: its loads and stores are always guarded)
         static_assert(BK == 128, "the streaming kernel's stages are 128 wide");

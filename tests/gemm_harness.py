@@ -57,7 +57,7 @@ def built_for(v, lc, la, lb, K=None, M=None, N=None):
     kernel space (C row-major: A row-major, B column-major; a column-major C swaps the
     operands); the whole-K streaming kernel (pipeline 7) needs at least one stage of 128 of
     K, 16-byte aligned rows (K a multiple of 8 where an operand is K-contiguous; M or N a multiple
-    of 8 where an operand is contiguous along it, and not on a 16-wide side of the tile)."""
+    of 8 where an operand is contiguous along it)."""
     if v.pipeline == 0:
         return True
     a_k, b_k = la == 0, lb == 1
@@ -66,8 +66,8 @@ def built_for(v, lc, la, lb, K=None, M=None, N=None):
     if v.pipeline == 7:
         rows, cols = (M, N) if lc == 0 else (N, M)
         return ((K is None or (K >= 128 and (K % 8 == 0 or not (a_k or b_k))))
-                and (a_k or (v.block_m != 16 and (rows is None or rows % 8 == 0)))
-                and (b_k or (v.block_n != 16 and (cols is None or cols % 8 == 0))))
+                and (a_k or rows is None or rows % 8 == 0)
+                and (b_k or cols is None or cols % 8 == 0))
     return (v.block_m % 128 == 0 or a_k) and (v.block_n % 128 == 0 or b_k)
 
 
