@@ -17,15 +17,21 @@
 //     bytes (a 64-wide side: one whole cache line, what the large operand wants) or 64 (a
 //     32-wide side: half the waste where the small operand has 16 rows), and the fragments
 //     are transposed on the way to registers by ds_read_b64_tr_b16;
-//   - a side may also be 16 wide: a small operand of at most 16
-//     rows then puts a quarter less through the compute unit's load path than 32 rows, half
-//     of them zeros (16 x 4096 x 14336: 22.9 -> 19.9 us), and 16 rows of the LARGE operand
-//     per workgroup make 256 tiles of N = 4096, a workgroup for every compute unit without
-//     any exchange between workgroups (32 x 4096 x 14336: 22.6 -> 19.4 us);
-//   - the LDS holds a ring of 3 or 4 stages of BK = 128 per workgroup, two workgroups to a
-//     compute unit (48..96 KB of loads in flight per compute unit: what it takes to cover
-//     the latency of HBM at 20..40 GB/s per compute unit), filled by buffer_load ... lds,
-//     1 KiB per instruction (4 rows x 256 bytes);
+//   - a side may also be 16 wide (k rows of 32 bytes where the operand is contiguous along
+//     M or N): a small operand of at most 16 rows then puts a quarter less through the
+//     compute unit's load path than 32 rows, half of them zeros (16 x 4096 x 14336: 22.9 ->
+//     19.9 us), and 16 rows of the LARGE operand per workgroup make 256 tiles of N = 4096, a
+//     workgroup for every compute unit without any exchange between workgroups
+//     (32 x 4096 x 14336: 22.6 -> 19.4 us);
+//   - the LDS holds a ring of 3 to 6 stages of BK = 128 per workgroup (what fits 76 KB), two
+//     workgroups to a compute unit (48..96 KB of loads in flight per compute unit: what it
+//     takes to cover the latency of HBM at 20..40 GB/s per compute unit), filled by
+//     buffer_load ... lds, 1 KiB per instruction (4 rows x 256 bytes);
+//   - where the tile grid is one tile high, the panels start their walk along K at
+//     staggered stages, so that the workgroups do not all ask the same memory channels at
+//     the same time;
+//   - the MFMAs are written out, accumulating in place: the compiler's own placement moved
+//     the accumulators around every stage;
 //   - the four waves split the K range of a stage (32 each) and every wave multiplies the
 //     whole tile on v_mfma_f32_16x16x32; at the end the four partial tiles are added in
 //     wave order through LDS and the sum is converted and stored;
@@ -42,12 +48,13 @@
 // LDS layout of a stage: the A tile (BM rows), then the B tile (BN rows).  K-contiguous
 // operand: a row is 16 chunks of 16 bytes, chunk c of row r in slot c ^ (r mod 16), so
 // that the 16 rows a fragment read touches per k chunk fall on 16 different slots (all 64
-// banks once).  M/N-contiguous operand: 128 k rows of 64 or 32 elements; the 32-byte
-// pieces of k row k are permuted within the row (mn_piece), so that the 4 k rows x 32
-// bytes that 16 lanes of a transposing read touch, and those of the next 16 lanes 8 rows
-// further on, fall on different banks (64 wide, in memory order, they are 4-way
-// conflicts: 16 x 8192 x 8192 with B row-major 29.6 us, with the pieces permuted 28.1 us;
-// B column-major, whose fragments are plain 16-byte reads, 24.3 us).
+// banks once).  M/N-contiguous operand: 128 k rows of 64, 32 or 16 elements; the 32-byte
+// pieces of k row k are permuted within the row (mn_piece; 16 wide: the rows themselves,
+// mn_row16), so that the 4 k rows x 32 bytes that 16 lanes of a transposing read touch, and
+// those of the next 16 lanes 8 rows further on, fall on different banks (64 wide, in memory
+// order, they are 4-way conflicts: 16 x 8192 x 8192 with B row-major 29.6 us, with the
+// pieces permuted 28.1 us; B column-major, whose fragments are plain 16-byte reads, 24.3 us,
+// at the time; the bank-conflict counter now reads the same for both kinds of kernel).
 //
 // Role with respect to the reference: as the other kernels, its gemm_impl (reference
 // rocm_wmma_gemm/include/rocm_wmma_gemm/kernel/kernel.hpp:108-556); the reference has no
