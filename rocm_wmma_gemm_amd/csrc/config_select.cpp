@@ -476,6 +476,23 @@ launch_plan select_plan_from(const tuned_entry* table, size_t count, size_t m, s
     return heuristic_plan(m, n, k, lc);
 }
 
+namespace
+{
+// What the whole-K streaming kernel asks of a shape (the pointers are the launch's business):
+// a stage of K, 16-byte aligned rows of either kind.
+bool streaming_takes(size_t m, size_t n, size_t k, int lc, int la, int lb)
+{
+    const size_t rows = lc == 0 ? m : n, cols = lc == 0 ? n : m;
+    bool         a_kmajor = la == 0, b_kmajor = lb == 1;
+    if(lc != 0)
+    {
+        std::swap(a_kmajor, b_kmajor);
+    }
+    return k >= 128 && ((!a_kmajor && !b_kmajor) || k % 8 == 0) && (a_kmajor || rows % 8 == 0)
+           && (b_kmajor || cols % 8 == 0);
+}
+} // namespace
+
 launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int la, int lb, size_t batch,
                         size_t cus)
 {
@@ -492,6 +509,20 @@ launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int 
        || (group != 0 && find_exact(tuned_table, tuned_count, m, n, k, 0, la, lb, lc, &plan)))
     {
         return plan;
+    }
+    // ... fewer than 16 rows (or columns) as 16 of them, where that entry runs on the streaming
+    // kernel: the tiles, the workgroups and the bytes moved are the same (rows past M are read
+    // as zeros), so the plan tuned for 16 is the plan for 1 to 15
+    // (8 x 4096 x 14336: 19.9 us on the entry's 32 x 16 tile, 23.6 on the estimate's pick)
+    if(std::min(m, n) < 16 && std::max(m, n) >= 512)
+    {
+        const size_t m16 = std::max<size_t>(m, 16), n16 = std::max<size_t>(n, 16);
+        if((find_exact(tuned_table, tuned_count, m16, n16, k, group, la, lb, lc, &plan)
+            || (group != 0 && find_exact(tuned_table, tuned_count, m16, n16, k, 0, la, lb, lc, &plan)))
+           && model_variants[plan.variant].pipeline == 7 && streaming_takes(m, n, k, lc, la, lb))
+        {
+            return plan;
+        }
     }
     // ... then the model for regular shapes, and the nearest tuned entry for the rest
     if(model_plan(m, n, k, lc, la, lb, &plan, 1, cus))
@@ -510,19 +541,9 @@ launch_plan select_plan(size_t m, size_t n, size_t k, int type_idx, int lc, int 
     // wants 16-byte aligned rows of either kind: a
     // shape that does not fit takes the shape heuristic's plan instead.
     const model_variant& v = model_variants[plan.variant];
-    if(v.pipeline == 7)
+    if(v.pipeline == 7 && !streaming_takes(m, n, k, lc, la, lb))
     {
-        const size_t rows = lc == 0 ? m : n, cols = lc == 0 ? n : m;
-        bool         a_kmajor = la == 0, b_kmajor = lb == 1;
-        if(lc != 0)
-        {
-            std::swap(a_kmajor, b_kmajor);
-        }
-        if(k < 128 || ((a_kmajor || b_kmajor) && k % 8 != 0) || (!a_kmajor && rows % 8 != 0)
-           || (!b_kmajor && cols % 8 != 0))
-        {
-            return heuristic_plan(m, n, k, lc);
-        }
+        return heuristic_plan(m, n, k, lc);
     }
     return plan;
 }

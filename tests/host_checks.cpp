@@ -214,6 +214,21 @@ static int check_select()
         if(tiles[q.variant].pipeline != 0 || q.split_k < 2)
             return fail("select: skinny shape with K = 4001");
     }
+    // fewer than 16 rows take the plan tuned for 16 rows of the same N, K and layouts when it
+    // is the streaming kernel's (and the shape suits that kernel)
+    {
+        const launch_plan q16 = select_plan(16, 4096, 14336, 0, 0, 0, 1), q3 = select_plan(3, 4096, 14336, 0, 0, 0, 1);
+        if(tiles[q16.variant].pipeline != 7 || q3.variant != q16.variant || q3.split_k != q16.split_k)
+            return fail("select: 3 rows take the plan of the tuned 16 rows");
+        // (the model alone would send 3 rows elsewhere: that is what the entry is for)
+        launch_plan by_model;
+        if(model_plan(3, 4096, 14336, 0, 0, 1, &by_model) && by_model.variant == q16.variant && by_model.split_k == q16.split_k)
+            return fail("select: the check above needs a shape where entry and estimate differ");
+        // A stored K x M with 3 rows: k rows of 6 bytes, not the streaming kernel's
+        const launch_plan r3 = select_plan(3, 4096, 14336, 0, 0, 1, 1);
+        if(tiles[r3.variant].pipeline == 7)
+            return fail("select: 3 rows that are not K-contiguous must not stream");
+    }
     // next to 1024^3, whose entries run on the streaming kernel: K-contiguous rows that are
     // not 16-byte aligned must not inherit that plan
     {
