@@ -189,6 +189,28 @@ def test_seeded_random_skinny_and_small_shapes_through_the_default_dispatch(load
     assert pipelines.get(7, 0) >= 25, pipelines  # the streaming kernel is what most of these run on
 
 
+def test_fewer_than_sixteen_rows_take_the_plan_tuned_for_sixteen(loader):
+    """1 to 15 rows (or columns) against an N x K that has a tuned entry for 16 rows on the
+    streaming kernel are served by that entry's plan (same tiles, rows past M read as zeros);
+    a small operand stored K x M with rows that are not 16-byte aligned is not.  Each element
+    against the oracle."""
+    N, K = 4096, 14336
+    want = loader.select(16, N, K, 0, 0, 0, 1)
+    assert loader.variants()[want[0]].pipeline == 7
+    for M in (1, 3, 8, 15):
+        assert loader.select(M, N, K, 0, 0, 0, 1) == want, M
+        A, B = make_inputs(M, N, K, 0, 1, O.F16, seed_a=60 + M, seed_b=61)
+        gpu = run_gpu(loader, A, B, M, N, K, 0, 0, 1, O.F16, O.F16)
+        check_against_oracle(gpu, A, B, M, N, K, 0, 0, 1, O.F16, O.F16)
+    # (A column-major: 8 rows are 16 bytes per k row and stream, 3 rows do not)
+    assert loader.variants()[loader.select(8, N, K, 0, 0, 1, 1)[0]].pipeline == 7
+    assert loader.variants()[loader.select(3, N, K, 0, 0, 1, 1)[0]].pipeline != 7
+    for M in (8, 3):
+        A, B = make_inputs(M, N, K, 1, 1, O.BF16, seed_a=70 + M, seed_b=71)
+        gpu = run_gpu(loader, A, B, M, N, K, 0, 1, 1, O.BF16, O.F32)
+        check_against_oracle(gpu, A, B, M, N, K, 0, 1, 1, O.BF16, O.F32)
+
+
 def test_seeded_random_large_shapes_through_the_default_dispatch(loader):
     """The same for 10 problems of many tiles (extents 1500..5200, K 500..4200, all
     alignment classes): every element through the row/column checksums, a 32-row band in
