@@ -38,6 +38,10 @@ SETS = {
     "projection": "4096,11008,4096:4096,4096,11008:8192,8192,4096:4096,12288,4096:8192,1024,8192:"
                   "4096,4096,14336:2048,8192,2048:12288,4096,4096:5120,5120,5120:8192,3584,7168:"
                   "7168,7168,7168:8192,28672,8192:8192,8192,28672",
+    # 256 to 1024 rows of activations against transformer weight matrices
+    "prefill": ":".join(f"{m},{n},{k}" for m in (256, 512, 1024)
+                        for n, k in ((4096, 4096), (8192, 8192), (4096, 14336), (14336, 4096),
+                                     (28672, 8192), (8192, 28672))),
     # many small problems in one strided-batch call (run with --batch_count, default 64)
     "batched": "128,128,128:256,256,256:512,512,512:1024,1024,1024:256,256,4096:"
                "384,640,512:1000,1000,1000:2048,2048,2048",
@@ -145,6 +149,7 @@ def main(argv=None) -> int:
     title = {"square": "Square matrices", "rectangle": "Rectangular matrices",
              "other": "Projection, skinny, ragged and long-K shapes",
              "projection": "Transformer projection shapes",
+             "prefill": "256 to 1024 rows against transformer weight matrices",
              "batched": f"Strided batches of {batch} small problems"}.get(a.set, "Selected shapes")
     flops = "2·M·N·K" if batch == 1 else f"{batch}·2·M·N·K"
     lines = [f"# {title}: this library, rocBLAS and hipBLASLt on one MI355X\n",
