@@ -1014,6 +1014,16 @@ def test_llm_projection_shapes(loader, M, N, K):
         _full_size_case(loader, M, N, K, lc, la, lb, "f32_f16", whole=M <= 128)
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 4096, 4096), (256, 28672, 8192), (512, 14336, 4096),
+                                   (512, 8192, 28672), (1024, 4096, 14336)])
+def test_a_few_hundred_rows_against_projection_weights(loader, M, N, K):
+    """256 to 1024 rows against transformer weight matrices, through the tuned entries of
+    these shapes (the streaming kernel, the 128x128 ring of 4, the persistent kernel with
+    and without a split, the ping-pong kernel with split-K, depending on shape and layout)."""
+    for (lc, la, lb), tname in [((0, 0, 1), "f16_f16"), ((0, 0, 0), "bf16_bf16"), ((1, 1, 1), "f32_bf16")]:
+        _full_size_case(loader, M, N, K, lc, la, lb, tname)
+
+
 @pytest.mark.parametrize("M,N,K", [(4095, 5121, 3001), (1000, 1000, 1000), (1024, 1024, 65536),
                                    (8191, 8191, 8191)])
 def test_edge_tile_and_long_k(loader, M, N, K):
