@@ -69,7 +69,7 @@ typedef struct rocm_wmma_gemm_variant_info
     int block_m, block_n, block_k; /* workgroup tile */
     int warps_m, warps_n;          /* wave grid inside the workgroup */
     int warp_tile_m, warp_tile_n;  /* 32x32 MFMA tiles per wave (0: a 16-wide side of the streaming kernel's tile) */
-    int pipeline;                  /* 0 = register-staged general path, 1 = direct-to-LDS, 2 = direct-to-LDS ping-pong, 3, 4 = 1, 2 on the 16x16x32 MFMA, 5 = one wave per SIMD, persistent workgroups, 6 = 1 with a ring of 4 tiles at BLOCK_K 64 */
+    int pipeline;                  /* 0 = register-staged general path, 1 = direct-to-LDS, 2 = direct-to-LDS ping-pong, 3, 4 = 1, 2 on the 16x16x32 MFMA, 5 = one wave per SIMD, persistent workgroups, 6 = 1 with a ring of 4 tiles at BLOCK_K 64, 7 = whole-K streaming kernel (tiles of 16 to 128 rows by 16 to 64 columns, one workgroup per tile over all of K, for skinny and small problems) */
     int lds_bytes;                 /* static LDS per workgroup */
     int threads;                   /* workgroup size */
 } rocm_wmma_gemm_variant_info;
@@ -152,8 +152,11 @@ int rocm_wmma_gemm_register_variant(int block_m, int block_n, int block_k, int w
  * call needs more).  Waits for the device to finish first.  Returns 0 when the buffer is
  * gone or was never there, 1 when it was kept because a call on a capturing stream has
  * used it (a graph may hold its address), ROCM_WMMA_GEMM_ERR_RUNTIME without a device.
- * The next call that needs scratch memory allocates again.  No counterpart in the
- * reference, which owns no memory. */
+ * The next call that needs scratch memory allocates again.  Also puts the arrival counters
+ * of shared tiles back to zero (they return to zero by themselves after every launch that
+ * runs to its end; a kernel killed in flight may leave one counting, which later launches
+ * ignore anyway because every launch tags its counts).  No counterpart in the reference,
+ * which owns no memory. */
 int rocm_wmma_gemm_workspace_release(void);
 
 /* Size of the fixed per-GPU scratch buffer behind rocm_wmma_gemm_noalloc. */
@@ -177,7 +180,10 @@ int rocm_wmma_gemm_workspace_release(void);
  *     call outside graph capture.
  *   - Every call on a GPU uses that GPU's one array, which keeps the previous call's
  *     contents; nothing has to start at zero (each kernel writes what a later one reads).
- *     Calls that overlap on one GPU (two streams, two threads) race on it: order them.
+ *     Calls of THIS entry point that overlap on one GPU (two streams, two threads, replays
+ *     of two captured graphs) race on the array and on the arrival counters of shared
+ *     tiles that go with it: order them.  Calls of the other entry points may overlap with
+ *     them freely: those use the library's allocated buffer and counters of their own.
  * Returns ROCM_WMMA_GEMM_OK or one of the codes above; a layout code outside {0, 1} is
  * ROCM_WMMA_GEMM_ERR_ARGUMENT here rather than a silent no-op. */
 int rocm_wmma_gemm_noalloc(int type_idx, void* C, void* A, void* B, size_t M, size_t N, size_t K,

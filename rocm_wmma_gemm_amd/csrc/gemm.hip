@@ -11,7 +11,9 @@
 #include <mutex>
 #include <stdexcept>
 #include <string>
+#include <tuple>
 #include <type_traits>
+#include <utility>
 
 #include "config_select.hpp"
 #include "kernel_table.hpp"
@@ -121,16 +123,50 @@ size_t out_bytes(int type_idx)
     return (type_idx == 1 || type_idx == 3) ? 4 : 2;
 }
 
+// Every kernel of the library is enqueued through this: the launch's own return code is kept
+// per host thread, so that the entry points that return a status report what THEIR launches
+// did, not an error some earlier call of anybody's left in the runtime's per-thread error
+// state (hipPeekAtLastError cannot tell the two apart).
+thread_local hipError_t launch_failure = hipSuccess;
+
+template<class... P, class... A, size_t... I>
+void enqueue_impl(void (*kernel)(P...), dim3 grid, dim3 block, hipStream_t stream, std::index_sequence<I...>,
+                  A&&... a)
+{
+    std::tuple<std::remove_cv_t<std::remove_reference_t<P>>...> params(std::forward<A>(a)...);
+    void*            ptrs[] = {static_cast<void*>(&std::get<I>(params))...};
+    const hipError_t rc = hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, ptrs, 0, stream);
+    if(rc != hipSuccess && launch_failure == hipSuccess)
+    {
+        launch_failure = rc;
+    }
+}
+
+template<class... P, class... A>
+void enqueue(void (*kernel)(P...), dim3 grid, dim3 block, hipStream_t stream, A&&... a)
+{
+    static_assert(sizeof...(P) == sizeof...(A), "one argument per kernel parameter");
+    enqueue_impl(kernel, grid, block, stream, std::index_sequence_for<P...>{}, std::forward<A>(a)...);
+}
+
 // Arrival counters of the whole-K streaming kernel's K slices (one per tile and batch entry
-// of a launch): zero when the code object is loaded, and put back to zero by the workgroup
-// that finishes a tile.  One array per GPU; launches that use it also hold the scratch
-// buffer below (their partial tiles live there), so they follow one another as its users do.
+// of a launch).  A counter holds (epoch << 8 | arrivals): the host gives every launch that
+// shares tiles an epoch of its own, a workgroup that finds another epoch in its counter
+// starts counting from zero, and the workgroup that finishes a tile puts the count back to
+// zero, so a replay of a captured launch (same epoch) starts from zero too and a count that
+// a killed kernel left behind cannot be mistaken for this launch's.  Two arrays per GPU:
+// one for the calls that lease the library's scratch buffer (the lease orders them, so they
+// never count in the same slots at the same time), one for the entry point that allocates
+// nothing, which takes no lease (its calls are ordered by the caller, like their scratch
+// array); a call of one kind never meets a call of the other in a counter.
 constexpr size_t stream_arrival_slots = 4096;
 __attribute__((used)) static __device__ unsigned int stream_arrivals[stream_arrival_slots];
-std::mutex    arrivals_mutex;
-unsigned int* arrivals_address[64] = {};
+__attribute__((used)) static __device__ unsigned int noalloc_arrivals[stream_arrival_slots];
+std::mutex            arrivals_mutex;
+unsigned int*         arrivals_address[64][2] = {};
+std::atomic<unsigned> arrival_epoch{0};
 
-unsigned int* arrivals_of_current_device()
+unsigned int* arrivals_of_current_device(bool noalloc)
 {
     int dev = -1;
     if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
@@ -138,17 +174,30 @@ unsigned int* arrivals_of_current_device()
         return nullptr;
     }
     std::lock_guard<std::mutex> lock(arrivals_mutex);
-    if(arrivals_address[dev] == nullptr)
+    if(arrivals_address[dev][0] == nullptr)
     {
-        void* p = nullptr;
-        if(hipGetSymbolAddress(&p, HIP_SYMBOL(stream_arrivals)) != hipSuccess || p == nullptr)
+        void *p = nullptr, *q = nullptr;
+        if(hipGetSymbolAddress(&p, HIP_SYMBOL(stream_arrivals)) != hipSuccess || p == nullptr
+           || hipGetSymbolAddress(&q, HIP_SYMBOL(noalloc_arrivals)) != hipSuccess || q == nullptr)
         {
             (void)hipGetLastError();
             return nullptr;
         }
-        arrivals_address[dev] = static_cast<unsigned int*>(p);
+        arrivals_address[dev][0] = static_cast<unsigned int*>(p);
+        arrivals_address[dev][1] = static_cast<unsigned int*>(q);
     }
-    return arrivals_address[dev];
+    return arrivals_address[dev][noalloc ? 1 : 0];
+}
+
+// an epoch for one launch that shares tiles: 24 bits, never zero (a fresh counter reads zero)
+unsigned int next_arrival_epoch()
+{
+    unsigned int e;
+    do
+    {
+        e = (arrival_epoch.fetch_add(1, std::memory_order_relaxed) + 1) & 0xffffffu;
+    } while(e == 0);
+    return e;
 }
 
 // Library-owned scratch memory, one buffer per device: fp32 partial planes of split-K
@@ -375,8 +424,8 @@ template<class OutT>
 void zero_fill(void* C, size_t count, hipStream_t stream)
 {
     const int blocks = static_cast<int>(std::min<size_t>((count + 255) / 256, 65535));
-    device::fill_zero<OutT><<<dim3(blocks), dim3(256), 0, stream>>>(static_cast<OutT*>(C),
-                                                                     static_cast<long long>(count));
+    enqueue(&device::fill_zero<OutT>, dim3(blocks), dim3(256), stream, static_cast<OutT*>(C),
+            static_cast<long long>(count));
 }
 
 // Variant that serves shapes a direct-to-LDS variant cannot take: the staged
@@ -484,7 +533,7 @@ int launch_streaming(int type_idx, const launch_plan& plan, const kernel_problem
     if(slices > 1)
     {
         const size_t bytes = tiles * nb_max * slices * tile_floats * sizeof(float);
-        arrivals           = arrivals_of_current_device();
+        arrivals           = arrivals_of_current_device(fixed != nullptr);
         if(fixed != nullptr)
         {
             partials = bytes <= fixed->bytes ? fixed->ptr : nullptr;
@@ -519,9 +568,11 @@ int launch_streaming(int type_idx, const launch_plan& plan, const kernel_problem
         args.k_slices       = static_cast<int>(slices);
         args.partials       = reinterpret_cast<float*>(partials);
         args.arrivals       = arrivals;
+        args.arrival_epoch  = slices > 1 ? next_arrival_epoch() : 0;
         args.blocks_per_batch = static_cast<int>(tiles);
         args.batches          = static_cast<int>(nb);
-        fn<<<dim3(static_cast<unsigned>(tiles * slices), static_cast<unsigned>(nb)), dim3(v.threads), 0, stream>>>(args);
+        enqueue(fn, dim3(static_cast<unsigned>(tiles * slices), static_cast<unsigned>(nb)), dim3(v.threads), stream,
+                args);
     }
     return 0;
 }
@@ -826,7 +877,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
                 jobs[1] = jobs[0];
             }
             // one launch for both operands: a dependent launch costs as much as a small copy
-            device::pack_padded<unsigned short><<<dim3(blocks, count, nb), dim3(256), 0, stream>>>(jobs[0], jobs[1]);
+            enqueue(&device::pack_padded<unsigned short>, dim3(blocks, count, nb), dim3(256), stream, jobs[0], jobs[1]);
         }
         if(copy_a)
         {
@@ -848,7 +899,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
     for(size_t b0 = 0; b0 < p.batch; b0 += batches_per_launch)
     {
         const size_t nb = std::min(batches_per_launch, p.batch - b0);
-        device::gemm_args args;
+        device::gemm_args args{};
         args.C = static_cast<char*>(p.C) + b0 * p.stride_c * sizeof(OutT);
         args.A = static_cast<const char*>(a_ptr) + b0 * stride_a * in_bytes;
         args.B = static_cast<const char*>(b_ptr) + b0 * stride_b * in_bytes;
@@ -871,6 +922,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         args.stream_units     = static_cast<int>(stream_units);
         args.k_tail           = k_tail;
         args.warm_ahead       = persistent && plan.touch > 0 ? std::min(plan.touch, 3) : 0;
+
         args.batch_by_xcd     = (persistent || v.pipeline == 6) && nb > 1 && split_k == 1 && stream_groups == 0
                                         && blocks_per_batch * nb < (size_t{1} << 31)
                                     ? 1
@@ -888,17 +940,17 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
                 grid = dim3(static_cast<unsigned>(stream_groups), 1);
             }
         }
-        fn<<<grid, dim3(v.threads), 0, stream>>>(args);
+        enqueue(fn, grid, dim3(v.threads), stream, args);
         if(stream_groups > 0)
         {
             if(stream_units % static_cast<size_t>(k_steps) != 0)
             {
                 // (ranges of whole tiles cut nothing)
-                device::reduce_stream_tiles<OutT>
-                    <<<dim3(static_cast<unsigned>(tiles * nb * (v.block_m * v.block_n / device::reduce_chunk_elems))),
-                       dim3(256), 0, stream>>>(static_cast<OutT*>(args.C), partials, args.M, args.N, v.block_m,
-                                               v.block_n, args.grid_m, args.grid_n, args.group, k_steps,
-                                               args.stream_units, args.batch_stride_c);
+                enqueue(&device::reduce_stream_tiles<OutT>,
+                        dim3(static_cast<unsigned>(tiles * nb * (v.block_m * v.block_n / device::reduce_chunk_elems))),
+                        dim3(256), stream, static_cast<OutT*>(args.C), partials, args.M, args.N, v.block_m,
+                        v.block_n, args.grid_m, args.grid_n, args.group, k_steps, args.stream_units,
+                        args.batch_stride_c);
             }
             continue;
         }
@@ -906,19 +958,17 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         {
             const long long plane  = static_cast<long long>(p.M) * static_cast<long long>(p.N);
             const int       blocks = static_cast<int>(std::min<long long>((plane + 255) / 256, 4096));
-            device::reduce_partials<OutT>
-                <<<dim3(blocks, static_cast<unsigned>(nb)), dim3(256), 0, stream>>>(
+            enqueue(&device::reduce_partials<OutT>, dim3(blocks, static_cast<unsigned>(nb)), dim3(256), stream,
                     static_cast<OutT*>(args.C), partials, plane, split_k, args.batch_stride_c);
         }
         else if(split_k > 1)
         {
-            device::reduce_split_tiles<OutT>
-                <<<dim3(static_cast<unsigned>((tiles - tail_begin)
-                                              * (v.block_m * v.block_n / device::reduce_chunk_elems)),
-                        static_cast<unsigned>(nb)),
-                   dim3(256), 0, stream>>>(static_cast<OutT*>(args.C), partials, args.M, args.N, v.block_m, v.block_n,
-                             args.grid_m, args.grid_n, args.group, args.tail_begin, split_k,
-                             args.batch_stride_c);
+            enqueue(&device::reduce_split_tiles<OutT>,
+                    dim3(static_cast<unsigned>((tiles - tail_begin)
+                                               * (v.block_m * v.block_n / device::reduce_chunk_elems)),
+                         static_cast<unsigned>(nb)),
+                    dim3(256), stream, static_cast<OutT*>(args.C), partials, args.M, args.N, v.block_m, v.block_n,
+                    args.grid_m, args.grid_n, args.group, args.tail_begin, split_k, args.batch_stride_c);
         }
     }
     return 0;
@@ -1011,13 +1061,15 @@ int run_by_type(int type_idx, const launch_plan* forced, void* C, void* A, void*
 
 // The same, for callers that take a status code instead of an exception (the entry points
 // that return int): a problem beyond the library's size limits, or a kernel that is not
-// there, becomes ROCM_WMMA_GEMM_ERR_LIMIT, and a launch that the runtime rejected
-// ROCM_WMMA_GEMM_ERR_RUNTIME.
+// there, becomes ROCM_WMMA_GEMM_ERR_LIMIT, and a launch of this call that the runtime rejected
+// ROCM_WMMA_GEMM_ERR_RUNTIME (an error that somebody else's earlier call left pending in the
+// runtime does not count, and stays pending for its owner).
 int run_with_status(int type_idx, const launch_plan* forced, void* C, void* A, void* B, size_t M,
                     size_t N, size_t K, size_t batch, int lc, int la, int lb, hipStream_t stream,
                     const fixed_scratch* fixed)
 {
     int rc;
+    launch_failure = hipSuccess; // what this call's own launches return is collected here
     try
     {
         rc = run_by_type(type_idx, forced, C, A, B, M, N, K, batch, lc, la, lb, stream, fixed);
@@ -1026,7 +1078,7 @@ int run_with_status(int type_idx, const launch_plan* forced, void* C, void* A, v
     {
         return ROCM_WMMA_GEMM_ERR_LIMIT;
     }
-    if(rc == 0 && hipPeekAtLastError() != hipSuccess)
+    if(rc == 0 && launch_failure != hipSuccess)
     {
         rc = ROCM_WMMA_GEMM_ERR_RUNTIME;
     }
@@ -1273,9 +1325,25 @@ int rocm_wmma_gemm_register_variant(int block_m, int block_n, int block_k, int w
 {
     using namespace rocm_wmma_gemm::host;
     if(block_m <= 0 || block_n <= 0 || block_k <= 0 || warps_m <= 0 || warps_n <= 0 || pipeline < 0
-       || pipeline > 7 || block_m % (32 * warps_m) != 0 || block_n % (32 * warps_n) != 0
-       || 64 * warps_m * warps_n > 1024 || type_idx < 0 || type_idx >= num_types || kernels == nullptr
-       || ((a_kmajor | b_kmajor) & ~1) || ring_bytes(block_m, block_n, block_k, pipeline) > 160 * 1024)
+       || pipeline > 7 || 64 * warps_m * warps_n > 1024 || type_idx < 0 || type_idx >= num_types
+       || kernels == nullptr || ((a_kmajor | b_kmajor) & ~1)
+       || ring_bytes(block_m, block_n, block_k, pipeline) > 160 * 1024)
+    {
+        return ROCM_WMMA_GEMM_ERR_ARGUMENT;
+    }
+    if(pipeline == 7)
+    {
+        // the streaming kernel's own tiles: sides of 16, 32 or 64, stages of 128, the wave
+        // grid spelling the tile in 32-row units (1 for a 16-wide side)
+        auto side_ok = [](int side, int waves) {
+            return (side == 16 && waves == 1) || ((side == 32 || side == 64) && side == 32 * waves);
+        };
+        if(block_k != 128 || block_m + block_n < 48 || !side_ok(block_m, warps_m) || !side_ok(block_n, warps_n))
+        {
+            return ROCM_WMMA_GEMM_ERR_ARGUMENT;
+        }
+    }
+    else if(block_m % (32 * warps_m) != 0 || block_n % (32 * warps_n) != 0)
     {
         return ROCM_WMMA_GEMM_ERR_ARGUMENT;
     }
@@ -1333,15 +1401,22 @@ int rocm_wmma_gemm_workspace_release(void)
         return ROCM_WMMA_GEMM_ERR_RUNTIME;
     }
     std::lock_guard<std::mutex> lock(workspace_mutex);
-    if(workspace_ptr[dev] == nullptr)
-    {
-        return 0;
-    }
-    if(workspace_lent_to_capture[dev])
+    if(workspace_ptr[dev] != nullptr && workspace_lent_to_capture[dev])
     {
         return 1; // a captured graph may hold its address
     }
     (void)hipDeviceSynchronize();
+    // (nothing of the library is in flight now) the arrival counters of shared tiles go back
+    // to zero as well, whatever an aborted kernel may have left in them
+    if(unsigned int* counters = arrivals_of_current_device(false))
+    {
+        (void)hipMemset(counters, 0, stream_arrival_slots * sizeof(unsigned int));
+        (void)hipMemset(arrivals_of_current_device(true), 0, stream_arrival_slots * sizeof(unsigned int));
+    }
+    if(workspace_ptr[dev] == nullptr)
+    {
+        return 0;
+    }
     (void)hipFree(workspace_ptr[dev]);
     workspace_ptr[dev]  = nullptr;
     workspace_size[dev] = 0;

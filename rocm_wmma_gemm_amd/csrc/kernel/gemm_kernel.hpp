@@ -87,8 +87,11 @@ struct gemm_args
                             // the XCD's L2 a tile time before the loads that need it; the
                             // workgroups that share an operand panel touch different quarters
     unsigned int* arrivals; // whole-K streaming kernel with k_slices > 1 only: one counter per
-                            // tile and batch entry, zero before the launch and zero again after
-                            // it; partials then holds [batch][tile][slice][BM][BN]
+                            // tile and batch entry; partials then holds
+                            // [batch][tile][slice][BM][BN]
+    unsigned int  arrival_epoch; // this launch's tag in those counters (24 bits, not zero): a
+                                 // counter holds (epoch << 8 | arrivals) and counts from zero
+                                 // for a workgroup that finds another epoch in it
 };
 
 // What one workgroup works on.  blockIdx.x enumerates the whole tiles first, then

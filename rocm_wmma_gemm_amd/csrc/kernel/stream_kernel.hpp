@@ -550,8 +550,20 @@ struct stream_gemm
         __shared__ unsigned int arrived_before;
         if(threadIdx.x == 0)
         {
-            arrived_before = __hip_atomic_fetch_add(args.arrivals + tile_lin, 1u, __ATOMIC_RELAXED,
-                                                    __HIP_MEMORY_SCOPE_AGENT);
+            // the counter holds (epoch << 8 | arrivals); a count under another launch's epoch
+            // (something a killed kernel left behind) starts from zero
+            unsigned int seen = __hip_atomic_load(args.arrivals + tile_lin, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for(;;)
+            {
+                const unsigned int count = (seen >> 8) == args.arrival_epoch ? (seen & 255u) : 0u;
+                if(__hip_atomic_compare_exchange_strong(args.arrivals + tile_lin, &seen,
+                                                        (args.arrival_epoch << 8) | (count + 1u), __ATOMIC_RELAXED,
+                                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+                {
+                    arrived_before = count;
+                    break;
+                }
+            }
         }
         __syncthreads();
         if(arrived_before != (unsigned int)(args.k_slices - 1))
@@ -585,7 +597,9 @@ struct stream_gemm
         }
         if(threadIdx.x == 0)
         {
-            __hip_atomic_store(args.arrivals + tile_lin, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // back to zero arrivals, for a replay of this launch (same epoch)
+            __hip_atomic_store(args.arrivals + tile_lin, args.arrival_epoch << 8, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 };

@@ -691,6 +691,57 @@ def test_what_lies_past_k_does_not_reach_c(loader):
     check_against_oracle(gpu[:M * N], A[:M * K], B[:K * N], M, N, K, 0, 1, 0, din, dout)
 
 
+def test_what_lies_past_k_does_not_reach_c_on_the_streaming_kernel(loader):
+    """The same for the whole-K streaming kernel (pipeline 7), which relies on the ends of its
+    buffer descriptors alone: a last stage of 128 that K cuts short must read zeros, whole
+    tiles and tiles shared by two workgroups alike.  K-contiguous operand: the row behind a
+    row starts with infinities (inside the allocation, right where the lanes past K would
+    fetch).  Operand contiguous along M or N: a second batch entry of infinities starts where
+    the k rows past K would be (K = 200, and K = 1001 where no operand is K-contiguous).
+    Ragged M and N on top, so that the rows past the edge of a tile are in play too."""
+    din, dout = TYPE_PAIRS["f16_f16"]
+    inf = np.uint16(0x7C00)
+    stream = [v for v in loader.variants() if v.pipeline == 7]
+    ran = set()
+    for v in stream:
+        for split in (1, 2):
+            # A row-major: row 5 begins with infinities; B column-major or row-major
+            M, N, K = 40, 136, 200
+            for lb in (1, 0):
+                if not built_for(v, 0, 0, lb, K, M, N):
+                    continue
+                A = O.init_matrix(M, K, 0, din, seed=311)
+                B = O.init_matrix(K, N, lb, din, seed=312)
+                A[5 * K:5 * K + 64] = inf
+                gpu = run_gpu(loader, A, B, M, N, K, 0, 0, lb, din, dout, variant=(v.index, 1, split))
+                check_against_oracle(gpu, A, B, M, N, K, 0, 0, lb, din, dout, rows=(0, 5))
+                check_against_oracle(gpu, A, B, M, N, K, 0, 0, lb, din, dout, rows=(6, M))
+                ran.add((v.index, split, 0, lb))
+            # B column-major: column 7 begins with infinities; A column-major
+            if built_for(v, 0, 1, 1, K, M, N):
+                A = O.init_matrix(M, K, 1, din, seed=313)
+                B = O.init_matrix(K, N, 1, din, seed=314)
+                B[7 * K:7 * K + 64] = inf
+                gpu = run_gpu(loader, A, B, M, N, K, 0, 1, 1, din, dout, variant=(v.index, 1, split))
+                g = O.bits_to_f32(gpu, dout).reshape(M, N)
+                cpu = O.bits_to_f32(O.gemm(A, B, M, N, K, 0, 1, 1, din, dout), dout).reshape(M, N)
+                keep = [j for j in range(N) if j != 7]
+                assert np.isfinite(g[:, keep]).all(), (v.index, split)
+                assert np.allclose(g[:, keep], cpu[:, keep], rtol=2e-3, atol=1e-2), (v.index, split)
+                ran.add((v.index, split, 1, 1))
+            # neither operand K-contiguous: the second batch entry, all infinities, lies where
+            # the first entry's k rows past K would be
+            for K2 in (200, 1001):
+                if not built_for(v, 0, 1, 0, K2, M, N):
+                    continue
+                A = np.concatenate([O.init_matrix(M, K2, 1, din, seed=315), np.full(M * K2, inf, np.uint16)])
+                B = np.concatenate([O.init_matrix(K2, N, 0, din, seed=316), np.full(K2 * N, inf, np.uint16)])
+                gpu = run_gpu(loader, A, B, M, N, K2, 0, 1, 0, din, dout, batch=2, variant=(v.index, 1, split))
+                check_against_oracle(gpu[:M * N], A[:M * K2], B[:K2 * N], M, N, K2, 0, 1, 0, din, dout)
+                ran.add((v.index, split, 1, 0, K2))
+    assert len({r[0] for r in ran}) == len(stream), "every streaming tile ran"
+
+
 def test_degenerate_arguments(loader):
     import torch
 
@@ -1010,7 +1061,12 @@ def test_float_bf16_8192_cubed(loader):
 @pytest.mark.parametrize("M,N,K", [(4096, 5120, 5120), (8192, 4096, 2048), (4096, 14336, 4096),
                                    (16, 8192, 8192), (64, 8192, 8192), (128, 8192, 8192)])
 def test_llm_projection_shapes(loader, M, N, K):
-    for (lc, la, lb) in [(0, 0, 1), (1, 0, 0)]:
+    """fp16 in, fp32 out, through the default dispatch (the tuned entries of these shapes) in
+    A row / B column / C row, A column / B row / C row, all row-major, all column-major and
+    A row / B row / C column: the skinny shapes compare the whole of C, the others in bands.
+    With A column-major the 16-, 64- and 128-row shapes run the streaming kernel's
+    transposing reads at N = K = 8192."""
+    for (lc, la, lb) in [(0, 0, 1), (0, 1, 0), (0, 0, 0), (1, 1, 1), (1, 0, 0)]:
         _full_size_case(loader, M, N, K, lc, la, lb, "f32_f16", whole=M <= 128)
 
 

@@ -81,3 +81,84 @@ def test_noalloc_entry_point_rejects_what_its_scratch_array_cannot_hold(loader):
     # and the array still serves the next call
     rc, want, got, _, _ = _both_ways(loader, 64, 8192, 8192, 0, 1, 0, "f32_f16")
     assert rc == RL.OK and torch.equal(got, want)
+
+
+def test_noalloc_and_ordinary_shared_tile_calls_on_two_streams(loader):
+    """Calls whose workgroups share tiles (whole-K streaming kernel, several workgroups per
+    tile) count their arrivals in per-GPU counters.  The ordinary entry points and the one
+    that allocates nothing each have counters of their own, so an ordinary call on one stream
+    and a no-alloc call on another may run at the same time: every result has the bits of
+    the same call run alone."""
+    import torch
+
+    import rocm_wmma_gemm_amd.loader as RL
+
+    M, N, K = 16, 1024, 8192
+    variant, _, split = loader.select(M, N, K, 0, 0, 0, 1)
+    assert loader.variants()[variant].pipeline == 7 and split > 1, (variant, split)
+    A, B = make_inputs(M, N, K, 0, 1, O.F16, seed_a=11, seed_b=12)
+    dA, dB = to_device(A, O.F16), to_device(B, O.F16)
+    want = torch.zeros(M * N, dtype=torch.float16, device="cuda")
+    loader.gemm(want, dA, dB, M, N, K, 0, 0, 1)
+    torch.cuda.synchronize()
+    check_against_oracle(to_host(want, O.F16), A, B, M, N, K, 0, 0, 1, O.F16, O.F16)
+    rounds = 40
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    out1 = [torch.full_like(want, float("nan")) for _ in range(rounds)]
+    out2 = [torch.full_like(want, float("nan")) for _ in range(rounds)]
+    for r in range(rounds):
+        loader.gemm(out1[r], dA, dB, M, N, K, 0, 0, 1, stream=s1)
+        assert loader.gemm_noalloc(out2[r], dA, dB, M, N, K, 0, 0, 1, stream=s2) == RL.OK
+    s1.synchronize()
+    s2.synchronize()
+    for r in range(rounds):
+        assert torch.equal(out1[r], want), ("ordinary", r)
+        assert torch.equal(out2[r], want), ("no-alloc", r)
+
+
+def test_noalloc_entry_point_under_graph_capture_without_a_library_buffer(loader):
+    """What the entry point is for: a caller that cannot allocate.  With the library's own
+    scratch buffer released, a split-K plan, a padded-copy plan and a shared-tile plan are
+    recorded into a HIP graph through the no-alloc entry point (a capture forbids
+    allocation and synchronisation: either would fail the capture), replayed with eager
+    work in between, and compared bit for bit with the eager results; device memory in use
+    does not change across the calls."""
+    import torch
+
+    import rocm_wmma_gemm_amd.loader as RL
+
+    cases = [(128, 4096, 4096, 1, 1, 0, "f16_f16"),      # split-K planes
+             (1025, 1031, 2049, 0, 0, 1, "bf16_bf16"),   # padded copies
+             (16, 1024, 8192, 0, 0, 1, "f16_f16")]       # workgroups that share tiles
+    dev = []
+    for (M, N, K, lc, la, lb, tname) in cases:
+        din, dout = TYPE_PAIRS[tname]
+        A, B = make_inputs(M, N, K, la, lb, din, seed_a=21, seed_b=22)
+        dA, dB = to_device(A, din), to_device(B, din)
+        want = torch.full((M * N,), float("nan"), dtype=torch_dtype(dout), device="cuda")
+        # (eager warm-up of the entry point: the one-time hipGetSymbolAddress per device)
+        assert loader.gemm_noalloc(want, dA, dB, M, N, K, lc, la, lb) == RL.OK
+        dev.append((dA, dB, want, torch.full_like(want, float("nan"))))
+    torch.cuda.synchronize()
+    # (gives the library's own buffer back, unless a graph captured by an earlier test
+    # holds it: either way the calls below must not touch, create or grow it)
+    loader.workspace_release()
+    free_before, _ = torch.cuda.mem_get_info()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for (M, N, K, lc, la, lb, tname), (dA, dB, want, out) in zip(cases, dev):
+            assert loader.gemm_noalloc(out, dA, dB, M, N, K, lc, la, lb) == RL.OK
+    for replay in range(3):
+        for (_, _, _, out) in dev:
+            out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for case, (_, _, want, out) in zip(cases, dev):
+            assert torch.equal(out, want), (replay, case)
+        # eager no-alloc work between the replays
+        M, N, K, lc, la, lb, tname = cases[0]
+        assert loader.gemm_noalloc(dev[0][3], dev[0][0], dev[0][1], M, N, K, lc, la, lb) == RL.OK
+        torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after >= free_before - (8 << 20), (free_before, free_after)  # (the graph's own nodes)
