@@ -193,6 +193,7 @@ def main() -> int:
         "wall_s_timed_region": round(wall_s, 4),
     }
     traffic = load_traffic()
+    stamp_now = R.source_stamp()
     out["roofline"] = {
         "bound": "mfma", "achieved": round(2.0 * M * N * K / avg_launch_s / 1e12, 2),
         "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -200,6 +201,10 @@ def main() -> int:
         "traffic": traffic.get("hbm_bytes_per_launch") if traffic else None,
         "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, recorded in "
                           "profiles/hbm_traffic.json (a counter run cannot share the timed run)",
+        # whether that record was measured on the sources this library is built from
+        "traffic_stamp": {"recorded_on": traffic.get("source_stamp") if traffic else None,
+                          "this_tree": stamp_now,
+                          "matches": bool(traffic) and traffic.get("source_stamp") == stamp_now},
         "kernel": "256x256x64 direct-to-LDS MFMA GEMM kernel solo_gemm (one wave per SIMD, 16x16x32 "
                   "MFMA), the tuned choice for this shape in all 8 layouts; one launch = one GEMM = "
                   "2*M*N*K FLOP",

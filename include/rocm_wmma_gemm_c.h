@@ -108,7 +108,15 @@ int rocm_wmma_gemm_select_batched(size_t M, size_t N, size_t K, size_t batch_cou
  * that share an operand panel touching different quarters), so that those lines are on
  * their way into the XCD's L2 a tile time before the loads that need them; it pays for a
  * long K whose operands outgrow the memory-side cache and costs a few percent elsewhere,
- * so the tuner decides.  0 = off; other kernels ignore it. */
+ * so the tuner decides.  0 = off; other kernels ignore it.  The value carries a second small
+ * field in bits 4-7: c > 0 = the persistent kernel walks the K tiles of a tile in runs of
+ * 2^(c-1) and, within every 8 runs, the workgroups of XCD x start at run x and wrap round,
+ * so that the XCDs that share an operand panel are never on the same run (each finds in the
+ * memory-side cache what another fetched first, instead of all of them waiting for memory at
+ * once); the sums of an element are added in that order, the same in every call.  Worth
+ * 7-10 % on operands beyond that cache with a K-contiguous operand, nothing elsewhere; the
+ * dispatcher's estimate sets runs of 8 there, the tuner decides per entry.  (JSON keys:
+ * "touch_ahead" for bits 0-3, "k_runs" for the run length.) */
 int rocm_wmma_gemm_select_ex(size_t M, size_t N, size_t K, size_t batch_count, int type_idx, int layout_c,
                              int layout_a, int layout_b, int* swizzle, int* split_k, int* touch_ahead);
 
@@ -121,8 +129,8 @@ int rocm_wmma_gemm_run_variant(int type_idx, int variant, int swizzle, int split
                                size_t batch_count, int layout_c, int layout_a, int layout_b,
                                void* stream);
 
-/* rocm_wmma_gemm_run_variant with the plan's touch_ahead field forced too (see
- * rocm_wmma_gemm_select_ex). */
+/* rocm_wmma_gemm_run_variant with the plan's touch_ahead field (both parts of it) forced too
+ * (see rocm_wmma_gemm_select_ex). */
 int rocm_wmma_gemm_run_variant_ex(int type_idx, int variant, int swizzle, int split_k, int touch_ahead,
                                   void* C, void* A, void* B, size_t M, size_t N, size_t K,
                                   size_t batch_count, int layout_c, int layout_a, int layout_b,
@@ -130,8 +138,9 @@ int rocm_wmma_gemm_run_variant_ex(int type_idx, int variant, int swizzle, int sp
 
 /* Adds a tile variant that was compiled outside this library (the tuner builds
  * rocm_wmma_gemm_amd/csrc/kernel_jit.hip for one tuple, type pair and pair of operand layouts
- * and passes that library's rwg_jit_kernels here: entry points for the three load modes,
- * 16-byte unguarded, 16-byte guarded, 2-byte; null where the pipeline has none).  The
+ * and passes that library's rwg_jit_kernels here: five entry points, for the three load modes,
+ * 16-byte unguarded, 16-byte guarded, 2-byte, then the twins of the first two that walk K in
+ * runs (see rocm_wmma_gemm_select_ex); null where the pipeline or tile has none).  The
  * variant gets the next index after the compiled ones and runs through
  * rocm_wmma_gemm_run_variant like any other; registering the same tuple again for another
  * type pair or layout pair adds those kernels to the same index.  operand *_kmajor: 1 if K is

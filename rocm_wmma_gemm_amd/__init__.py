@@ -15,7 +15,8 @@ from .loader import (  # noqa: F401
     library_path,
     m_layout,
     row_major,
+    source_stamp,
 )
 
 __all__ = ["Loader", "GemmLibraryError", "VariantInfo", "m_layout", "row_major", "col_major",
-           "library_path", "build_library"]
+           "library_path", "build_library", "source_stamp"]

@@ -70,8 +70,18 @@ def load_entries(path: str, type_group: int, variants: list[dict]) -> list[tuple
         rows.append((int(r["M"]), int(r["N"]), int(r["K"]), type_group,
                      LAYOUT_CODE[lay["A"]], LAYOUT_CODE[lay["B"]], LAYOUT_CODE[lay["C"]],
                      variant_of(cfg, variants), int(cfg.get("swizzle", 4)),
-                     split_field(cfg), int(cfg.get("touch_ahead", 0))))
+                     split_field(cfg), touch_field(cfg)))
     return rows
+
+
+def touch_field(cfg: dict) -> int:
+    """The plan's fourth field: bits 0-3 the distance of the line touches ("touch_ahead"),
+    bits 4-7 the code of the K run length ("k_runs": 0 = K tiles in order, else a power of two
+    up to 16, coded as log2 + 1)."""
+    run = int(cfg.get("k_runs", 0))
+    if run < 0 or run > 16 or (run & (run - 1)):
+        raise ValueError(f"k_runs must be 0 or a power of two up to 16, not {run}")
+    return (int(cfg.get("touch_ahead", 0)) & 15) | (run.bit_length() << 4)
 
 
 def split_field(cfg: dict) -> int:

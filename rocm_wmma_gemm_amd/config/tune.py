@@ -122,7 +122,9 @@ GENES = {
     "waves": [(1, 2), (2, 1), (1, 4), (4, 1), (2, 2), (2, 4), (4, 2)],
     "swizzle": [1, 4, 8, 16, -4, -8],
     "split": [1, 2, 4, 8, 16, 32, -1, -2, -3, -4, -6, -8],
-    "touch": [0, 1],
+    # the plan's fourth field: line touches one K tile ahead (1), K tiles in runs of 8 with the
+    # XCDs out of step (64 = code 4 in bits 4-7), both (65)
+    "touch": [0, 1, 64, 65],
 }
 GENE_ORDER = list(GENES)
 
@@ -145,8 +147,8 @@ def tile_feasible(t: Tile, a_kmajor: bool, b_kmajor: bool) -> bool:
     if t.pipeline == 7:
         # whole-K streaming kernel: small tiles (at most one side 16 wide), stages of 128,
         # either layout of an operand
-        return (t.block_k == 128 and t.block_m in (16, 32, 64) and t.block_n in (16, 32, 64)
-                and t.block_m + t.block_n >= 48
+        return (t.block_k == 128 and t.block_m in (16, 32, 64, 128) and t.block_n in (16, 32, 64, 128)
+                and 48 <= t.block_m + t.block_n <= 192
                 and (t.warps_m, t.warps_n) == (max(1, t.block_m // 32), max(1, t.block_n // 32)))
     if t.block_m % (32 * t.warps_m) or t.block_n % (32 * t.warps_n):
         return False
@@ -216,6 +218,11 @@ def touch_feasible(t: Tile, touch: int, K: int) -> bool:
     return touch == 0 or (t.pipeline == 5 and K >= 8192)
 
 
+def k_run_of(touch: int) -> int:
+    code = (touch >> 4) & 15
+    return 0 if code == 0 else 1 << (code - 1)
+
+
 def decode(genes: tuple) -> tuple:
     """(tile, swizzle, split, touch) of a gene tuple."""
     g = dict(zip(GENE_ORDER, genes))
@@ -239,7 +246,7 @@ def tuple_of(cfg: dict):
              cfg.get("block_k", 64), cfg["warps_m"], cfg["warps_n"], cfg.get("pipeline", 0))
     split = -1 if cfg.get("stream_k") else (-cfg["tail_split"] if cfg.get("tail_split", 0) > 1
                                             else cfg.get("split_k", 1))
-    return t, cfg.get("swizzle", 4), split, cfg.get("touch_ahead", 0)
+    return t, cfg.get("swizzle", 4), split, (cfg.get("touch_ahead", 0) & 15) | (int(cfg.get("k_runs", 0)).bit_length() << 4)
 
 
 def config_json(t, swizzle: int, split_k: int, touch: int = 0) -> dict:
@@ -252,8 +259,10 @@ def config_json(t, swizzle: int, split_k: int, touch: int = 0) -> dict:
         cfg["tail_split"] = -split_k
     if split_k == -1:
         cfg["stream_k"] = 1
-    if touch > 0:
-        cfg["touch_ahead"] = touch
+    if touch & 15:
+        cfg["touch_ahead"] = touch & 15
+    if k_run_of(touch):
+        cfg["k_runs"] = k_run_of(touch)
     return cfg
 
 

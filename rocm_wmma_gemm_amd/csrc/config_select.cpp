@@ -267,7 +267,12 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
                 out->variant = i;
                 out->swizzle = 4;
                 out->split_k = split;
-                out->touch   = 0;
+                // operands that outgrow the 256 MB memory-side cache, one of them K-contiguous:
+                // the XCDs of the persistent kernel walk K out of step (runs of 8 K tiles)
+                out->touch = v.pipeline == 5 && (a_kmajor || b_kmajor) && kt >= 64
+                                     && (rows + cols) * k * 2 * batch >= (size_t{256} << 20)
+                                 ? plan_touch_field(0, 8)
+                                 : 0;
             }
         };
         // whole tiles
@@ -377,6 +382,10 @@ bool stream_plan(size_t rows, size_t cols, size_t k, bool a_kmajor, bool b_kmajo
             continue;
         }
         const size_t bm = v.block_m, bn = v.block_n;
+        if(bm > 64 || bn > 64)
+        {
+            continue; // the tiles with a 128-wide side are the tuner's to pick: no constants fitted
+        }
         // an operand that is not K-contiguous: k rows of 16-byte pieces; on a 32-wide side of
         // the tile (k rows of 64 bytes, half a cache line a request) only while it is skinny
         // and stays in L2 (1024 x 1024 x 4096 with A column-major: 28.4 us on the 32 x 64

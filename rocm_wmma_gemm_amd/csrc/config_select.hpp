@@ -28,9 +28,31 @@ struct launch_plan
     int swizzle; // band height of the tile map: s > 0 bands of s tile rows, s < 0 bands of -s tile columns
     int split_k; // K slices (1 = off); -s (s > 1) = split only the last, partial wave of tiles s
                  // ways; -1 = persistent kernel walks by K tile (equal K tiles per workgroup)
-    int touch = 0; // persistent kernel: d > 0 = touch the cache lines of the K tile d tiles past
-                   // the one being loaded (see gemm_args::warm_ahead); 0 = off
+    int touch = 0; // persistent kernel, two small fields.  Bits 0-3: d > 0 = touch the cache lines of
+                   // the K tile d tiles past the one being loaded (see gemm_args::warm_ahead); 0 = off.
+                   // Bits 4-7: c > 0 = walk the K tiles in runs of 2^(c-1), the XCDs out of step by
+                   // whole runs (see gemm_args::k_block); 0 = in order.
 };
+
+// the two fields of launch_plan::touch
+constexpr int plan_touch_distance(int touch)
+{
+    return touch & 15;
+}
+constexpr int plan_k_run(int touch)
+{
+    return ((touch >> 4) & 15) == 0 ? 0 : 1 << (((touch >> 4) & 15) - 1);
+}
+// run: 0 or a power of two up to 16
+constexpr int plan_touch_field(int distance, int run)
+{
+    int code = 0;
+    for(int r = run; r > 0; r >>= 1)
+    {
+        ++code;
+    }
+    return (distance & 15) | (code << 4);
+}
 
 struct tuned_entry
 {

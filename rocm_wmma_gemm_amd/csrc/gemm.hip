@@ -488,9 +488,9 @@ bool streaming_ok(const kernel_problem& p, const variant_desc& v)
     {
         return false;
     }
-    // byte offsets inside a tile: 64 rows of K elements, or K rows of the operand's width
-    const unsigned long long span_a = p.a_kmajor ? 64ull * p.K * 2 : 1ull * p.K * p.M * 2;
-    const unsigned long long span_b = p.b_kmajor ? 64ull * p.K * 2 : 1ull * p.K * p.N * 2;
+    // byte offsets inside a tile: its rows of K elements, or K rows of the operand's width
+    const unsigned long long span_a = p.a_kmajor ? 1ull * v.block_m * p.K * 2 : 1ull * p.K * p.M * 2;
+    const unsigned long long span_b = p.b_kmajor ? 1ull * v.block_n * p.K * 2 : 1ull * p.K * p.N * 2;
     return span_a < (1ull << 31) && span_b < (1ull << 31);
 }
 
@@ -895,6 +895,21 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         // reference kernel_launcher.hpp:119-125 throws the same way
         throw std::runtime_error("No kernel available for the requested configuration and layout");
     }
+    // a plan that walks K in runs takes the kernel's twin built for that, where there is one
+    int k_run = v.pipeline == 5 ? plan_k_run(plan.touch) : 0;
+    if(k_run > 0)
+    {
+        kernel_fn twin = mode < k_runs_twin - 1 ? lookup_kernel(type_idx, p.a_kmajor, p.b_kmajor, plan.variant, mode + k_runs_twin)
+                                                : nullptr;
+        if(twin != nullptr)
+        {
+            fn = twin;
+        }
+        else
+        {
+            k_run = 0;
+        }
+    }
 
     for(size_t b0 = 0; b0 < p.batch; b0 += batches_per_launch)
     {
@@ -921,7 +936,9 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         args.batches          = static_cast<int>(nb);
         args.stream_units     = static_cast<int>(stream_units);
         args.k_tail           = k_tail;
-        args.warm_ahead       = persistent && plan.touch > 0 ? std::min(plan.touch, 3) : 0;
+        args.warm_ahead       = persistent ? std::min(plan_touch_distance(plan.touch), 3) : 0;
+        args.k_block          = k_run;
+
 
         args.batch_by_xcd     = (persistent || v.pipeline == 6) && nb > 1 && split_k == 1 && stream_groups == 0
                                         && blocks_per_batch * nb < (size_t{1} << 31)
@@ -1314,7 +1331,7 @@ int rocm_wmma_gemm_run_variant_ex(int type_idx, int variant, int swizzle, int sp
     plan.variant = variant;
     plan.swizzle = swizzle;
     plan.split_k = split_k;
-    plan.touch   = touch_ahead < 0 ? 0 : touch_ahead;
+    plan.touch   = touch_ahead < 0 ? 0 : touch_ahead & 0xff;
     return run_with_status(type_idx, &plan, C, A, B, M, N, K, batch_count, layout_c, layout_a,
                            layout_b, stream_of(stream), nullptr);
 }
@@ -1333,12 +1350,13 @@ int rocm_wmma_gemm_register_variant(int block_m, int block_n, int block_k, int w
     }
     if(pipeline == 7)
     {
-        // the streaming kernel's own tiles: sides of 16, 32 or 64, stages of 128, the wave
-        // grid spelling the tile in 32-row units (1 for a 16-wide side)
+        // the streaming kernel's own tiles: sides of 16, 32, 64 or 128 (at most 192 together),
+        // stages of 128, the wave grid spelling the tile in 32-row units (1 for a 16-wide side)
         auto side_ok = [](int side, int waves) {
-            return (side == 16 && waves == 1) || ((side == 32 || side == 64) && side == 32 * waves);
+            return (side == 16 && waves == 1) || ((side == 32 || side == 64 || side == 128) && side == 32 * waves);
         };
-        if(block_k != 128 || block_m + block_n < 48 || !side_ok(block_m, warps_m) || !side_ok(block_n, warps_n))
+        if(block_k != 128 || block_m + block_n < 48 || block_m + block_n > 192 || !side_ok(block_m, warps_m)
+           || !side_ok(block_n, warps_n))
         {
             return ROCM_WMMA_GEMM_ERR_ARGUMENT;
         }

@@ -92,6 +92,10 @@ struct gemm_args
     unsigned int  arrival_epoch; // this launch's tag in those counters (24 bits, not zero): a
                                  // counter holds (epoch << 8 | arrivals) and counts from zero
                                  // for a workgroup that finds another epoch in it
+    int           k_block; // persistent kernel built with K_RUNS only.  b > 0 (a power of two): the K
+                           // tiles of an item are walked in runs of b, and within every 8 runs the
+                           // workgroups of XCD x take run x first and wrap round (solo_gemm::run
+                           // says why); 0: in order
 };
 
 // What one workgroup works on.  blockIdx.x enumerates the whole tiles first, then

@@ -92,7 +92,8 @@ template<in_kind IN,
          int  WAVES_M,
          int  WAVES_N,
          int  STAGES,
-         bool GUARD_C = false>
+         bool GUARD_C = false,
+         bool K_RUNS  = false>
 struct solo_gemm
 {
     using InT = typename std::conditional<IN == in_kind::f16, _Float16, __bf16>::type;
@@ -831,6 +832,46 @@ struct solo_gemm
         int        stream_left = cur.nk;
         int        stream_next = cur.next;
         bool       stream_ends = cur.ends_k;
+        // The order of an item's K tiles in the kernels built with K_RUNS (args.k_block = b, a
+        // power of two): runs of b tiles; within every 8 runs the workgroups of XCD x take
+        // run x first, then x + 1, ... and wrap round.
+        // Workgroups that all walk K in step make every XCD that needs a panel ask for the
+        // same lines at the same moment, so every L2 miss waits for HBM (a fabric read took
+        // 850 cycles against 620 for a kernel whose XCDs are not in step, and with operands
+        // beyond the 256 MB memory-side cache that wait is what bounds the K loop: each CU
+        // has only so many lines in flight).  Out of step by whole runs, each XCD is the first
+        // to ask memory for a share of the runs of a panel and finds the others in the
+        // memory-side cache, fetched by the XCD that was there first; and unlike a constant
+        // offset between XCDs, which leaves one XCD first everywhere and as slow as before,
+        // the roles change with every run.  The workgroups of ONE XCD still walk in step:
+        // they share panels through its L2.  4096 x 4096 x 28672 bf16 with both operands
+        // K-contiguous 1235 -> 1365 TFLOP/s, 8192 x 8192 x 28672 1250 -> 1340; nothing
+        // gained where the operands fit that cache, and the bookkeeping costs 1..2 % there,
+        // hence a kernel of its own.  An operand that is contiguous along M or N never had
+        // the problem (a k row of a tile is four whole lines).
+        const int  perm_xcd    = (int)(blockIdx.x & 7);
+        const int  perm_span   = K_RUNS ? 8 * args.k_block : 0; // K tiles of 8 runs (0: in order)
+        const int  perm_shift  = K_RUNS && args.k_block > 0 ? 31 - __builtin_clz((unsigned int)args.k_block) : 0;
+        int        stream_t    = 0; // place in the walk
+        int        stream_k    = 0; // K tile there
+        int        stream_nk   = cur.nk;
+        const InT* a_item      = cur.a;
+        const InT* b_item      = cur.b;
+        auto k_of = [&](int t, int nk) {
+            // (the last runs that do not fill a group of 8 are walked as they are)
+            if(perm_span == 0 || t >= (nk & ~(perm_span - 1)))
+            {
+                return t;
+            }
+            const int r = t & (perm_span - 1), run = r >> perm_shift, off = r & (args.k_block - 1);
+            return (t - r) + ((((run + perm_xcd) & 7) << perm_shift) | off);
+        };
+        if constexpr(K_RUNS)
+        {
+            stream_k = k_of(0, stream_nk);
+            a_src += stream_k * a_step;
+            b_src += stream_k * b_step;
+        }
         // Line touches (args.warm_ahead = distance in K tiles, + 4 for "every workgroup touches
         // whole tiles"): which quarter of a K tile's lines this workgroup touches.  The
         // workgroups that share an A panel differ in their tile column, those that share a B
@@ -857,6 +898,11 @@ struct solo_gemm
         auto advance = [&]() {
             a_src += a_step;
             b_src += b_step;
+            if constexpr(K_RUNS)
+            {
+                ++stream_t;
+                ++stream_k;
+            }
             if(--stream_left == 0)
             {
                 const work_item nx = decode(args, wk, stream_next < wk.end ? stream_next : wk.begin);
@@ -868,10 +914,31 @@ struct solo_gemm
                 stream_next        = nx.next;
                 stream_ends        = nx.ends_k;
                 stream_quarters    = quarters_of(nx);
+                if constexpr(K_RUNS)
+                {
+                    a_item    = nx.a;
+                    b_item    = nx.b;
+                    stream_nk = nx.nk;
+                    stream_t  = 0;
+                    stream_k  = 0;
+                }
+            }
+            if constexpr(K_RUNS)
+            {
+                if(perm_span != 0 && (stream_t & (args.k_block - 1)) == 0)
+                {
+                    // the first tile of a run: wherever the order puts it
+                    stream_k = k_of(stream_t, stream_nk);
+                    a_src    = a_item + stream_k * a_step;
+                    b_src    = b_item + stream_k * b_step;
+                }
             }
         };
-        // whether the tile at (a_src, b_src) is a last K tile held only in part
-        auto partial_tile = [&]() { return k_ragged && stream_ends && stream_left == 1; };
+        // whether the tile at (a_src, b_src) is a last K tile held only in part (the item's
+        // last tile in K order, wherever the walk has it)
+        auto partial_tile = [&]() {
+            return k_ragged && stream_ends && (K_RUNS ? stream_k == stream_nk - 1 : stream_left == 1);
+        };
 
         const unsigned int lds_addr   = (unsigned int)(size_t)lds;
         const unsigned int wave_block = lds_addr + wave * 1024; // this wave's block 0, stage 0
@@ -1027,7 +1094,9 @@ struct solo_gemm
                 step<1, plan_a>(c0, fa[0], fb[0], fa[1], fb[1], acc);
                 __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
                 __builtin_amdgcn_s_barrier();
-                if(warm_dist != 0 && stream_left > warm_dist)
+                // (and of the same run, where the K tiles are walked in runs)
+                if(warm_dist != 0 && stream_left > warm_dist
+                   && (perm_span == 0 || (stream_t & (args.k_block - 1)) + warm_dist < args.k_block))
                 {
                     // a K tile further down the stream than the one whose loads follow, if it
                     // is the same item's

@@ -105,8 +105,10 @@ struct stream_gemm
     static constexpr int LOADS_B = BN / 16;
     static constexpr int PER     = LOADS_A + LOADS_B;
     static constexpr int MAX_SLICES = 8; // workgroups that may share a tile (args.k_slices)
-    static_assert((BM == 16 || BM == 32 || BM == 64) && (BN == 16 || BN == 32 || BN == 64) && BM + BN >= 48,
-                  "tiles of 16, 32 or 64 rows and columns");
+    static_assert((BM == 16 || BM == 32 || BM == 64 || BM == 128) && (BN == 16 || BN == 32 || BN == 64 || BN == 128)
+                      && BM + BN >= 48 && BM + BN <= 192,
+                  "tiles of 16, 32, 64 or 128 rows and columns, three stages of which fit the LDS");
+    static_assert(LDS_BYTES <= 160 * 1024, "the ring must fit the 160 KB LDS");
     static_assert(DEPTH >= 3 && (DEPTH - 1) * PER < 64, "ring depth against the 6-bit vmcnt");
     static_assert(WAVES * BM * BN * 4 <= LDS_BYTES, "the partial tiles of the waves reuse the ring");
 
@@ -146,10 +148,12 @@ struct stream_gemm
     // k rows, and the next 16 lanes the same 8 rows further on: W = 64, rows 128 bytes apart,
     // rows k and k + 2 and the rows 8 further all start on the same bank; W = 32, rows k and
     // k + 4 do (the 4 rows of a group do not meet), and the rows 8 further.
+    // W = 128, rows 256 bytes apart: the 4 rows of a group all start on the same bank, so
+    // each goes to another 32-byte place (k mod 4), and the rows 8 further on 128 bytes off.
     template<int W>
     __device__ __forceinline__ static int mn_piece(int k)
     {
-        return W == 64 ? ((k & 3) ^ ((k >> 3) & 1)) : ((k >> 3) & 1);
+        return W == 128 ? ((k & 3) ^ (((k >> 3) & 1) << 2)) : W == 64 ? ((k & 3) ^ ((k >> 3) & 1)) : ((k >> 3) & 1);
     }
 
     // W = 16: k rows of 32 bytes, 32 of them per 1 KiB load.  The 4 rows that 16 lanes of a
@@ -216,6 +220,35 @@ struct stream_gemm
         f[1] = u32x4{l1.x, l1.y, h1.x, h1.y};
         f[2] = u32x4{l2.x, l2.y, h2.x, h2.y};
         f[3] = u32x4{l3.x, l3.y, h3.x, h3.y};
+    }
+
+    // a 128-wide side: rows of 256 bytes, eight column pieces, the 4 rows further on 1024
+    // bytes later (two statements of four pieces: sixteen results in one would hold 32
+    // registers early-clobbered at once)
+    __device__ __forceinline__ static void transposed(unsigned int addr, u32x4 (&f)[8])
+    {
+#pragma unroll
+        for(int h = 0; h < 2; ++h)
+        {
+            const unsigned int a0 = addr ^ (128u * h), a1 = a0 ^ 32u, a2 = a0 ^ 64u, a3 = a0 ^ 96u;
+            uint2              l0, h0, l1, h1, l2, h2, l3, h3;
+            asm volatile("ds_read_b64_tr_b16 %0, %8\n\t"
+                         "ds_read_b64_tr_b16 %1, %8 offset:1024\n\t"
+                         "ds_read_b64_tr_b16 %2, %9\n\t"
+                         "ds_read_b64_tr_b16 %3, %9 offset:1024\n\t"
+                         "ds_read_b64_tr_b16 %4, %10\n\t"
+                         "ds_read_b64_tr_b16 %5, %10 offset:1024\n\t"
+                         "ds_read_b64_tr_b16 %6, %11\n\t"
+                         "ds_read_b64_tr_b16 %7, %11 offset:1024\n\t"
+                         "s_waitcnt lgkmcnt(0)"
+                         : "=&v"(l0), "=&v"(h0), "=&v"(l1), "=&v"(h1), "=&v"(l2), "=&v"(h2), "=&v"(l3), "=&v"(h3)
+                         : "v"(a0), "v"(a1), "v"(a2), "v"(a3)
+                         : "memory");
+            f[4 * h + 0] = u32x4{l0.x, l0.y, h0.x, h0.y};
+            f[4 * h + 1] = u32x4{l1.x, l1.y, h1.x, h1.y};
+            f[4 * h + 2] = u32x4{l2.x, l2.y, h2.x, h2.y};
+            f[4 * h + 3] = u32x4{l3.x, l3.y, h3.x, h3.y};
+        }
     }
 
     // a 32-wide side: rows of 64 bytes, two column pieces

@@ -16,7 +16,9 @@ namespace host
 #define RWG_VARIANT(IDX, BM, BN, BK, WM, WN, PIPE)                              \
     {entry<BM, BN, BK, WM, WN, PIPE, device::load_mode::vec_unguarded>(),       \
      entry<BM, BN, BK, WM, WN, PIPE, device::load_mode::vec_guarded>(),         \
-     entry<BM, BN, BK, WM, WN, PIPE, device::load_mode::scalar>()},
+     entry<BM, BN, BK, WM, WN, PIPE, device::load_mode::scalar>(),             \
+     entry<BM, BN, BK, WM, WN, PIPE, device::load_mode::vec_unguarded, true>(), \
+     entry<BM, BN, BK, WM, WN, PIPE, device::load_mode::vec_guarded, true>()},
 
 const kernel_fn RWG_CAT(kernel_slice_, RWG_TYPE, RWG_AK, RWG_BK)[num_variants][num_modes] = {
 #include "variants.def"

@@ -34,7 +34,11 @@ constexpr int num_variants = 0
 #undef RWG_VARIANT
 
 constexpr int num_types = 4; // f16_f16, f32_f16, bf16_bf16, f32_bf16
-constexpr int num_modes = 3; // device::load_mode
+constexpr int num_load_modes = 3; // device::load_mode
+// kernels per variant: one per load mode, then the twins of the 16-byte unguarded and guarded
+// kernels that walk K in runs (persistent 256 x 256 x 64 kernel only; nullptr elsewhere)
+constexpr int num_modes     = 5;
+constexpr int k_runs_twin   = 3; // mode m < 2 has its twin at m + k_runs_twin
 
 using kernel_fn = void (*)(const device::gemm_args);
 

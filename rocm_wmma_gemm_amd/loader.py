@@ -82,6 +82,26 @@ def build_library(jobs: int = 8, force: bool = False) -> str:
     return os.path.join(_DEFAULT_LIB_DIR, "librocm_wmma_gemm_gfx950.so")
 
 
+def source_stamp() -> str:
+    """Sixteen hex digits over everything a kernel launch of the library depends on: the
+    kernel and host sources under csrc/ (the generated table left out) and the tuned
+    tables.  A counter summary under profiles/ records the stamp of the tree it was measured
+    on, so that a reader (and bench.py) can tell whether it still describes this library."""
+    import glob
+    import hashlib
+
+    files = []
+    for pattern in ("csrc/*.hip", "csrc/*.hpp", "csrc/*.cpp", "csrc/*.def", "csrc/kernel/*.hpp",
+                    "config/gemm_config_gfx950_*.json", "config/model_gfx950.json"):
+        files += glob.glob(os.path.join(_HERE, pattern))
+    h = hashlib.sha256()
+    for path in sorted(f for f in files if not f.endswith("config_generated.hpp")):
+        h.update(os.path.relpath(path, _HERE).encode())
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def detect_arch() -> str:
     import torch
 

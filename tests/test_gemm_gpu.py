@@ -376,7 +376,8 @@ def test_whole_k_streaming_kernel_agrees_with_oracle(loader):
 
     stream = [v for v in loader.variants() if v.pipeline == 7]
     assert {(v.block_m, v.block_n) for v in stream} == {(32, 32), (64, 32), (32, 64), (64, 64),
-                                                       (16, 32), (16, 64), (32, 16), (64, 16)}
+                                                       (16, 32), (16, 64), (32, 16), (64, 16),
+                                                       (128, 64), (64, 128), (128, 32), (32, 128)}
     # (K = 200, 1000 and 1352: a last stage that K cuts short; 1001 where no operand is K-contiguous)
     shapes = [(16, 2048, 1024), (100, 1000, 384), (128, 512, 128), (33, 65, 2048), (2048, 24, 512),
               (40, 520, 200), (1000, 1000, 1000), (64, 128, 1352)]
@@ -402,7 +403,8 @@ def test_whole_k_streaming_kernel_agrees_with_oracle(loader):
                     except AssertionError as e:
                         raise AssertionError(f"variant {v.index} {M}x{N}x{K} C{lc} A{la} B{lb} {tname}: {e}") from None
     # every tile ran with every pair of operand layouts
-    every = {(32, 32), (64, 32), (32, 64), (64, 64), (16, 32), (16, 64), (32, 16), (64, 16)}
+    every = {(32, 32), (64, 32), (32, 64), (64, 64), (16, 32), (16, 64), (32, 16), (64, 16),
+             (128, 64), (64, 128), (128, 32), (32, 128)}
     for pair in ((0, 1), (0, 0), (1, 1), (1, 0)):
         assert {(bm, bn) for (bm, bn, lc, la, lb) in ran if (la, lb) == pair} == every, pair
     # a strided batch, and bit-identical repeats
@@ -624,6 +626,62 @@ def test_batch_entries_dealt_by_xcd_agree_with_oracle(loader):
                 except AssertionError as e:
                     raise AssertionError(f"variant {v.index} {M}x{N}x{K} batch {b}/{batch} "
                                          f"layouts C{lc} A{la} B{lb} {tname}: {e}") from None
+
+
+def test_k_tiles_walked_in_runs_out_of_step_between_xcds(loader):
+    """The plan's K-run field on the persistent kernel: the K tiles of a tile are walked in runs
+    of 1 to 16, and within every 8 runs the workgroups of XCD x start at run x.  Against the
+    oracle on K that is whole groups of runs, K with runs left over (walked in order), a
+    partial last K tile, ragged M and N, several items per workgroup, batch entries, every
+    tile split along K, the split tail wave, the walk by K tile, and line touches on top;
+    three runs compared bit for bit (an element's sum has one order, whoever computes it)."""
+    solo = [v for v in loader.variants() if v.pipeline == 5 and v.block_k == 64]
+    assert solo
+    v256 = next(v for v in solo if (v.block_m, v.block_n) == (256, 256))
+    field = lambda run, touch=0: touch | (run.bit_length() << 4)  # noqa: E731
+    cases = [  # M, N, K, batch, split field, run length, touch distance, variant
+        (512, 512, 2048, 1, 1, 1, 0, v256),      # 32 K tiles: 4 groups of 8 runs of 1
+        (512, 768, 4096, 1, 1, 4, 0, v256),      # 64 K tiles: 2 groups of runs of 4
+        (256, 512, 8192 + 192, 1, 1, 8, 0, v256),  # 131 K tiles: 2 groups of runs of 8 and 3 tiles in order
+        (300, 520, 4096 + 40, 1, 1, 2, 0, v256),  # ragged M, N and a partial last K tile
+        (2304, 2304, 1024, 1, 1, 2, 0, v256),    # 81 tiles: workgroups with two items
+        (256, 256, 1088, 5, 1, 1, 0, v256),      # batch entries, 17 K tiles
+        (512, 512, 8192, 1, 2, 4, 0, v256),      # every tile in two K slices of 64 tiles
+        (4352, 256, 2048, 1, -2, 2, 0, v256),    # the tail wave split in two
+        (768, 512, 4096, 1, -1, 4, 0, v256),     # walk by K tile: ranges cut anywhere
+        (512, 512, 16384, 1, 1, 8, 1, v256),     # with line touches inside the runs
+        (512, 512, 4096, 1, 1, 16, 0, v256),     # 64 K tiles are less than a group of runs of 16: in order
+    ] + [(384, 576, 2048 + 64, 1, 1, 2, 0, v) for v in solo if v is not v256]
+    for n, (M, N, K, batch, split, run, touch, v) in enumerate(cases):
+        tname = "f16_f16" if n % 2 == 0 else "f32_bf16"
+        din, dout = TYPE_PAIRS[tname]
+        for (lc, la, lb) in [l for l in [(0, 0, 1), (1, 1, 0), (0, 0, 0), (1, 1, 1)] if built_for(v, *l)]:
+            import torch
+
+            A = np.concatenate([O.init_matrix(M, K, la, din, seed=330 + b) for b in range(batch)])
+            B = np.concatenate([O.init_matrix(K, N, lb, din, seed=360 + b) for b in range(batch)])
+            dA, dB = to_device(A, din), to_device(B, din)
+            outs = []
+            for _ in range(3):
+                dC = torch.full((M * N * batch,), float("nan"), dtype=torch_dtype(dout), device="cuda")
+                rc = loader.run_variant(v.index, 4, split, dC, dA, dB, M, N, K, lc, la, lb, batch_count=batch,
+                                        touch_ahead=field(run, touch))
+                assert rc == 0, (rc, M, N, K, split, run)
+                outs.append(dC)
+            torch.cuda.synchronize()
+            gpu = to_host(outs[0], dout)
+            for b in range(batch):
+                try:
+                    check_against_oracle(gpu[b * M * N:(b + 1) * M * N], A[b * M * K:(b + 1) * M * K],
+                                         B[b * K * N:(b + 1) * K * N], M, N, K, lc, la, lb, din, dout)
+                except AssertionError as e:
+                    raise AssertionError(f"variant {v.index} {M}x{N}x{K} batch {b}/{batch} split {split} runs of "
+                                         f"{run} touch {touch} layouts C{lc} A{la} B{lb} {tname}: {e}") from None
+            assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2]), (M, N, K, split, run)
+    # the dispatcher's estimate asks for runs where the operands outgrow the memory-side cache
+    variant, _, _, touch = loader.select_ex(8192, 8192, 20480, 2, 0, 0, 1)
+    assert loader.variants()[variant].pipeline == 5 and (touch >> 4) == 4, (variant, touch)
+    assert loader.select_ex(4096, 4096, 3072, 2, 0, 0, 1)[3] >> 4 == 0
 
 
 def test_partial_last_k_tile_on_the_persistent_kernel(loader):

@@ -299,6 +299,21 @@ def test_shipped_json_matches_reference_schema():
         assert {"warps_m", "warps_n", "warp_tile_m", "warp_tile_n", "swizzle", "bits"} <= set(conf["config"])
 
 
+def test_every_shipped_entry_says_which_type_pair_it_was_timed_on():
+    """The reference's tuner writes an entry only from a timing of that entry (reference
+    rocm_wmma_gemm/config/tune.py:692-770, 905-913).  Here a table serves two type pairs, so
+    every entry records the pair it was timed on, and that pair is one the table serves."""
+    import json
+
+    cfg_dir = os.path.join(ROOT, "rocm_wmma_gemm_amd", "config")
+    for name, served in (("f16", ("f16_f16", "bf16_bf16")), ("f32", ("f32_f16", "f32_bf16"))):
+        doc = json.load(open(os.path.join(cfg_dir, f"gemm_config_gfx950_{name}.json")))
+        missing = [(c["range"], c["layout"]) for c in doc["configurations"] if "timed_on" not in c]
+        assert not missing, f"{len(missing)} entries of the {name} table without timed_on, e.g. {missing[0]}"
+        wrong = [c for c in doc["configurations"] if c["timed_on"] not in served]
+        assert not wrong, f"{name} table: entry timed on {wrong[0]['timed_on']}"
+
+
 def _mfma_loops(asm_text):
     """(function, [lines]) for every loop (label .. backward branch to it) that holds an MFMA."""
     out = []
