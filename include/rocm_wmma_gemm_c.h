@@ -114,9 +114,14 @@ int rocm_wmma_gemm_select_batched(size_t M, size_t N, size_t K, size_t batch_cou
  * so that the XCDs that share an operand panel are never on the same run (each finds in the
  * memory-side cache what another fetched first, instead of all of them waiting for memory at
  * once); the sums of an element are added in that order, the same in every call.  Worth
- * 7-10 % on operands beyond that cache with a K-contiguous operand, nothing elsewhere; the
- * dispatcher's estimate sets runs of 8 there, the tuner decides per entry.  (JSON keys:
- * "touch_ahead" for bits 0-3, "k_runs" for the run length.) */
+ * 7-10 % on operands beyond that cache with a K-contiguous operand, nothing elsewhere.  And a
+ * third in bits 8-9: c > 0 = within every aligned group of 2^c K tiles the workgroup of tile
+ * (i, j) starts at tile (i + j) mod 2^c of the group and wraps round, so that the workgroups
+ * of an XCD that share an operand panel ask for a line at different times and all but the
+ * first find it in L2: worth 14-17 % on the same problems; the dispatcher's estimate sets
+ * groups of 4 there, the tuner decides per entry.  Both leave the sums of an element in one
+ * fixed order, the same in every call.  (JSON keys: "touch_ahead" for bits 0-3, "k_runs" for
+ * the run length, "k_group" for the group size.) */
 int rocm_wmma_gemm_select_ex(size_t M, size_t N, size_t K, size_t batch_count, int type_idx, int layout_c,
                              int layout_a, int layout_b, int* swizzle, int* split_k, int* touch_ahead);
 

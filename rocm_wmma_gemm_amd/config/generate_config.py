@@ -77,11 +77,15 @@ def load_entries(path: str, type_group: int, variants: list[dict]) -> list[tuple
 def touch_field(cfg: dict) -> int:
     """The plan's fourth field: bits 0-3 the distance of the line touches ("touch_ahead"),
     bits 4-7 the code of the K run length ("k_runs": 0 = K tiles in order, else a power of two
-    up to 16, coded as log2 + 1)."""
+    up to 16, coded as log2 + 1), bits 8-9 the code of the K group ("k_group": 0, 2, 4 or 8,
+    coded as log2)."""
     run = int(cfg.get("k_runs", 0))
     if run < 0 or run > 16 or (run & (run - 1)):
         raise ValueError(f"k_runs must be 0 or a power of two up to 16, not {run}")
-    return (int(cfg.get("touch_ahead", 0)) & 15) | (run.bit_length() << 4)
+    group = int(cfg.get("k_group", 0))
+    if group not in (0, 2, 4, 8):
+        raise ValueError(f"k_group must be 0, 2, 4 or 8, not {group}")
+    return (int(cfg.get("touch_ahead", 0)) & 15) | (run.bit_length() << 4) | ((group.bit_length() - 1 if group else 0) << 8)
 
 
 def split_field(cfg: dict) -> int:

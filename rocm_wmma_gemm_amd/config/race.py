@@ -170,7 +170,7 @@ def gpu_timer(type_name: str, reps: int, warmup: int):
             cache["B"] = (torch.rand(K * N, device="cuda") * 2 - 1).to(in_dtype)
             cache["C"] = torch.empty(M * N, dtype=c_dtype, device="cuda")
         return time_candidate(L, torch, v.index, int(cfg.get("swizzle", 1)), hook_split(cfg),
-                              (int(cfg.get("touch_ahead", 0)) & 15) | (int(cfg.get("k_runs", 0)).bit_length() << 4), cache["C"], cache["A"], cache["B"], M, N, K,
+                              (int(cfg.get("touch_ahead", 0)) & 15) | (int(cfg.get("k_runs", 0)).bit_length() << 4) | ((int(cfg.get("k_group", 0)).bit_length() - 1 if cfg.get("k_group", 0) else 0) << 8), cache["C"], cache["A"], cache["B"], M, N, K,
                               LAYOUT_CODE[lc], LAYOUT_CODE[la], LAYOUT_CODE[lb], reps, warmup)
 
     return timer

@@ -123,8 +123,9 @@ GENES = {
     "swizzle": [1, 4, 8, 16, -4, -8],
     "split": [1, 2, 4, 8, 16, 32, -1, -2, -3, -4, -6, -8],
     # the plan's fourth field: line touches one K tile ahead (1), K tiles in runs of 8 with the
-    # XCDs out of step (64 = code 4 in bits 4-7), both (65)
-    "touch": [0, 1, 64, 65],
+    # XCDs out of step (64 = code 4 in bits 4-7), workgroups that start each group of 4 or 8
+    # K tiles at different tiles (0x200, 0x300 = codes 2, 3 in bits 8-9)
+    "touch": [0, 1, 64, 0x200, 0x300],
 }
 GENE_ORDER = list(GENES)
 
@@ -223,6 +224,17 @@ def k_run_of(touch: int) -> int:
     return 0 if code == 0 else 1 << (code - 1)
 
 
+def k_group_of(touch: int) -> int:
+    code = (touch >> 8) & 3
+    return 0 if code == 0 else 1 << code
+
+
+def touch_field_of(cfg: dict) -> int:
+    group = int(cfg.get("k_group", 0))
+    return ((cfg.get("touch_ahead", 0) & 15) | (int(cfg.get("k_runs", 0)).bit_length() << 4)
+            | ((group.bit_length() - 1 if group else 0) << 8))
+
+
 def decode(genes: tuple) -> tuple:
     """(tile, swizzle, split, touch) of a gene tuple."""
     g = dict(zip(GENE_ORDER, genes))
@@ -246,7 +258,7 @@ def tuple_of(cfg: dict):
              cfg.get("block_k", 64), cfg["warps_m"], cfg["warps_n"], cfg.get("pipeline", 0))
     split = -1 if cfg.get("stream_k") else (-cfg["tail_split"] if cfg.get("tail_split", 0) > 1
                                             else cfg.get("split_k", 1))
-    return t, cfg.get("swizzle", 4), split, (cfg.get("touch_ahead", 0) & 15) | (int(cfg.get("k_runs", 0)).bit_length() << 4)
+    return t, cfg.get("swizzle", 4), split, touch_field_of(cfg)
 
 
 def config_json(t, swizzle: int, split_k: int, touch: int = 0) -> dict:
@@ -263,6 +275,8 @@ def config_json(t, swizzle: int, split_k: int, touch: int = 0) -> dict:
         cfg["touch_ahead"] = touch & 15
     if k_run_of(touch):
         cfg["k_runs"] = k_run_of(touch)
+    if k_group_of(touch):
+        cfg["k_group"] = k_group_of(touch)
     return cfg
 
 

@@ -267,11 +267,13 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
                 out->variant = i;
                 out->swizzle = 4;
                 out->split_k = split;
-                // operands that outgrow the 256 MB memory-side cache, one of them K-contiguous:
-                // the XCDs of the persistent kernel walk K out of step (runs of 8 K tiles)
-                out->touch = v.pipeline == 5 && (a_kmajor || b_kmajor) && kt >= 64
-                                     && (rows + cols) * k * 2 * batch >= (size_t{256} << 20)
-                                 ? plan_touch_field(0, 8)
+                // operands that outgrow the 256 MB memory-side cache and are K-contiguous (both, or
+                // one of them with a K of 20480 and more: 8192 x 8192 x 16384 with B row-major loses
+                // 2 % to it, x 28672 gains 5 %): the workgroups of the persistent kernel start each
+                // group of 4 K tiles at different tiles
+                out->touch = v.pipeline == 5 && (rows + cols) * k * 2 * batch >= (size_t{256} << 20)
+                                     && ((a_kmajor && b_kmajor && kt >= 64) || ((a_kmajor || b_kmajor) && kt >= 320))
+                                 ? plan_touch_field(0, 0, 4)
                                  : 0;
             }
         };

@@ -32,6 +32,8 @@ struct launch_plan
                    // the K tile d tiles past the one being loaded (see gemm_args::warm_ahead); 0 = off.
                    // Bits 4-7: c > 0 = walk the K tiles in runs of 2^(c-1), the XCDs out of step by
                    // whole runs (see gemm_args::k_block); 0 = in order.
+                   // Bits 8-9: c > 0 = within groups of 2^c K tiles the workgroups start at different
+                   // tiles (see gemm_args::k_group); 0 = in order.
 };
 
 // the two fields of launch_plan::touch
@@ -43,15 +45,19 @@ constexpr int plan_k_run(int touch)
 {
     return ((touch >> 4) & 15) == 0 ? 0 : 1 << (((touch >> 4) & 15) - 1);
 }
-// run: 0 or a power of two up to 16
-constexpr int plan_touch_field(int distance, int run)
+constexpr int plan_k_group(int touch)
+{
+    return ((touch >> 8) & 3) == 0 ? 0 : 1 << ((touch >> 8) & 3);
+}
+// run: 0 or a power of two up to 16; group: 0, 2, 4 or 8
+constexpr int plan_touch_field(int distance, int run, int group = 0)
 {
     int code = 0;
     for(int r = run; r > 0; r >>= 1)
     {
         ++code;
     }
-    return (distance & 15) | (code << 4);
+    return (distance & 15) | (code << 4) | ((group == 2 ? 1 : group == 4 ? 2 : group == 8 ? 3 : 0) << 8);
 }
 
 struct tuned_entry

@@ -897,7 +897,8 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
     }
     // a plan that walks K in runs takes the kernel's twin built for that, where there is one
     int k_run = v.pipeline == 5 ? plan_k_run(plan.touch) : 0;
-    if(k_run > 0)
+    int k_group = v.pipeline == 5 ? plan_k_group(plan.touch) : 0;
+    if(k_run > 0 || k_group > 0)
     {
         kernel_fn twin = mode < k_runs_twin - 1 ? lookup_kernel(type_idx, p.a_kmajor, p.b_kmajor, plan.variant, mode + k_runs_twin)
                                                 : nullptr;
@@ -907,7 +908,8 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         }
         else
         {
-            k_run = 0;
+            k_run   = 0;
+            k_group = 0;
         }
     }
 
@@ -938,6 +940,7 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         args.k_tail           = k_tail;
         args.warm_ahead       = persistent ? std::min(plan_touch_distance(plan.touch), 3) : 0;
         args.k_block          = k_run;
+        args.k_group          = k_group;
 
 
         args.batch_by_xcd     = (persistent || v.pipeline == 6) && nb > 1 && split_k == 1 && stream_groups == 0
@@ -1331,7 +1334,7 @@ int rocm_wmma_gemm_run_variant_ex(int type_idx, int variant, int swizzle, int sp
     plan.variant = variant;
     plan.swizzle = swizzle;
     plan.split_k = split_k;
-    plan.touch   = touch_ahead < 0 ? 0 : touch_ahead & 0xff;
+    plan.touch   = touch_ahead < 0 ? 0 : touch_ahead & 0x3ff;
     return run_with_status(type_idx, &plan, C, A, B, M, N, K, batch_count, layout_c, layout_a,
                            layout_b, stream_of(stream), nullptr);
 }

@@ -96,6 +96,10 @@ struct gemm_args
                            // tiles of an item are walked in runs of b, and within every 8 runs the
                            // workgroups of XCD x take run x first and wrap round (solo_gemm::run
                            // says why); 0: in order
+    int           k_group; // the same kernels.  g = 2, 4 or 8: within every aligned group of g K tiles
+                           // the workgroup of tile (i, j) starts at tile (i + j) mod g of the group and
+                           // wraps round, so that the workgroups of an XCD that share a panel ask for
+                           // a line at different times and all but the first find it in L2; 0: in order
 };
 
 // What one workgroup works on.  blockIdx.x enumerates the whole tiles first, then

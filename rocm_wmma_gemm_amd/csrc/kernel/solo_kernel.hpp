@@ -601,6 +601,7 @@ struct solo_gemm
         int        batch;
         int        row0, col0;
         int        nk; // K tiles, at least one
+        int        cls; // tile row + tile column: which K tile of a group the item starts at (args.k_group)
         const InT* a; // first K tile of the operands
         const InT* b;
         const InT* a_end; // where the loads' range ends (see limits)
@@ -709,6 +710,7 @@ struct solo_gemm
         x.b = scalar_pointer(static_cast<const InT*>(args.B) + x.batch * args.batch_stride_b
                              + x.col0 * b_sr + (long long)step_begin * BK * b_sk);
         x.ends_k = step_begin + x.nk == k_steps_total;
+        x.cls    = __builtin_amdgcn_readfirstlane(x.row0 / BM + x.col0 / BN);
         limits(args, x);
         return x;
     }
@@ -849,6 +851,18 @@ struct solo_gemm
         // gained where the operands fit that cache, and the bookkeeping costs 1..2 % there,
         // hence a kernel of its own.  An operand that is contiguous along M or N never had
         // the problem (a k row of a tile is four whole lines).
+        // The same one level down (args.k_group = g): within every aligned group of g K tiles
+        // the workgroup of tile (i, j) starts at tile (i + j) mod g and wraps round.  The 8
+        // workgroups of an XCD that share an A panel (a tile row) and the 4 that share a B
+        // panel (a tile column) then ask for a line at g different times: the first waits for
+        // the fabric, the others find the line in L2 instead of queueing behind the same
+        // miss, and a compute unit's lines in flight turn over that much faster (the XCD's
+        // L2 holds the g K tiles of its 12 panels: 1.5 MB of 4 at g = 4).  By tile row or by
+        // tile column alone it is worth half as much, and a constant offset (every row a K
+        // tile further on, all the way) nothing: whoever is ahead stays ahead and as slow
+        // as before.  4096 x 4096 x 28672 bf16, both operands K-contiguous: 1245 -> 1460
+        // TFLOP/s with g = 4 (1365 with the runs by XCD alone, 1425 with both; the vendor
+        // kernel of the same tile 1560), 8192 x 8192 x 28672 1250 -> 1430.
         const int  perm_xcd    = (int)(blockIdx.x & 7);
         const int  perm_span   = K_RUNS ? 8 * args.k_block : 0; // K tiles of 8 runs (0: in order)
         const int  perm_shift  = K_RUNS && args.k_block > 0 ? 31 - __builtin_clz((unsigned int)args.k_block) : 0;
@@ -857,7 +871,13 @@ struct solo_gemm
         int        stream_nk   = cur.nk;
         const InT* a_item      = cur.a;
         const InT* b_item      = cur.b;
+        int stream_cls = cur.cls;
         auto k_of = [&](int t, int nk) {
+            // (the last tiles that do not fill a group are walked as they are)
+            if(args.k_group > 0 && t < (nk & ~(args.k_group - 1)))
+            {
+                t = (t & ~(args.k_group - 1)) | ((t + stream_cls) & (args.k_group - 1));
+            }
             // (the last runs that do not fill a group of 8 are walked as they are)
             if(perm_span == 0 || t >= (nk & ~(perm_span - 1)))
             {
@@ -919,13 +939,14 @@ struct solo_gemm
                     a_item    = nx.a;
                     b_item    = nx.b;
                     stream_nk = nx.nk;
-                    stream_t  = 0;
-                    stream_k  = 0;
+                    stream_t   = 0;
+                    stream_k   = 0;
+                    stream_cls = nx.cls;
                 }
             }
             if constexpr(K_RUNS)
             {
-                if(perm_span != 0 && (stream_t & (args.k_block - 1)) == 0)
+                if((perm_span != 0 && (stream_t & (args.k_block - 1)) == 0) || args.k_group > 0)
                 {
                     // the first tile of a run: wherever the order puts it
                     stream_k = k_of(stream_t, stream_nk);
@@ -1096,7 +1117,8 @@ struct solo_gemm
                 __builtin_amdgcn_s_barrier();
                 // (and of the same run, where the K tiles are walked in runs)
                 if(warm_dist != 0 && stream_left > warm_dist
-                   && (perm_span == 0 || (stream_t & (args.k_block - 1)) + warm_dist < args.k_block))
+                   && (perm_span == 0 || (stream_t & (args.k_block - 1)) + warm_dist < args.k_block)
+                   && args.k_group == 0)
                 {
                     // a K tile further down the stream than the one whose loads follow, if it
                     // is the same item's

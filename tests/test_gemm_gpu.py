@@ -629,8 +629,9 @@ def test_batch_entries_dealt_by_xcd_agree_with_oracle(loader):
 
 
 def test_k_tiles_walked_in_runs_out_of_step_between_xcds(loader):
-    """The plan's K-run field on the persistent kernel: the K tiles of a tile are walked in runs
-    of 1 to 16, and within every 8 runs the workgroups of XCD x start at run x.  Against the
+    """The plan's K-order fields on the persistent kernel: the K tiles of a tile are walked in runs
+    of 1 to 16, and within every 8 runs the workgroups of XCD x start at run x; within groups of
+    2, 4 or 8 K tiles the workgroup of tile (i, j) starts at tile (i + j) of the group.  Against the
     oracle on K that is whole groups of runs, K with runs left over (walked in order), a
     partial last K tile, ragged M and N, several items per workgroup, batch entries, every
     tile split along K, the split tail wave, the walk by K tile, and line touches on top;
@@ -638,8 +639,15 @@ def test_k_tiles_walked_in_runs_out_of_step_between_xcds(loader):
     solo = [v for v in loader.variants() if v.pipeline == 5 and v.block_k == 64]
     assert solo
     v256 = next(v for v in solo if (v.block_m, v.block_n) == (256, 256))
-    field = lambda run, touch=0: touch | (run.bit_length() << 4)  # noqa: E731
-    cases = [  # M, N, K, batch, split field, run length, touch distance, variant
+    field = lambda run, touch=0: (touch & 15) | (run.bit_length() << 4) | (touch & 0x300)  # noqa: E731
+    cases = [  # M, N, K, batch, split field, run length, touch distance (+ K group code << 8), variant
+        (512, 768, 4096 + 64, 1, 1, 0, 0x200, v256),   # groups of 4 K tiles, one tile left over
+        (768, 512, 2048, 1, 1, 0, 0x300, v256),        # groups of 8
+        (300, 520, 1024 + 40, 1, 1, 0, 0x100, v256),   # groups of 2, ragged M, N and a partial last K tile
+        (2304, 2304, 1024, 1, 1, 0, 0x200, v256),      # workgroups with two items
+        (256, 256, 1088, 3, 2, 0, 0x200, v256),        # batch entries, two K slices of 9 and 8 tiles
+        (768, 512, 4096, 1, -1, 0, 0x200, v256),       # walk by K tile
+        (512, 512, 8192, 1, 1, 8, 0x200, v256),        # groups inside runs
         (512, 512, 2048, 1, 1, 1, 0, v256),      # 32 K tiles: 4 groups of 8 runs of 1
         (512, 768, 4096, 1, 1, 4, 0, v256),      # 64 K tiles: 2 groups of runs of 4
         (256, 512, 8192 + 192, 1, 1, 8, 0, v256),  # 131 K tiles: 2 groups of runs of 8 and 3 tiles in order
@@ -680,8 +688,9 @@ def test_k_tiles_walked_in_runs_out_of_step_between_xcds(loader):
             assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2]), (M, N, K, split, run)
     # the dispatcher's estimate asks for runs where the operands outgrow the memory-side cache
     variant, _, _, touch = loader.select_ex(8192, 8192, 20480, 2, 0, 0, 1)
-    assert loader.variants()[variant].pipeline == 5 and (touch >> 4) == 4, (variant, touch)
+    assert loader.variants()[variant].pipeline == 5 and (touch >> 8) == 2, (variant, touch)
     assert loader.select_ex(4096, 4096, 3072, 2, 0, 0, 1)[3] >> 4 == 0
+    assert loader.select_ex(8192, 8192, 16384, 2, 0, 0, 0)[3] >> 4 == 0  # B row-major: not before K = 20480
 
 
 def test_partial_last_k_tile_on_the_persistent_kernel(loader):
