@@ -270,10 +270,11 @@ bool model_plan(size_t m, size_t n, size_t k, int lc, int la, int lb, launch_pla
                 // operands that outgrow the 256 MB memory-side cache and are K-contiguous (both, or
                 // one of them with a K of 20480 and more: 8192 x 8192 x 16384 with B row-major loses
                 // 2 % to it, x 28672 gains 5 %): the workgroups of the persistent kernel start each
-                // group of 4 K tiles at different tiles
-                out->touch = v.pipeline == 5 && (rows + cols) * k * 2 * batch >= (size_t{256} << 20)
+                // group of 8 K tiles at different tiles.  (At 268 MB, 4096 x 4096 x 16384 and
+                // 8192^3, the plain walk is level or 3 % ahead; at 335 MB the groups gain 17 %.)
+                out->touch = v.pipeline == 5 && (rows + cols) * k * 2 * batch >= (size_t{300} << 20)
                                      && ((a_kmajor && b_kmajor && kt >= 64) || ((a_kmajor || b_kmajor) && kt >= 320))
-                                 ? plan_touch_field(0, 0, 4)
+                                 ? plan_touch_field(0, 0, 8)
                                  : 0;
             }
         };

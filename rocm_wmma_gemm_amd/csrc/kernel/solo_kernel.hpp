@@ -343,16 +343,27 @@ struct solo_gemm
     };
     using no_loads = load_plan<0, 1, 0, 0>;
 
+    // Scalar work of the caller's that wants a place among the MFMAs of a step: called
+    // behind every MFMA with its number as a type.
+    struct no_hook
+    {
+        template<class M>
+        __device__ __forceinline__ void operator()(M) const
+        {
+        }
+    };
+
     // MFMA number M of a step and the memory instructions that follow it: fragment
     // M / FRAG_GAP (A fragments first, then B) of K step READ_KK of the tile at c.rd
     // into (na, nb), and the load PLAN puts here, bound for c.fill.
-    template<int M, int READ_KK, class PLAN>
+    template<int M, int READ_KK, class PLAN, class HOOK>
     __device__ __forceinline__ static void slot(const step_ctx& c,
                                                 const u32x4 (&fa)[TM],
                                                 const u32x4 (&fb)[TN],
                                                 u32x4 (&na)[TM],
                                                 u32x4 (&nb)[TN],
-                                                f32x4 (&acc)[TM][TN])
+                                                f32x4 (&acc)[TM][TN],
+                                                const HOOK& hook)
     {
         constexpr bool HAS_LOAD = PLAN::count > 0 && M >= PLAN::first
                                   && (M - PLAN::first) % PLAN::gap == 0
@@ -390,32 +401,35 @@ struct solo_gemm
                 nb[U - TM] = c.ob.template fragment_pinned<U - TM, READ_KK>(c.rd + A_BYTES);
             }
         }
+        hook(std::integral_constant<int, M>{});
     }
 
-    template<int READ_KK, class PLAN, int... M>
+    template<int READ_KK, class PLAN, class HOOK, int... M>
     __device__ __forceinline__ static void slots(std::integer_sequence<int, M...>,
                                                  const step_ctx& c,
                                                  const u32x4 (&fa)[TM],
                                                  const u32x4 (&fb)[TN],
                                                  u32x4 (&na)[TM],
                                                  u32x4 (&nb)[TN],
-                                                 f32x4 (&acc)[TM][TN])
+                                                 f32x4 (&acc)[TM][TN],
+                                                 const HOOK& hook)
     {
-        (slot<M, READ_KK, PLAN>(c, fa, fb, na, nb, acc), ...);
+        (slot<M, READ_KK, PLAN>(c, fa, fb, na, nb, acc, hook), ...);
     }
 
     // One K step: the MFMAs on (fa, fb) with the reads and loads between them.
-    template<int READ_KK, class PLAN>
+    template<int READ_KK, class PLAN, class HOOK = no_hook>
     __device__ __forceinline__ static void step(const step_ctx& c,
                                                 const u32x4 (&fa)[TM],
                                                 const u32x4 (&fb)[TN],
                                                 u32x4 (&na)[TM],
                                                 u32x4 (&nb)[TN],
-                                                f32x4 (&acc)[TM][TN])
+                                                f32x4 (&acc)[TM][TN],
+                                                const HOOK& hook = HOOK{})
     {
         __builtin_amdgcn_sched_barrier(0);
         slots<READ_KK, PLAN>(
-            std::make_integer_sequence<int, MFMAS>{}, c, fa, fb, na, nb, acc);
+            std::make_integer_sequence<int, MFMAS>{}, c, fa, fb, na, nb, acc, hook);
         __builtin_amdgcn_sched_barrier(0);
     }
 
@@ -860,35 +874,42 @@ struct solo_gemm
         // L2 holds the g K tiles of its 12 panels: 1.5 MB of 4 at g = 4).  By tile row or by
         // tile column alone it is worth half as much, and a constant offset (every row a K
         // tile further on, all the way) nothing: whoever is ahead stays ahead and as slow
-        // as before.  4096 x 4096 x 28672 bf16, both operands K-contiguous: 1245 -> 1460
-        // TFLOP/s with g = 4 (1365 with the runs by XCD alone, 1425 with both; the vendor
-        // kernel of the same tile 1560), 8192 x 8192 x 28672 1250 -> 1430.
+        // as before.  4096 x 4096 x 28672 bf16, both operands K-contiguous: 1240 -> 1440
+        // TFLOP/s with g = 4, 1480 with g = 8 (1365 with the runs by XCD alone, 1425 with
+        // runs and groups; the vendor kernel of the same tile 1525), 8192 x 8192 x 28672
+        // 1250 -> 1460 (1530).  Where the operands fit the memory-side cache the plain walk is
+        // level or ahead (8192^3 1590 against 1580, 4096^3 1490 against 1460).
+        // (Written without branches, masks that are zero where an order does not apply, so that
+        // the few scalar instructions sit among the MFMAs instead of in blocks of their own.)
         const int  perm_xcd    = (int)(blockIdx.x & 7);
         const int  perm_span   = K_RUNS ? 8 * args.k_block : 0; // K tiles of 8 runs (0: in order)
         const int  perm_shift  = K_RUNS && args.k_block > 0 ? 31 - __builtin_clz((unsigned int)args.k_block) : 0;
+        const int  span_mask   = perm_span > 0 ? perm_span - 1 : 0;
+        const int  run_mask    = K_RUNS && args.k_block > 0 ? args.k_block - 1 : 0;
+        const int  group_mask  = K_RUNS && args.k_group > 0 ? args.k_group - 1 : 0;
         int        stream_t    = 0; // place in the walk
         int        stream_k    = 0; // K tile there
         int        stream_nk   = cur.nk;
         const InT* a_item      = cur.a;
         const InT* b_item      = cur.b;
-        int stream_cls = cur.cls;
-        auto k_of = [&](int t, int nk) {
-            // (the last tiles that do not fill a group are walked as they are)
-            if(args.k_group > 0 && t < (nk & ~(args.k_group - 1)))
-            {
-                t = (t & ~(args.k_group - 1)) | ((t + stream_cls) & (args.k_group - 1));
-            }
-            // (the last runs that do not fill a group of 8 are walked as they are)
-            if(perm_span == 0 || t >= (nk & ~(perm_span - 1)))
-            {
-                return t;
-            }
-            const int r = t & (perm_span - 1), run = r >> perm_shift, off = r & (args.k_block - 1);
-            return (t - r) + ((((run + perm_xcd) & 7) << perm_shift) | off);
+        int        stream_cls  = cur.cls;
+        const int  runs_apply  = perm_span != 0 ? ~span_mask : 0;
+        // (the last tiles that do not fill a group are walked as they are)
+        auto in_group = [&](int t, int nk, int cls) {
+            const int gm = t < (nk & ~group_mask) ? group_mask : 0;
+            return (t & ~gm) | ((t + cls) & gm);
         };
+        // (the last runs that do not fill a group of 8 are walked as they are; none at all when
+        // there are no runs)
+        auto in_runs = [&](int k, int nk) {
+            const int r  = k & span_mask;
+            const int kr = (k - r) + (((((r >> perm_shift) + perm_xcd) & 7) << perm_shift) | (r & run_mask));
+            return k < (nk & runs_apply) ? kr : k;
+        };
+        auto k_of = [&](int t, int nk, int cls) { return in_runs(in_group(t, nk, cls), nk); };
         if constexpr(K_RUNS)
         {
-            stream_k = k_of(0, stream_nk);
+            stream_k = k_of(0, stream_nk, stream_cls);
             a_src += stream_k * a_step;
             b_src += stream_k * b_step;
         }
@@ -915,13 +936,47 @@ struct solo_gemm
             return (unsigned int)__builtin_amdgcn_readfirstlane(qa | (qb << 8));
         };
         unsigned int stream_quarters = quarters_of(cur);
+        // Where the order puts the tile after the current one, worked out ahead of advance():
+        // in the K loop from among the MFMAs of the second step (the scalar instructions cost
+        // nothing there; behind the last MFMA they are 3..4 % of a tile's time).
+        int        k_next = 0;
+        const InT* a_next = a_src;
+        const InT* b_next = b_src;
+        auto plan_next = [&](auto part) {
+            if constexpr(K_RUNS)
+            {
+                constexpr int PART = decltype(part)::value; // (-1: all of it)
+                if constexpr(PART == 0 || PART == -1)
+                {
+                    k_next = in_group(stream_t + 1, stream_nk, stream_cls);
+                }
+                if constexpr(PART == 1 || PART == -1)
+                {
+                    k_next = in_runs(k_next, stream_nk);
+                }
+                if constexpr(PART == 2 || PART == -1)
+                {
+                    a_next = a_item + k_next * a_step;
+                }
+                if constexpr(PART == 3 || PART == -1)
+                {
+                    b_next = b_item + k_next * b_step;
+                }
+            }
+        };
+        constexpr std::integral_constant<int, -1> whole{};
         auto advance = [&]() {
-            a_src += a_step;
-            b_src += b_step;
             if constexpr(K_RUNS)
             {
                 ++stream_t;
-                ++stream_k;
+                stream_k = k_next;
+                a_src    = a_next;
+                b_src    = b_next;
+            }
+            else
+            {
+                a_src += a_step;
+                b_src += b_step;
             }
             if(--stream_left == 0)
             {
@@ -936,22 +991,14 @@ struct solo_gemm
                 stream_quarters    = quarters_of(nx);
                 if constexpr(K_RUNS)
                 {
-                    a_item    = nx.a;
-                    b_item    = nx.b;
-                    stream_nk = nx.nk;
+                    a_item     = nx.a;
+                    b_item     = nx.b;
+                    stream_nk  = nx.nk;
                     stream_t   = 0;
-                    stream_k   = 0;
                     stream_cls = nx.cls;
-                }
-            }
-            if constexpr(K_RUNS)
-            {
-                if((perm_span != 0 && (stream_t & (args.k_block - 1)) == 0) || args.k_group > 0)
-                {
-                    // the first tile of a run: wherever the order puts it
-                    stream_k = k_of(stream_t, stream_nk);
-                    a_src    = a_item + stream_k * a_step;
-                    b_src    = b_item + stream_k * b_step;
+                    stream_k   = k_of(0, nx.nk, nx.cls);
+                    a_src      = nx.a + stream_k * a_step;
+                    b_src      = nx.b + stream_k * b_step;
                 }
             }
         };
@@ -982,6 +1029,7 @@ struct solo_gemm
                 issue_loads(std::make_integer_sequence<int, VM_LOADS>{}, la.or_else(part, la_tail),
                             lb.or_else(part, lb_tail), wave_block + s * STAGE, descriptor(a_src, a_end),
                             descriptor(b_src, b_end));
+                plan_next(whole);
                 advance();
             }
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(3 * VM_LOADS));
@@ -1004,6 +1052,7 @@ struct solo_gemm
                 __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * VM_LOADS));
                 __builtin_amdgcn_s_barrier();
                 step<0, plan>(c, ca, cb, na, nb, acc);
+                plan_next(whole);
                 advance();
                 here = there;
             };
@@ -1067,6 +1116,7 @@ struct solo_gemm
             issue_loads(std::make_integer_sequence<int, VM_LOADS>{}, la.or_else(part, la_tail),
                         lb.or_else(part, lb_tail), wave_block, descriptor(a_src, a_end), descriptor(b_src, b_end));
         }
+        plan_next(whole);
         advance();
         bool part_prev = partial_tile();
         issue_loads(std::make_integer_sequence<int, LOADS_B>{}, la.or_else(part_prev, la_tail),
@@ -1076,6 +1126,7 @@ struct solo_gemm
         const InT* b_prev     = b_src;
         const InT* a_end_prev = a_end;
         const InT* b_end_prev = b_end;
+        plan_next(whole);
         advance();
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(LOADS_B));
         __builtin_amdgcn_s_barrier();
@@ -1135,7 +1186,14 @@ struct solo_gemm
                                         (stream_quarters >> 8) * (B_KMAJOR ? b_ld * 2 : 128))));
                     }
                 }
-                step<0, plan_b>(c1, fa[1], fb[1], fa[0], fb[0], acc);
+                step<0, plan_b>(c1, fa[1], fb[1], fa[0], fb[0], acc, [&](auto m) {
+                    // (a few scalar instructions behind each of four MFMAs)
+                    constexpr int AT = decltype(m)::value;
+                    if constexpr(AT >= 4 && AT <= 16 && AT % 4 == 0)
+                    {
+                        plan_next(std::integral_constant<int, AT / 4 - 1>{});
+                    }
+                });
                 a_prev     = a_src;
                 b_prev     = b_src;
                 a_end_prev = a_end;

@@ -686,9 +686,10 @@ def test_k_tiles_walked_in_runs_out_of_step_between_xcds(loader):
                     raise AssertionError(f"variant {v.index} {M}x{N}x{K} batch {b}/{batch} split {split} runs of "
                                          f"{run} touch {touch} layouts C{lc} A{la} B{lb} {tname}: {e}") from None
             assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2]), (M, N, K, split, run)
-    # the dispatcher's estimate asks for runs where the operands outgrow the memory-side cache
+    # the dispatcher's estimate asks for groups of 8 where the operands outgrow the memory-side cache
     variant, _, _, touch = loader.select_ex(8192, 8192, 20480, 2, 0, 0, 1)
-    assert loader.variants()[variant].pipeline == 5 and (touch >> 8) == 2, (variant, touch)
+    assert loader.variants()[variant].pipeline == 5 and (touch >> 8) == 3, (variant, touch)
+    assert loader.select_ex(6144, 6144, 10240, 2, 0, 0, 1)[3] >> 4 == 0  # 252 MB: fits
     assert loader.select_ex(4096, 4096, 3072, 2, 0, 0, 1)[3] >> 4 == 0
     assert loader.select_ex(8192, 8192, 16384, 2, 0, 0, 0)[3] >> 4 == 0  # B row-major: not before K = 20480
 
