@@ -311,7 +311,7 @@ def linkage_tree(pop, n_genes):
     return fos
 
 
-def gomea(domains, feasible, evaluate, budget, rng, first_population=8, seeds=(), log=None):
+def gomea(domains, feasible, evaluate, budget, rng, first_population=8, seeds=(), log=None, stats=None):
     """Minimises evaluate(genes) over the product of `domains` (a list of value lists)
     restricted to feasible(genes).  evaluate returns a time, or None for a candidate that
     turned out not to run (failed compile, kernel not built for the layout).  At most
@@ -408,6 +408,35 @@ def gomea(domains, feasible, evaluate, budget, rng, first_population=8, seeds=()
                 else:
                     x, cx = best[0], best[1]
             out.append(x)
+        return diversify(out)
+
+    refills = [0]  # candidates timed only to refill a population (they do not count as progress)
+
+    def diversify(pop):
+        """Forced improvement turns members into copies of the best solution, and a
+        population of copies teaches the next linkage tree nothing.  When fewer than half of
+        the members are distinct, up to a quarter of them (copies only) are replaced by fresh
+        random solutions.  (The reference keeps its populations apart with a niching hall of
+        fame, tune.py:186-240; with 7 genes this is enough.)"""
+        if len(set(pop)) * 2 >= len(pop):
+            return pop
+        seen, out, quota = set(), [], max(1, len(pop) // 4)
+        for x in pop:
+            if x in seen and quota > 0:
+                y = random_solution()
+                if y is not None and y not in seen and y not in pop:
+                    known = y in cache
+                    c = cost(y)
+                    if c is not None:
+                        refills[0] += 0 if known else 1
+                        note(y, c)
+                        if math.isfinite(c):
+                            quota -= 1
+                            seen.add(y)
+                            out.append(y)
+                            continue
+            seen.add(x)
+            out.append(x)
         return out
 
     def polish():
@@ -429,7 +458,7 @@ def gomea(domains, feasible, evaluate, budget, rng, first_population=8, seeds=()
 
     populations, size, tick, stalls = [], first_population, 0, 0
     while len(cache) < budget and stalls < 3:
-        before = len(cache)
+        before = len(cache) - refills[0]
         if not populations or tick % (4 ** len(populations)) == 0 or stalls:
             pop = new_population(size)
             if pop:
@@ -441,10 +470,12 @@ def gomea(domains, feasible, evaluate, budget, rng, first_population=8, seeds=()
         tick += 1
         # a round that timed nothing new: the populations have converged; the next round
         # starts a larger one at once, and three such rounds in a row end the search
-        stalls = stalls + 1 if len(cache) == before else 0
+        stalls = stalls + 1 if len(cache) - refills[0] == before else 0
         if stalls == 1:
             polish()
     polish()
+    if stats is not None:
+        stats["refills"] = refills[0]  # candidates timed to replace copies in a population
     return best[0], best[1], len(cache)
 
 

@@ -494,6 +494,10 @@ bool streaming_ok(const kernel_problem& p, const variant_desc& v)
     return span_a < (1ull << 31) && span_b < (1ull << 31);
 }
 
+// from this size on the streaming kernel reads an operand with the non-temporal hint (the
+// memory-side cache holds 256 MB)
+constexpr size_t stream_once_bytes = size_t{256} << 20;
+
 template<class OutT>
 int launch_streaming(int type_idx, const launch_plan& plan, const kernel_problem& p, hipStream_t stream,
                      const fixed_scratch* fixed)
@@ -569,6 +573,10 @@ int launch_streaming(int type_idx, const launch_plan& plan, const kernel_problem
         args.partials       = reinterpret_cast<float*>(partials);
         args.arrivals       = arrivals;
         args.arrival_epoch  = slices > 1 ? next_arrival_epoch() : 0;
+        // an operand that one row (column) of tiles reads once and that cannot stay in the
+        // memory-side cache for the next call either is loaded with the non-temporal hint
+        args.stream_once    = (grid_m == 1 && p.N * p.K * in_bytes * nb >= stream_once_bytes ? 1 : 0)
+                           | (grid_n == 1 && p.M * p.K * in_bytes * nb >= stream_once_bytes ? 2 : 0);
         args.blocks_per_batch = static_cast<int>(tiles);
         args.batches          = static_cast<int>(nb);
         enqueue(fn, dim3(static_cast<unsigned>(tiles * slices), static_cast<unsigned>(nb)), dim3(v.threads), stream,

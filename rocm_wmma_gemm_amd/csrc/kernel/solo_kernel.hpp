@@ -387,6 +387,12 @@ struct solo_gemm
         }
         else
         {
+#ifdef RWG_SOLO_PROBE_HALF_MFMAS
+            // Timing probe, results WRONG (never defined in a build that ships): the MFMAs
+            // of the lower half of the wave tile that carry no load are left out, to see what
+            // a pass over half a tile would cost with the loads and fragment reads unchanged.
+            if constexpr(M / TN < TM / 2)
+#endif
             mfma_16x16x32_pinned<IN>(acc[M / TN][M % TN], fa[M / TN], fb[M % TN]);
         }
         if constexpr(M % FRAG_GAP == 0 && M / FRAG_GAP < FRAGS)

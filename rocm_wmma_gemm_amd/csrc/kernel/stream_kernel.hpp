@@ -131,15 +131,28 @@ struct stream_gemm
     // One 1 KiB load: lane l's 16 bytes go to lds_block + 16 l.  (The compiler does not
     // look for hazards around inline assembly: four wait states cover M0 and a descriptor
     // or offset that a v_readfirstlane has just written.)
+    // `once`: with the non-temporal hint (gemm_args::stream_once; the same for every lane).
     __device__ __forceinline__ static void load_block(unsigned int lds_block, unsigned int voff, const u32x4& rsrc,
-                                                      unsigned int soff)
+                                                      unsigned int soff, bool once)
     {
-        asm volatile("s_mov_b32 m0, %[ldsb]\n\t"
-                     "s_nop 4\n\t"
-                     "buffer_load_dwordx4 %[voff], %[rsrc], %[soff] offen lds"
-                     :
-                     : [ldsb] "s"(lds_block), [voff] "v"(voff), [rsrc] "s"(rsrc), [soff] "s"(soff)
-                     : "memory");
+        if(once)
+        {
+            asm volatile("s_mov_b32 m0, %[ldsb]\n\t"
+                         "s_nop 4\n\t"
+                         "buffer_load_dwordx4 %[voff], %[rsrc], %[soff] offen nt lds"
+                         :
+                         : [ldsb] "s"(lds_block), [voff] "v"(voff), [rsrc] "s"(rsrc), [soff] "s"(soff)
+                         : "memory");
+        }
+        else
+        {
+            asm volatile("s_mov_b32 m0, %[ldsb]\n\t"
+                         "s_nop 4\n\t"
+                         "buffer_load_dwordx4 %[voff], %[rsrc], %[soff] offen lds"
+                         :
+                         : [ldsb] "s"(lds_block), [voff] "v"(voff), [rsrc] "s"(rsrc), [soff] "s"(soff)
+                         : "memory");
+        }
     }
 
     // M/N-contiguous operand, W elements wide (a k row of 2 W bytes; 512 / W k rows per 1 KiB
@@ -398,6 +411,7 @@ struct stream_gemm
         const int stages_all = (args.K + BK - 1) / BK, stages_per = (stages_all + args.k_slices - 1) / args.k_slices;
         const int first      = slice * stages_per;
         const int stages     = stages_all - first < stages_per ? stages_all - first : stages_per; // >= 1 (host)
+        const bool once_a = (args.stream_once & 2) != 0, once_b = (args.stream_once & 1) != 0;
         auto      issue      = [&](int stage, int slot_index) {
             const unsigned int base = lds_addr + slot_index * STAGE + wave * 1024;
             const bool         last = first + stage == stages_all - 1; // the stage that K may cut short
@@ -406,13 +420,13 @@ struct stream_gemm
             for(int i = 0; i < LOADS_A; ++i)
             {
                 load_block(base + i * 4096, va, rsrc_a,
-                           __builtin_amdgcn_readfirstlane((unsigned int)(first + stage) * stage_a + i * step_a));
+                           __builtin_amdgcn_readfirstlane((unsigned int)(first + stage) * stage_a + i * step_a), once_a);
             }
 #pragma unroll
             for(int i = 0; i < LOADS_B; ++i)
             {
                 load_block(base + A_BYTES + i * 4096, vb, rsrc_b,
-                           __builtin_amdgcn_readfirstlane((unsigned int)(first + stage) * stage_b + i * step_b));
+                           __builtin_amdgcn_readfirstlane((unsigned int)(first + stage) * stage_b + i * step_b), once_b);
             }
         };
         // Where the tile grid is one tile high (a skinny M or N: no two workgroups read the

@@ -1138,6 +1138,31 @@ def test_llm_projection_shapes(loader, M, N, K):
         _full_size_case(loader, M, N, K, lc, la, lb, "f32_f16", whole=M <= 128)
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 28672, 8192), (24, 8192, 28672)])
+def test_a_few_rows_against_weights_beyond_the_memory_side_cache(loader, M, N, K):
+    """470 MB of weights against 16 or 24 rows: the streaming kernel reads an operand of 256 MB
+    and more, which one row (or column) of tiles walks exactly once, with the non-temporal
+    hint.  Every element of C against the oracle, through the default dispatch and with
+    streaming tiles forced (whole tiles and two workgroups per tile), B as the large operand
+    (C row-major) and A (C column-major: the transposed problem)."""
+    stream = {(v.block_m, v.block_n): v.index for v in loader.variants() if v.pipeline == 7}
+    ran = 0
+    for (lc, la, lb) in [(0, 0, 1), (0, 0, 0), (1, 1, 1), (1, 0, 1)]:
+        din, dout = TYPE_PAIRS["f32_f16"]
+        A, B = make_inputs(M, N, K, la, lb, din)
+        check_against_oracle(run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout), A, B, M, N, K, lc, la, lb, din, dout)
+        small_first = lc == 0  # kernel space: rows = M (C row-major) or N (C column-major)
+        for (small, large), split in [((32, 64), 1), ((16, 64), 2), ((32, 32), 1)]:
+            tile = (small, large) if small_first else (large, small)
+            v = loader.variants()[stream[tile]]
+            if not built_for(v, lc, la, lb, K, M, N):
+                continue
+            gpu = run_gpu(loader, A, B, M, N, K, lc, la, lb, din, dout, variant=(v.index, 1, split))
+            check_against_oracle(gpu, A, B, M, N, K, lc, la, lb, din, dout)
+            ran += 1
+    assert ran >= 6, ran
+
+
 @pytest.mark.parametrize("M,N,K", [(256, 4096, 4096), (256, 28672, 8192), (512, 14336, 4096),
                                    (512, 8192, 28672), (1024, 4096, 14336)])
 def test_a_few_hundred_rows_against_projection_weights(loader, M, N, K):

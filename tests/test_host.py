@@ -524,6 +524,15 @@ def test_gomea_finds_the_optimum_of_a_linked_landscape_with_a_fake_timer():
     # the budget is a hard limit and a landscape with nothing feasible ends at once
     best, ms, evals = T.gomea(domains, lambda g: False, fake_ms, budget=50, rng=random.Random(0))
     assert best is None and evals == 0
+    # a population that has collapsed onto copies of the best solution is refilled with fresh
+    # random members (a needle in a flat landscape: every member is soon a copy of the first
+    # one that improved), within the budget, and the needle is found
+    flat = [list(range(6))] * 5
+    stats = {}
+    best, ms, evals = T.gomea(flat, lambda g: True, lambda g: 1.0 if g == (3, 1, 4, 1, 5) else 2.0 + 0.001 * sum(g),
+                              budget=400, rng=random.Random(2), stats=stats)
+    assert evals <= 400 and stats["refills"] > 0, (evals, stats)
+    assert ms <= 2.0
     # a table entry round-trips through the genes
     cfg = T.config_json(T.Tile(256, 256, 64, 2, 2, 5), 8, -4, 1)
     assert cfg["tail_split"] == 4 and cfg["touch_ahead"] == 1
