@@ -131,11 +131,12 @@ struct stream_gemm
     // One 1 KiB load: lane l's 16 bytes go to lds_block + 16 l.  (The compiler does not
     // look for hazards around inline assembly: four wait states cover M0 and a descriptor
     // or offset that a v_readfirstlane has just written.)
-    // `once`: with the non-temporal hint (gemm_args::stream_once; the same for every lane).
+    // ONCE: with the non-temporal hint (gemm_args::stream_once).
+    template<bool ONCE>
     __device__ __forceinline__ static void load_block(unsigned int lds_block, unsigned int voff, const u32x4& rsrc,
-                                                      unsigned int soff, bool once)
+                                                      unsigned int soff)
     {
-        if(once)
+        if constexpr(ONCE)
         {
             asm volatile("s_mov_b32 m0, %[ldsb]\n\t"
                          "s_nop 4\n\t"
@@ -411,22 +412,26 @@ struct stream_gemm
         const int stages_all = (args.K + BK - 1) / BK, stages_per = (stages_all + args.k_slices - 1) / args.k_slices;
         const int first      = slice * stages_per;
         const int stages     = stages_all - first < stages_per ? stages_all - first : stages_per; // >= 1 (host)
-        const bool once_a = (args.stream_once & 2) != 0, once_b = (args.stream_once & 1) != 0;
-        auto      issue      = [&](int stage, int slot_index) {
+        // (the hints are template arguments: the walk over the stages below exists in four
+        // copies, one test per launch picks one; a test per load, two branches each, cost a
+        // third of the time of a 64 x 64 stage)
+        auto issue_as = [&](int stage, int slot_index, auto once_a, auto once_b) {
             const unsigned int base = lds_addr + slot_index * STAGE + wave * 1024;
             const bool         last = first + stage == stages_all - 1; // the stage that K may cut short
             const unsigned int va = last ? voff_a_tail : voff_a, vb = last ? voff_b_tail : voff_b;
 #pragma unroll
             for(int i = 0; i < LOADS_A; ++i)
             {
-                load_block(base + i * 4096, va, rsrc_a,
-                           __builtin_amdgcn_readfirstlane((unsigned int)(first + stage) * stage_a + i * step_a), once_a);
+                load_block<decltype(once_a)::value>(
+                    base + i * 4096, va, rsrc_a,
+                    __builtin_amdgcn_readfirstlane((unsigned int)(first + stage) * stage_a + i * step_a));
             }
 #pragma unroll
             for(int i = 0; i < LOADS_B; ++i)
             {
-                load_block(base + A_BYTES + i * 4096, vb, rsrc_b,
-                           __builtin_amdgcn_readfirstlane((unsigned int)(first + stage) * stage_b + i * step_b), once_b);
+                load_block<decltype(once_b)::value>(
+                    base + A_BYTES + i * 4096, vb, rsrc_b,
+                    __builtin_amdgcn_readfirstlane((unsigned int)(first + stage) * stage_b + i * step_b));
             }
         };
         // Where the tile grid is one tile high (a skinny M or N: no two workgroups read the
@@ -449,11 +454,6 @@ struct stream_gemm
             const int at = (stage < stages ? stage : stages - 1) + turn;
             return at >= stages ? at - stages : at;
         };
-
-        for(int t = 0; t < DEPTH - 1; ++t)
-        {
-            issue(clamped(t), t);
-        }
 
         f32x4 acc[TM][TN];
 #pragma unroll
@@ -478,6 +478,12 @@ struct stream_gemm
         const int tr_off_b = mn_read_offset<BN>(wave, sub, slot);
         using lds_u32x4    = __attribute__((address_space(3))) u32x4;
 
+        auto walk = [&](auto once_a, auto once_b) {
+        auto issue = [&](int stage, int slot) { issue_as(stage, slot, once_a, once_b); };
+        for(int t = 0; t < DEPTH - 1; ++t)
+        {
+            issue(clamped(t), t);
+        }
         int slot_index = 0; // of stage t
         for(int t = 0; t < stages; ++t)
         {
@@ -526,6 +532,24 @@ struct stream_gemm
                 }
             }
             slot_index = slot_index + 1 == DEPTH ? 0 : slot_index + 1;
+        }
+        };
+        const int once = __builtin_amdgcn_readfirstlane(args.stream_once);
+        if(once == 0)
+        {
+            walk(std::false_type{}, std::false_type{});
+        }
+        else if(once == 1)
+        {
+            walk(std::false_type{}, std::true_type{});
+        }
+        else if(once == 2)
+        {
+            walk(std::true_type{}, std::false_type{});
+        }
+        else
+        {
+            walk(std::true_type{}, std::true_type{});
         }
 
         // every load has landed and every wave has read its last stage: the ring becomes
