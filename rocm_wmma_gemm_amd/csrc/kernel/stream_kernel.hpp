@@ -478,12 +478,16 @@ struct stream_gemm
         const int tr_off_b = mn_read_offset<BN>(wave, sub, slot);
         using lds_u32x4    = __attribute__((address_space(3))) u32x4;
 
+        // (The accumulators enter and leave a copy of the walk through settle(): where the
+        // copies meet again the compiler may move them between registers, and it does not know
+        // that the multiply_adds before such a move are still on the matrix pipeline.)
         auto walk = [&](auto once_a, auto once_b) {
         auto issue = [&](int stage, int slot) { issue_as(stage, slot, once_a, once_b); };
         for(int t = 0; t < DEPTH - 1; ++t)
         {
             issue(clamped(t), t);
         }
+        settle(acc);
         int slot_index = 0; // of stage t
         for(int t = 0; t < stages; ++t)
         {
@@ -533,6 +537,7 @@ struct stream_gemm
             }
             slot_index = slot_index + 1 == DEPTH ? 0 : slot_index + 1;
         }
+        settle(acc);
         };
         const int once = __builtin_amdgcn_readfirstlane(args.stream_once);
         if(once == 0)

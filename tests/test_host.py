@@ -431,6 +431,43 @@ def test_tile_ring_of_the_direct_kernels_stays_deep_for_transposed_operands(tmp_
         assert len(waits) <= 1, func
 
 
+def test_streaming_kernel_never_moves_an_accumulator_right_behind_an_mfma(tmp_path):
+    """The streaming kernel's MFMAs are inline assembly, so the compiler knows nothing of
+    their latency: where it moves accumulators between registers on its own (the copies of
+    the stage walk meet again behind their loops) the source must have put wait states in
+    between (settle()), or the move reads a register that the matrix pipeline has not
+    written yet.  Every v_accvgpr_* the compiler emits must be at least 16 cycles of s_nop
+    away from the MFMA before it in the listing; each copy of the walk must also keep its
+    loads and MFMAs in one loop block."""
+    hipcc = "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not found")
+    asm = tmp_path / "stream_isa.s"
+    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature",
+           "-Xclang", "-packed-fp32-ops", "-I" + os.path.join(ROOT, "rocm_wmma_gemm_amd", "csrc"),
+           "-S", "--cuda-device-only", "-o", str(asm), os.path.join(ROOT, "tests", "stream_isa.hip")]
+    subprocess.run(cmd, check=True, capture_output=True, timeout=600)
+    code = [l.strip() for l in asm.read_text().split("\n")]
+    code = [l for l in code if l and not l.startswith((";", "."))]
+    nops, seen_mfma, moves, mfmas = 0, False, 0, 0
+    for n, ins in enumerate(code):
+        if ins.startswith("v_mfma"):
+            seen_mfma, nops, mfmas = True, 0, mfmas + 1
+        elif ins.startswith("s_nop"):
+            nops += int(ins.split()[1]) + 1
+        elif re.match(r"^_Z\w+:", ins):
+            seen_mfma = False  # next kernel
+        elif ins.startswith("v_accvgpr"):
+            moves += 1
+            assert not seen_mfma or nops >= 16, f"line {n}: {ins} only {nops} wait states behind an MFMA"
+    # (all twelve tiles, four copies of each walk)
+    assert mfmas == 4 * (16 + 4 + 16 + 4 + 8 + 8 + 2 + 2 + 4 + 32 + 32 + 16) and moves > 0, (mfmas, moves)
+    loops = [body for f, body in _mfma_loops(asm.read_text()) if "stream_gemm" in f]
+    assert len(loops) >= 48, len(loops)  # four copies of the walk in each of the twelve kernels
+    for body in loops:
+        assert any("buffer_load_dwordx4" in b for b in body), "a stage's loads left its loop"
+
+
 # ---------------------------------------------------------------- tuner (search space, GOMEA, run-time compile)
 def _tune_module():
     sys.path.insert(0, os.path.join(ROOT, "rocm_wmma_gemm_amd", "config"))
