@@ -256,7 +256,7 @@ def test_race_head_to_head_tie_goes_to_the_lower_median():
 
     # rounds: (1.0 vs 1.2) cfg1, (cfg2 1.3 vs cfg1 1.0) cfg1, (1.0 vs 1.4) cfg1, (cfg2 1.5, cfg1 1.0) cfg1
     assert race.head_to_head(timer, None, {"a": 1}, {"a": 2}, 4)[:3] == (1, 4, 0)
-    both = iter([1.0, 2.0, 1.0, 3.0])  # cfg1 wins round 1, cfg2 (timed first, 1.0) wins round 2
+    both = iter([1.0, 2.0, 1.0, 3.0])  # cfg1 wins the first heat, cfg2 (timed first, 1.0) the second
 
     w = race.head_to_head(lambda k, c: next(both), None, {"a": 1}, {"a": 2}, 2)
     assert w[1:3] == (1, 1) and w[0] == 2 and w[3:] == (2.0, 1.5)
