@@ -143,9 +143,10 @@ int rocm_wmma_gemm_run_variant_ex(int type_idx, int variant, int swizzle, int sp
 
 /* Adds a tile variant that was compiled outside this library (the tuner builds
  * rocm_wmma_gemm_amd/csrc/kernel_jit.hip for one tuple, type pair and pair of operand layouts
- * and passes that library's rwg_jit_kernels here: five entry points, for the three load modes,
+ * and passes that library's rwg_jit_kernels here: nine entry points, for the three load modes,
  * 16-byte unguarded, 16-byte guarded, 2-byte, then the twins of the first two that walk K in
- * runs (see rocm_wmma_gemm_select_ex); null where the pipeline or tile has none).  The
+ * runs (see rocm_wmma_gemm_select_ex), then those twins with non-temporal loads of B and of A;
+ * null where the pipeline or tile has none).  The
  * variant gets the next index after the compiled ones and runs through
  * rocm_wmma_gemm_run_variant like any other; registering the same tuple again for another
  * type pair or layout pair adds those kernels to the same index.  operand *_kmajor: 1 if K is

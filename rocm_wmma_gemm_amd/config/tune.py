@@ -529,7 +529,7 @@ class JitBuilder:
             idx = None
             if path is not None:
                 h = ctypes.CDLL(path, mode=os.RTLD_NOW | os.RTLD_LOCAL)
-                kernels = (ctypes.c_void_p * 3).in_dll(h, "rwg_jit_kernels")
+                kernels = (ctypes.c_void_p * 9).in_dll(h, "rwg_jit_kernels")  # (host::num_modes)
                 rc = self._lib.rocm_wmma_gemm_register_variant(
                     t.block_m, t.block_n, t.block_k, t.warps_m, t.warps_n, t.pipeline, type_idx,
                     int(ak), int(bk), ctypes.cast(kernels, ctypes.c_void_p))

@@ -495,8 +495,10 @@ bool streaming_ok(const kernel_problem& p, const variant_desc& v)
 }
 
 // from this size on the streaming kernel reads an operand with the non-temporal hint (the
-// memory-side cache holds 256 MB)
-constexpr size_t stream_once_bytes = size_t{256} << 20;
+// memory-side cache holds 256 MB), and the persistent kernel one that a single row (column) of
+// its tiles reads
+constexpr size_t stream_once_bytes   = size_t{256} << 20;
+constexpr size_t read_once_tile_rows = 1;
 
 template<class OutT>
 int launch_streaming(int type_idx, const launch_plan& plan, const kernel_problem& p, hipStream_t stream,
@@ -903,13 +905,28 @@ int launch(int type_idx, const launch_plan& plan_in, const kernel_problem& p, hi
         // reference kernel_launcher.hpp:119-125 throws the same way
         throw std::runtime_error("No kernel available for the requested configuration and layout");
     }
-    // a plan that walks K in runs takes the kernel's twin built for that, where there is one
+    // a plan that walks K in runs takes the kernel's twin built for that, where there is one;
+    // so does a problem with an operand of 256 MB and more that one row (column) of tiles
+    // reads: the twin with non-temporal loads of that operand (solo_gemm says why)
     int k_run = v.pipeline == 5 ? plan_k_run(plan.touch) : 0;
     int k_group = v.pipeline == 5 ? plan_k_group(plan.touch) : 0;
-    if(k_run > 0 || k_group > 0)
+    const size_t per_launch = std::min(batches_per_launch, p.batch);
+    const int    once       = v.pipeline != 5 ? 0
+                              : grid_m <= read_once_tile_rows && p.N * p.K * in_bytes * per_launch >= stream_once_bytes ? 1
+                              : grid_n <= read_once_tile_rows && p.M * p.K * in_bytes * per_launch >= stream_once_bytes ? 2
+                                                                                                                      : 0;
+    if(k_run > 0 || k_group > 0 || once != 0)
     {
-        kernel_fn twin = mode < k_runs_twin - 1 ? lookup_kernel(type_idx, p.a_kmajor, p.b_kmajor, plan.variant, mode + k_runs_twin)
-                                                : nullptr;
+        auto twin_of = [&](int which) {
+            return mode < k_runs_twin - 1 ? lookup_kernel(type_idx, p.a_kmajor, p.b_kmajor, plan.variant,
+                                                          mode + k_runs_twin + once_stride * which)
+                                          : nullptr;
+        };
+        kernel_fn twin = twin_of(once);
+        if(twin == nullptr && once != 0 && (k_run > 0 || k_group > 0))
+        {
+            twin = twin_of(0); // (a registered variant may hold the first twins only)
+        }
         if(twin != nullptr)
         {
             fn = twin;

@@ -82,6 +82,17 @@ __device__ __forceinline__ void mfma_16x16x32_pinned(f32x4& acc, const u32x4& fa
     }
 }
 
+// K_RUNS: the twin that walks an item's K tiles in runs and groups (run(), below).
+// ONCE (twin only): bit 0, the K-loop loads of B carry the non-temporal hint, bit 1, those of
+// A.  For an operand of 256 MB and more that a single row (column) of tiles reads, so that
+// every line of it is wanted exactly once: it cannot stay in the memory-side cache for
+// anybody, and without the hint its lines push out the small operand's and the partial sums'.
+// bf16, 256 rows against 28672 x 8192 weights through the tuned plans: 820 -> 908 TFLOP/s
+// with B column-major, 836 -> 860 row-major, fp32 out 802 -> 908 with everything
+// column-major.  With two to four rows of tiles the hint is worth +6..15 % on the plain walk
+// but loses 2..14 % with the K order, whose point is that the second sharer finds the line
+// in L2 (hinted lines are the first to go), and with 32 rows of tiles, where the panels are
+// shared between XCDs through the memory-side cache, it costs 15 %: the host sets it by shape.
 template<in_kind IN,
          class OutT,
          bool A_KMAJOR,
@@ -93,7 +104,8 @@ template<in_kind IN,
          int  WAVES_N,
          int  STAGES,
          bool GUARD_C = false,
-         bool K_RUNS  = false>
+         bool K_RUNS  = false,
+         int  ONCE    = 0>
 struct solo_gemm
 {
     using InT = typename std::conditional<IN == in_kind::f16, _Float16, __bf16>::type;
@@ -250,7 +262,8 @@ struct solo_gemm
     // destination) is written before the MFMA, which fills the wait state M0 needs
     // before the load may use it.  lds_block = LDS byte address of this wave's block 0
     // of the operand's stage; LDS_IMM = i * WAVES * 1024.
-    template<int LDS_IMM>
+    // NT: the load carries the non-temporal hint (ONCE, below).
+    template<int LDS_IMM, bool NT = false>
     __device__ __forceinline__ static void mfma_and_load(f32x4&       acc,
                                                          const u32x4& fa,
                                                          const u32x4& fb,
@@ -259,25 +272,51 @@ struct solo_gemm
                                                          const u32x4& rsrc,
                                                          unsigned int soff)
     {
-        if constexpr(IN == in_kind::f16)
+        if constexpr(NT)
         {
-            asm volatile("s_add_u32 m0, %[ldsb], %[imm]\n\t"
-                         "v_mfma_f32_16x16x32_f16 %[acc], %[b], %[a], %[acc]\n\t"
-                         "buffer_load_dwordx4 %[voff], %[rsrc], %[soff] offen lds"
-                         : [acc] "+a"(acc)
-                         : [b] "v"(fb), [a] "v"(fa), [ldsb] "s"(lds_block), [imm] "n"(LDS_IMM),
-                           [voff] "v"(voff), [rsrc] "s"(rsrc), [soff] "s"(soff)
-                         : "memory", "scc");
+            if constexpr(IN == in_kind::f16)
+            {
+                asm volatile("s_add_u32 m0, %[ldsb], %[imm]\n\t"
+                             "v_mfma_f32_16x16x32_f16 %[acc], %[b], %[a], %[acc]\n\t"
+                             "buffer_load_dwordx4 %[voff], %[rsrc], %[soff] offen nt lds"
+                             : [acc] "+a"(acc)
+                             : [b] "v"(fb), [a] "v"(fa), [ldsb] "s"(lds_block), [imm] "n"(LDS_IMM),
+                               [voff] "v"(voff), [rsrc] "s"(rsrc), [soff] "s"(soff)
+                             : "memory", "scc");
+            }
+            else
+            {
+                asm volatile("s_add_u32 m0, %[ldsb], %[imm]\n\t"
+                             "v_mfma_f32_16x16x32_bf16 %[acc], %[b], %[a], %[acc]\n\t"
+                             "buffer_load_dwordx4 %[voff], %[rsrc], %[soff] offen nt lds"
+                             : [acc] "+a"(acc)
+                             : [b] "v"(fb), [a] "v"(fa), [ldsb] "s"(lds_block), [imm] "n"(LDS_IMM),
+                               [voff] "v"(voff), [rsrc] "s"(rsrc), [soff] "s"(soff)
+                             : "memory", "scc");
+            }
         }
         else
         {
-            asm volatile("s_add_u32 m0, %[ldsb], %[imm]\n\t"
-                         "v_mfma_f32_16x16x32_bf16 %[acc], %[b], %[a], %[acc]\n\t"
-                         "buffer_load_dwordx4 %[voff], %[rsrc], %[soff] offen lds"
-                         : [acc] "+a"(acc)
-                         : [b] "v"(fb), [a] "v"(fa), [ldsb] "s"(lds_block), [imm] "n"(LDS_IMM),
-                           [voff] "v"(voff), [rsrc] "s"(rsrc), [soff] "s"(soff)
-                         : "memory", "scc");
+            if constexpr(IN == in_kind::f16)
+            {
+                asm volatile("s_add_u32 m0, %[ldsb], %[imm]\n\t"
+                             "v_mfma_f32_16x16x32_f16 %[acc], %[b], %[a], %[acc]\n\t"
+                             "buffer_load_dwordx4 %[voff], %[rsrc], %[soff] offen lds"
+                             : [acc] "+a"(acc)
+                             : [b] "v"(fb), [a] "v"(fa), [ldsb] "s"(lds_block), [imm] "n"(LDS_IMM),
+                               [voff] "v"(voff), [rsrc] "s"(rsrc), [soff] "s"(soff)
+                             : "memory", "scc");
+            }
+            else
+            {
+                asm volatile("s_add_u32 m0, %[ldsb], %[imm]\n\t"
+                             "v_mfma_f32_16x16x32_bf16 %[acc], %[b], %[a], %[acc]\n\t"
+                             "buffer_load_dwordx4 %[voff], %[rsrc], %[soff] offen lds"
+                             : [acc] "+a"(acc)
+                             : [b] "v"(fb), [a] "v"(fa), [ldsb] "s"(lds_block), [imm] "n"(LDS_IMM),
+                               [voff] "v"(voff), [rsrc] "s"(rsrc), [soff] "s"(soff)
+                             : "memory", "scc");
+            }
         }
     }
 
@@ -373,14 +412,14 @@ struct solo_gemm
             constexpr int V = PLAN::begin + (M - PLAN::first) / PLAN::gap; // load of the tile
             if constexpr(V < op_a::PER_WAVE)
             {
-                mfma_and_load<V * WAVES * 1024>(acc[M / TN][M % TN], fa[M / TN], fb[M % TN], c.fill,
+                mfma_and_load<V * WAVES * 1024, (ONCE & 2) != 0>(acc[M / TN][M % TN], fa[M / TN], fb[M % TN], c.fill,
                                                 c.la.template vector_offset<V>(), c.rsrc_a,
                                                 V * c.la.stride);
             }
             else
             {
                 constexpr int W = V - op_a::PER_WAVE;
-                mfma_and_load<A_BYTES + W * WAVES * 1024>(acc[M / TN][M % TN], fa[M / TN], fb[M % TN],
+                mfma_and_load<A_BYTES + W * WAVES * 1024, (ONCE & 1) != 0>(acc[M / TN][M % TN], fa[M / TN], fb[M % TN],
                                                           c.fill, c.lb.template vector_offset<W>(),
                                                           c.rsrc_b, W * c.lb.stride);
             }

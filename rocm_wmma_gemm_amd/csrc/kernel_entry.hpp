@@ -23,18 +23,19 @@ constexpr device::in_kind kIn = (RWG_TYPE < 2) ? device::in_kind::f16 : device::
 using out_t = std::conditional<RWG_TYPE == 0, _Float16,
                                std::conditional<RWG_TYPE == 2, __bf16, float>::type>::type;
 
-template<int BM, int BN, int BK, int WM, int WN, int PIPE, device::load_mode MODE, bool K_RUNS = false>
+template<int BM, int BN, int BK, int WM, int WN, int PIPE, device::load_mode MODE, bool K_RUNS = false, int ONCE = 0>
 constexpr kernel_fn entry()
 {
     static_assert(PIPE >= 0 && PIPE <= 7, "unknown pipeline");
     if constexpr(K_RUNS)
     {
-        // the twin that walks K in runs, XCDs out of step: the large persistent tile only
+        // the twin that walks K in runs and groups (ONCE: with non-temporal loads of B, 1, or
+        // A, 2): the large persistent tile only
         if constexpr(MODE != device::load_mode::scalar && PIPE == 5 && BM == 256 && BN == 256 && BK == 64)
         {
             return &device::gemm_entry<
                 device::solo_gemm<kIn, out_t, RWG_AK != 0, RWG_BK != 0, BM, BN, BK, WM, WN, 2,
-                                  MODE == device::load_mode::vec_guarded, true>>;
+                                  MODE == device::load_mode::vec_guarded, true, ONCE>>;
         }
         else
         {

@@ -26,7 +26,8 @@ extern const void* const rwg_jit_kernels[host::num_modes];
 extern const int         rwg_jit_description[9];
 
 // kernels by load mode: 16-byte unguarded, 16-byte guarded, 2-byte, then the K-run twins of
-// the first two (null for every tuple but the persistent 256 x 256 x 64 tile)
+// the first two, and those twins with non-temporal loads of B and of A (null for every tuple
+// but the persistent 256 x 256 x 64 tile)
 const void* const rwg_jit_kernels[host::num_modes] = {
     reinterpret_cast<const void*>(host::entry<RWG_JIT_BM, RWG_JIT_BN, RWG_JIT_BK, RWG_JIT_WM, RWG_JIT_WN,
                                               RWG_JIT_PIPE, device::load_mode::vec_unguarded>()),
@@ -38,6 +39,14 @@ const void* const rwg_jit_kernels[host::num_modes] = {
                                               RWG_JIT_PIPE, device::load_mode::vec_unguarded, true>()),
     reinterpret_cast<const void*>(host::entry<RWG_JIT_BM, RWG_JIT_BN, RWG_JIT_BK, RWG_JIT_WM, RWG_JIT_WN,
                                               RWG_JIT_PIPE, device::load_mode::vec_guarded, true>()),
+    reinterpret_cast<const void*>(host::entry<RWG_JIT_BM, RWG_JIT_BN, RWG_JIT_BK, RWG_JIT_WM, RWG_JIT_WN,
+                                              RWG_JIT_PIPE, device::load_mode::vec_unguarded, true, 1>()),
+    reinterpret_cast<const void*>(host::entry<RWG_JIT_BM, RWG_JIT_BN, RWG_JIT_BK, RWG_JIT_WM, RWG_JIT_WN,
+                                              RWG_JIT_PIPE, device::load_mode::vec_guarded, true, 1>()),
+    reinterpret_cast<const void*>(host::entry<RWG_JIT_BM, RWG_JIT_BN, RWG_JIT_BK, RWG_JIT_WM, RWG_JIT_WN,
+                                              RWG_JIT_PIPE, device::load_mode::vec_unguarded, true, 2>()),
+    reinterpret_cast<const void*>(host::entry<RWG_JIT_BM, RWG_JIT_BN, RWG_JIT_BK, RWG_JIT_WM, RWG_JIT_WN,
+                                              RWG_JIT_PIPE, device::load_mode::vec_guarded, true, 2>()),
 };
 
 // block_m, block_n, block_k, warps_m, warps_n, pipeline, type pair, A K-contiguous, B K-contiguous

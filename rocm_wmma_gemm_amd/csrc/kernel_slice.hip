@@ -18,7 +18,11 @@ namespace host
      entry<BM, BN, BK, WM, WN, PIPE, device::load_mode::vec_guarded>(),         \
      entry<BM, BN, BK, WM, WN, PIPE, device::load_mode::scalar>(),             \
      entry<BM, BN, BK, WM, WN, PIPE, device::load_mode::vec_unguarded, true>(), \
-     entry<BM, BN, BK, WM, WN, PIPE, device::load_mode::vec_guarded, true>()},
+     entry<BM, BN, BK, WM, WN, PIPE, device::load_mode::vec_guarded, true>(),      \
+     entry<BM, BN, BK, WM, WN, PIPE, device::load_mode::vec_unguarded, true, 1>(), \
+     entry<BM, BN, BK, WM, WN, PIPE, device::load_mode::vec_guarded, true, 1>(),   \
+     entry<BM, BN, BK, WM, WN, PIPE, device::load_mode::vec_unguarded, true, 2>(), \
+     entry<BM, BN, BK, WM, WN, PIPE, device::load_mode::vec_guarded, true, 2>()},
 
 const kernel_fn RWG_CAT(kernel_slice_, RWG_TYPE, RWG_AK, RWG_BK)[num_variants][num_modes] = {
 #include "variants.def"

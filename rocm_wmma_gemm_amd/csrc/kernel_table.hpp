@@ -36,9 +36,11 @@ constexpr int num_variants = 0
 constexpr int num_types = 4; // f16_f16, f32_f16, bf16_bf16, f32_bf16
 constexpr int num_load_modes = 3; // device::load_mode
 // kernels per variant: one per load mode, then the twins of the 16-byte unguarded and guarded
-// kernels that walk K in runs (persistent 256 x 256 x 64 kernel only; nullptr elsewhere)
-constexpr int num_modes     = 5;
+// kernels that walk K in runs and groups (persistent 256 x 256 x 64 kernel only; nullptr
+// elsewhere), then those twins with non-temporal loads of B, then of A
+constexpr int num_modes     = 9;
 constexpr int k_runs_twin   = 3; // mode m < 2 has its twin at m + k_runs_twin
+constexpr int once_stride   = 2; // and the twin that reads B (1) or A (2) once at m + k_runs_twin + once_stride * which
 
 using kernel_fn = void (*)(const device::gemm_args);
 

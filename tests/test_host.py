@@ -359,7 +359,7 @@ def test_hand_scheduled_kernel_keeps_accumulators_in_place(tmp_path):
         # loop is the shortest span that holds MFMAs
         if "solo_gemm" in f and (f not in loops or len(body) < len(loops[f])):
             loops[f] = body
-    assert len(loops) == 6, "an MFMA loop in each instantiated kernel expected"
+    assert len(loops) == 7, "an MFMA loop in each instantiated kernel expected"
     for func, body in loops.items():
         whole = text[text.index(func + ":"):]
         whole = whole[:whole.index(".Lfunc_end")]
@@ -368,6 +368,9 @@ def test_hand_scheduled_kernel_keeps_accumulators_in_place(tmp_path):
             f"{func}: MFMAs outside the main loop (peeled or duplicated code)"
         bad = [b for b in body if re.search(r"v_accvgpr_|scratch_", b)]
         assert not bad, f"{func}: accumulator traffic or spills inside the MFMA loop: {bad[:3]}"
+        # the read-once twin: the hint on B's loads in the loop (12 of a tile's 16 are B's or A's in turn)
+        hinted = sum(bool(re.search(r"buffer_load_dwordx4 .* nt lds", b)) for b in body)
+        assert hinted == (8 if func.endswith("Lb1ELi1EEEEEvNS0_9gemm_argsE") else 0), (func, hinted)
     # on every path that leaves the MFMA loop: two s_nop 15 before anything names an AGPR
     for func, body in loops.items():
         whole = text[text.index(func + ":"):]
